@@ -1,0 +1,94 @@
+/* qvb8_amd.h -- C ABI of libqvb8_amd.so: QVB8 / QVB8R dequantize-inside-the-matmul on MI355X (gfx950).
+ *
+ * Every entry point takes raw DEVICE pointers, sizes and a HIP stream (hipStream_t passed as void*; NULL =
+ * the default stream), launches asynchronously on that stream on the CURRENT device, never synchronises and
+ * never allocates device memory (scratch is a caller-supplied workspace).  Return value: 0 on success, a
+ * negative qvb8_status otherwise; qvb8_last_error() gives the message of the calling thread's last failure.
+ * Inputs are borrowed and never written.  The functions are re-entrant; the only state is read-once
+ * configuration (environment variables) and cached device properties.
+ *
+ * Each function names the interface of the reference extension it stands in for
+ * (src/qv_band/formats/qvb8/backends/cuda_qvb8/qvb8_cuda.cu, pybind table at :2673-2691).
+ *
+ * Common operands ("the pack"), as the reference's tensors (qvb8_cuda.cu:1424-1431, formats/qvb8/decode.py:30-43):
+ *   ids      u8[ids_bytes]  bit-packed row-major ids, LSB first, rows back to back, >= 8 pad bytes at the end,
+ *                           base address 4-byte aligned
+ *   min_s    f32[Q]         row origin          tau_s  f32[Q]   row step
+ *   nbits    u8[Q]          row width, 1..14    bit_off i64[Q]  absolute bit of the row's first id
+ *   esc_idx  i64[n_esc]     flat positions q*P+c, ascending     esc_vals f32[n_esc]  exact values
+ * value(q, c) = fmaf((float)id, tau_s[q], min_s[q]) in fp32, escapes overwrite.
+ */
+#ifndef QVB8_AMD_H
+#define QVB8_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum qvb8_dtype { QVB8_F32 = 0, QVB8_F16 = 1, QVB8_BF16 = 2 };
+
+enum qvb8_status {
+    QVB8_OK = 0,
+    QVB8_ERR_ARG = -1,        /* bad argument (shape, range, alignment, null pointer) */
+    QVB8_ERR_WORKSPACE = -2,  /* workspace too small */
+    QVB8_ERR_LAUNCH = -3,     /* the HIP runtime refused a launch */
+    QVB8_ERR_UNSUPPORTED = -4 /* configuration this build does not cover */
+};
+
+/* Library identification: ABI version (bumped on any signature change). */
+int qvb8_abi_version(void);
+/* Message of the calling thread's most recent failure ("" if none). Valid until that thread's next call. */
+const char* qvb8_last_error(void);
+
+/* ---- dense restore ------------------------------------------------------------------------------------- */
+
+/* Dense (Q, P) restore, each value rounded ONCE to out_dtype: out[q*P+c] = (T)fmaf(id, tau_s[q], min_s[q]).
+ * Bit-exact with the reference restore.  Escapes are NOT applied (see qvb8_scatter_escapes).
+ * Replaces: qvb8_decode_launch / qvb8_decode_all(_v3)  qvb8_cuda.cu:535-649; out_dtype QVB8_F16 = ext.decode
+ * (:651-699), QVB8_BF16 = ext.decode_bf16 (:1711-1727), QVB8_F32 = the fp32 band value of decode.py:196-209. */
+int qvb8_decode(const uint8_t* ids, int64_t ids_bytes, const float* min_s, const float* tau_s,
+                const uint8_t* nbits, const int64_t* bit_off, int64_t Q, int64_t P,
+                int out_dtype, void* out, void* stream);
+
+/* out[esc_idx[e]] = (T)esc_vals[e] for every escape: the overwrite the reference does with
+ * index_copy_(0, esc_idx, esc_vals.to(dt))  qvb8_cuda.cu:689-697, 1721-1725.  n_out = Q*P (bounds check). */
+int qvb8_scatter_escapes(void* out, int out_dtype, int64_t n_out, const int64_t* esc_idx,
+                         const float* esc_vals, int64_t n_esc, void* stream);
+
+/* Certificate re-check on the GPU: result[0] = max |restored[i] - original[i]| (as float bits),
+ * result[1] = number of elements with |restored - original| >= tau or a non-finite difference.
+ * `result` is u32[2] in device memory; the call initialises it.  Differences are taken in fp32 after exact
+ * widening.  No counterpart in the reference's extension: the reference certifies at pack time on the CPU
+ * (formats/qvb8/module.py:66-78 states the bound); this re-verifies it where the weights live. */
+int qvb8_certify(const void* restored, int restored_dtype, const void* original, int original_dtype,
+                 int64_t n, float tau, uint32_t* result, void* stream);
+
+/* ---- activations ----------------------------------------------------------------------------------------- */
+
+/* out_f16[i] = fp16(clamp(x[i], -65504, 65504)), NaN kept.  Replaces saturating_half  qvb8_cuda.cu:761-841. */
+int qvb8_sat_half(const void* x, int x_dtype, int64_t n, void* out_f16, void* stream);
+
+/* ---- fused decode + GEMV, M = 1..8 ---------------------------------------------------------------------- */
+
+/* Bytes of workspace qvb8_gemv needs for this shape (0 is possible). */
+int64_t qvb8_gemv_workspace_bytes(int64_t M, int64_t Q, int64_t P);
+
+/* Y[m, q] = sum_c sat_half(X[m, c]) * value(q, c), fp32 accumulate, Y is f32 (M, Q) row-major.
+ * X is (M, P) row-major in x_dtype, rows 16-byte aligned; 1 <= M <= 8.  The band value is the fp32 one (not
+ * narrowed); escapes are corrected after the main pass in ascending order without atomics, so results are
+ * reproducible run to run.
+ * Replaces: ext.gemv (M=1) qvb8_gemv_forward :1416-1512, ext.gemv_multi qvb8_gemv_multi_forward :1059-1166
+ * (kernels qvb8_gemv_multi_v3 :375-453, qvb8_fix_escapes :507-533, qvb8_splitk_combine :463-470). */
+int qvb8_gemv(const void* X, int x_dtype, int64_t M,
+              const uint8_t* ids, int64_t ids_bytes, const float* min_s, const float* tau_s,
+              const uint8_t* nbits, const int64_t* bit_off, int64_t Q, int64_t P,
+              const int64_t* esc_idx, const float* esc_vals, int64_t n_esc,
+              float* Y, void* workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QVB8_AMD_H */

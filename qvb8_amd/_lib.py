@@ -1,0 +1,87 @@
+"""ctypes binding of libqvb8_amd.so: one Python function per C entry point of
+include/qvb8_amd.h, taking torch tensors for device memory and the current torch
+stream.  A failed call raises RuntimeError with the library's message; a missing
+library raises NativeLibraryError.  Nothing here computes anything."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+from .common.errors import NativeLibraryError
+
+_LIB = None
+F32, F16, BF16 = 0, 1, 2
+_DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+
+# every symbol include/qvb8_amd.h declares
+SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_scatter_escapes", "qvb8_certify",
+           "qvb8_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv")
+
+
+def lib_path() -> str:
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libqvb8_amd.so")
+
+
+def load(build_if_missing: bool = True):
+    """The loaded library.  Built with hipcc on first use when it is not there."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = lib_path()
+    if not os.path.exists(path):
+        if not build_if_missing:
+            raise NativeLibraryError(f"{path} is missing: run `python -m qvb8_amd.build`")
+        from . import build as _b
+        try:
+            _b.build(verbose=False)
+        except Exception as ex:                      # noqa: BLE001
+            raise NativeLibraryError(f"cannot build {path}: {ex}") from None
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as ex:
+        raise NativeLibraryError(f"cannot load {path}: {ex}") from None
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    lib.qvb8_abi_version.restype = i32
+    lib.qvb8_last_error.restype = ctypes.c_char_p
+    lib.qvb8_decode.argtypes = [vp, i64, vp, vp, vp, vp, i64, i64, i32, vp, vp]
+    lib.qvb8_scatter_escapes.argtypes = [vp, i32, i64, vp, vp, i64, vp]
+    lib.qvb8_certify.argtypes = [vp, i32, vp, i32, i64, ctypes.c_float, vp, vp]
+    lib.qvb8_sat_half.argtypes = [vp, i32, i64, vp, vp]
+    lib.qvb8_gemv_workspace_bytes.argtypes = [i64, i64, i64]
+    lib.qvb8_gemv_workspace_bytes.restype = i64
+    lib.qvb8_gemv.argtypes = [vp, i32, i64, vp, i64, vp, vp, vp, vp, i64, i64, vp, vp, i64, vp, vp, i64, vp]
+    for name in SYMBOLS:
+        fn = getattr(lib, name)
+        if fn.restype is ctypes.c_int and name not in ("qvb8_abi_version",):
+            pass
+    _LIB = lib
+    return lib
+
+
+def _check(rc: int, lib):
+    if rc != 0:
+        msg = lib.qvb8_last_error()
+        raise RuntimeError((msg.decode() if msg else f"qvb8 native call failed ({rc})"))
+
+
+def dtype_code(dt) -> int:
+    try:
+        return _DT[dt]
+    except KeyError:
+        raise RuntimeError(f"qvb8: unsupported dtype {dt}") from None
+
+
+def ptr(t) -> int | None:
+    return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+def stream_of(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def require_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("qvb8: inputs must be GPU tensors (there is no CPU path)")

@@ -1,0 +1,165 @@
+"""The QVB8 operator functions, with the names and positional argument orders of the
+reference's `qvb8_cuda` extension module (qvb8_cuda.cu:2673-2691), implemented by
+libqvb8_amd.so.  torch is used for device memory (outputs come from torch's caching
+allocator, like the reference's torch::empty) and for the current stream only.
+
+    forward(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)   any M
+    gemv(...)            M = 1, X fp16        gemv_multi(...)   M = 1..8
+    decode(ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)       (Q, P) fp16
+    decode_bf16(...)     (Q, P) bf16
+Additions without a counterpart there: decode_f32 (the fp32 band value), certify,
+saturating_half.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def _check_pack(ids, min_s, row_nbits, row_bit_off, tau_s):
+    _lib.require_cuda(ids, min_s, row_nbits, row_bit_off, tau_s)
+    if ids.dtype != torch.uint8:
+        raise RuntimeError("ids must be uint8")
+    if min_s.dtype != torch.float32 or tau_s.dtype != torch.float32:
+        raise RuntimeError("min_s and tau_s must be fp32")
+    if row_nbits.dtype != torch.uint8:
+        raise RuntimeError("row_nbits must be uint8")
+    if row_bit_off.dtype != torch.int64:
+        raise RuntimeError("row_bit_off must be int64")
+    Q = min_s.numel()
+    if tau_s.numel() != Q or row_nbits.numel() != Q or row_bit_off.numel() != Q:
+        raise RuntimeError("per-row metadata lengths differ")
+    return Q
+
+
+def _check_escapes(esc_idx, esc_vals):
+    n = 0 if esc_idx is None else esc_idx.numel()
+    if n:
+        _lib.require_cuda(esc_idx, esc_vals)
+        if esc_idx.dtype != torch.int64 or esc_vals.dtype != torch.float32 or esc_vals.numel() != n:
+            raise RuntimeError("escapes must be int64 positions and float32 values of equal length")
+    return n
+
+
+def _decode_to(code, dtype, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
+    lib = _lib.load()
+    Q = _check_pack(ids, min_s, row_nbits, row_bit_off, tau_s)
+    n_esc = _check_escapes(esc_idx, esc_vals)
+    ids, min_s, tau_s = ids.contiguous(), min_s.contiguous(), tau_s.contiguous()
+    row_nbits, row_bit_off = row_nbits.contiguous(), row_bit_off.contiguous()
+    with torch.cuda.device(ids.device):
+        out = torch.empty((Q, int(P)), dtype=dtype, device=ids.device)
+        st = _lib.stream_of(ids)
+        _lib._check(lib.qvb8_decode(_lib.ptr(ids), ids.numel(), _lib.ptr(min_s), _lib.ptr(tau_s), _lib.ptr(row_nbits),
+                                    _lib.ptr(row_bit_off), Q, int(P), code, _lib.ptr(out), st), lib)
+        if n_esc:
+            ei, ev = esc_idx.contiguous(), esc_vals.contiguous()
+            _lib._check(lib.qvb8_scatter_escapes(_lib.ptr(out), code, out.numel(), _lib.ptr(ei), _lib.ptr(ev), n_esc, st), lib)
+    return out
+
+
+def decode(ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
+    """Dense (Q, P) fp16 weight: fp16(fma(id, tau_s, min_s)), escapes written over it."""
+    return _decode_to(_lib.F16, torch.float16, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)
+
+
+def decode_bf16(ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
+    """Dense (Q, P) bf16 weight, the band value rounded once to bf16."""
+    return _decode_to(_lib.BF16, torch.bfloat16, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)
+
+
+def decode_f32(ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
+    """Dense (Q, P) fp32 band values (what the GEMV multiplies), escapes exact."""
+    return _decode_to(_lib.F32, torch.float32, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)
+
+
+def certify(restored: torch.Tensor, original: torch.Tensor, tau: float):
+    """(max |restored - original|, number of elements not strictly under tau), computed
+    on the GPU.  One host read of 8 bytes."""
+    lib = _lib.load()
+    _lib.require_cuda(restored, original)
+    if restored.numel() != original.numel():
+        raise RuntimeError("certify: tensors differ in size")
+    a, b = restored.contiguous(), original.contiguous()
+    with torch.cuda.device(a.device):
+        res = torch.empty(2, dtype=torch.int32, device=a.device)
+        _lib._check(lib.qvb8_certify(_lib.ptr(a), _lib.dtype_code(a.dtype), _lib.ptr(b), _lib.dtype_code(b.dtype),
+                                     a.numel(), float(tau), res.data_ptr(), _lib.stream_of(a)), lib)
+    host = res.cpu()
+    return float(host[:1].view(torch.float32)[0]), int(host[1]) & 0xFFFFFFFF
+
+
+def saturating_half(X: torch.Tensor) -> torch.Tensor:
+    """Activations as fp16, clamped to +-65504 (NaN kept).  fp16 input is returned as is."""
+    if X.dtype == torch.float16:
+        return X.contiguous()
+    lib = _lib.load()
+    _lib.require_cuda(X)
+    Xc = X.contiguous()
+    if Xc.dtype not in (torch.float32, torch.bfloat16):
+        Xc = Xc.float()
+    with torch.cuda.device(Xc.device):
+        out = torch.empty(Xc.shape, dtype=torch.float16, device=Xc.device)
+        _lib._check(lib.qvb8_sat_half(_lib.ptr(Xc), _lib.dtype_code(Xc.dtype), Xc.numel(), _lib.ptr(out),
+                                      _lib.stream_of(Xc)), lib)
+    return out
+
+
+def gemv_multi(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
+    """(M, P) x packed (Q, P) -> fp32 (M, Q), 1 <= M <= 8: one pass over the packed ids."""
+    lib = _lib.load()
+    Q = _check_pack(ids, min_s, row_nbits, row_bit_off, tau_s)
+    n_esc = _check_escapes(esc_idx, esc_vals)
+    _lib.require_cuda(X)
+    if X.dim() != 2 or X.shape[1] != int(P):
+        raise RuntimeError(f"X must be (M, {int(P)})")
+    M = X.shape[0]
+    if not 1 <= M <= 8:
+        raise RuntimeError(f"qvb8 GEMV-multi: M={M} is outside the instantiated range 1..8; callers above "
+                           f"this (forward) route M>8 to the small-M GEMM")
+    Xc = X.contiguous()
+    if Xc.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        Xc = Xc.float()
+    ids, min_s, tau_s = ids.contiguous(), min_s.contiguous(), tau_s.contiguous()
+    row_nbits, row_bit_off = row_nbits.contiguous(), row_bit_off.contiguous()
+    with torch.cuda.device(Xc.device):
+        Y = torch.empty((M, Q), dtype=torch.float32, device=Xc.device)
+        ei = esc_idx.contiguous() if n_esc else None
+        ev = esc_vals.contiguous() if n_esc else None
+        _lib._check(lib.qvb8_gemv(_lib.ptr(Xc), _lib.dtype_code(Xc.dtype), M, _lib.ptr(ids), ids.numel(),
+                                  _lib.ptr(min_s), _lib.ptr(tau_s), _lib.ptr(row_nbits), _lib.ptr(row_bit_off),
+                                  Q, int(P), _lib.ptr(ei), _lib.ptr(ev), n_esc, _lib.ptr(Y), None, 0,
+                                  _lib.stream_of(Xc)), lib)
+    return Y
+
+
+def gemv(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
+    """M = 1 entry: X holds P fp16 values; returns fp32 (1, Q)."""
+    if X.dtype != torch.float16:
+        raise RuntimeError("X must be fp16")
+    if X.numel() != int(P):
+        raise RuntimeError("X length must equal P")
+    return gemv_multi(X.reshape(1, int(P)), ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)
+
+
+def _forward(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, out_half):
+    M = 1 if X.dim() == 1 else X.shape[0]
+    if M <= 8:
+        return gemv_multi(X.reshape(M, int(P)), ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)
+    # M > 8: certified fp16 weight once, then a library GEMM with fp32 accumulate
+    W = decode(ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)
+    Xh = saturating_half(X)
+    if out_half:
+        return torch.mm(Xh, W.t())
+    return torch.mm(Xh, W.t(), out_dtype=torch.float32)
+
+
+def forward(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
+    """Any M.  M <= 8: fused GEMV, fp32 (M, Q).  M > 8: fp16 restore + GEMM, fp32 result."""
+    return _forward(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, False)
+
+
+def forward_half(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
+    """As forward, but the M > 8 GEMM stores fp16."""
+    return _forward(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, True)
