@@ -88,6 +88,41 @@ int qvb8_gemv(const void* X, int x_dtype, int64_t M,
               const int64_t* esc_idx, const float* esc_vals, int64_t n_esc,
               float* Y, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- fused decode + small-M GEMM on the matrix cores, M = 1..48 ------------------------------------------- */
+
+enum qvb8_mma_flags {
+    QVB8_MMA_SATURATE_X = 1   /* bf16 X: values beyond +-65504 count as +-65504 (what the fp16 paths of the reference
+                                 multiply); without it bf16 X is used as it is (the reference's bf16 mode) */
+};
+
+/* Row records of the matrix-core path: one u64 per row, in tile order (position i describes row perm[i], or row i
+ * when perm is NULL).  Built once per weight (at load) and passed to every qvb8_mma call, so that a call never
+ * chases perm -> nbits/bit_off before it can request ids.  Counterpart of the per-weight launch metadata the
+ * reference computes once in QVBandLinearV8._mma_order  formats/qvb8/module.py:230-277 (perm, tile_nb). */
+int64_t qvb8_mma_rowinfo_bytes(int64_t Q);
+int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, const int32_t* perm, int64_t Q, int64_t P,
+                     int64_t ids_bytes, uint64_t* rowinfo, void* stream);
+
+/* Workspace qvb8_mma needs when it is called WITHOUT row records (it then builds them itself first). */
+int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
+
+/* Y[m, q] = sum_c X[m, c] * value(q, c), fp32 accumulate on v_mfma 16x16x32, Y f32 (M, Q) row-major.
+ * X is (M, P) fp16 or bf16 (x_dtype QVB8_F16 / QVB8_BF16), 16-byte aligned, P % 128 == 0, 1 <= M <= 48.
+ * The ids enter the matrix product exactly (as bias + id in X's own 16-bit format) and tau_s / min_s are applied
+ * in fp32 afterwards, so the result equals X times the UN-narrowed fp32 band value, escapes exact.
+ * `perm` (i32[Q], position -> row, or NULL): order in which rows are grouped into tiles of 16; rows sorted by
+ * width keep each tile on one decode pass (any order is correct).  `rowinfo`: from qvb8_mma_prepare for the same
+ * perm, or NULL (then `workspace` must hold qvb8_mma_workspace_bytes).  Widths 4..8 on dword-aligned rows take the
+ * fast path; other rows are read element by element.
+ * Replaces: ext.mma_multi  qvb8_mma_multi_forward qvb8_cuda.cu:2566-2671 (kernels :2321-2441, escape fix
+ * :2503-2548), and, through the Python module, the M <= 8 GEMV of :1059-1166 when P % 128 == 0. */
+int qvb8_mma(const void* X, int x_dtype, int64_t M,
+             const uint8_t* ids, int64_t ids_bytes, const float* min_s, const float* tau_s,
+             const uint8_t* nbits, const int64_t* bit_off, int64_t Q, int64_t P,
+             const int64_t* esc_idx, const float* esc_vals, int64_t n_esc,
+             const int32_t* perm, const uint64_t* rowinfo, int flags, float* Y,
+             void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -79,36 +79,63 @@ __device__ __forceinline__ uint32_t field_of(const uint32_t (&w)[kMaxFastNb]) {
     else return __builtin_amdgcn_alignbit(w[d + 1], w[d], s) & mask;
 }
 
-// The three steps of turning two adjacent ids into a biased fp16 pair are written as single instructions: left
-// to itself the compiler splits the 2*NB-bit extract into two masked halves and spends one to two more
-// operations per pair.
-template <int S, int W>
-__device__ __forceinline__ uint32_t bfe_const(uint32_t w) {
+// Ids 2*PR and 2*PR+1 of a lane's slice as an fp16 pair with each id in the low mantissa bits of `bias`:
+//   e = bits [2*PR*NB, +2*NB) of the slice          v_bfe_u32, or v_alignbit_b32 + v_and_b32 across a dword edge
+//   t = (e << (16 - NB)) | e                        v_lshl_or_b32: the second id lands on bit 16
+//   r = (t & mask) | bias                           v_bitop3_b32
+// Written as one instruction sequence: left to itself the compiler splits the 2*NB-bit extract into two masked
+// halves and spends one to two more operations per pair.
+template <int NB, int PR>
+__device__ __forceinline__ uint32_t pair_bits(const uint32_t (&w)[kMaxFastNb], uint32_t mask, uint32_t bias) {
+    constexpr int bit = PR * 2 * NB, d = bit >> 5, s = bit & 31, W = 2 * NB;
     uint32_t r;
-    asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "n"(S), "n"(W));
-    return r;
-}
-template <int SH>
-__device__ __forceinline__ uint32_t shl_or_self(uint32_t e) {      // (e << SH) | e
-    uint32_t r;
-    asm("v_lshl_or_b32 %0, %1, %2, %1" : "=v"(r) : "v"(e), "n"(SH));
-    return r;
-}
-__device__ __forceinline__ uint32_t and_or(uint32_t t, uint32_t mask, uint32_t bias) {   // (t & mask) | bias
-    uint32_t r;
-    asm("v_bitop3_b32 %0, %1, %2, %3 bitop3:0xea" : "=v"(r) : "v"(t), "v"(mask), "v"(bias));
+    if constexpr (s + W <= 32) {
+        asm("v_bfe_u32 %0, %1, %4, %5\n\t"
+            "v_lshl_or_b32 %0, %0, %6, %0\n\t"
+            "v_bitop3_b32 %0, %0, %2, %3 bitop3:0xea"
+            : "=&v"(r) : "v"(w[d]), "v"(mask), "v"(bias), "n"(s), "n"(W), "n"(16 - NB));
+    } else {
+        asm("v_alignbit_b32 %0, %2, %1, %5\n\t"
+            "v_and_b32 %0, %6, %0\n\t"
+            "v_lshl_or_b32 %0, %0, %7, %0\n\t"
+            "v_bitop3_b32 %0, %0, %3, %4 bitop3:0xea"
+            : "=&v"(r) : "v"(w[d]), "v"(w[d + 1]), "v"(mask), "v"(bias), "n"(s), "n"((1 << W) - 1), "n"(16 - NB));
+    }
     return r;
 }
 
-// Ids 2*PR and 2*PR+1 of the lane's slice as a | b << 16, plus bits the caller masks off (a << (16-NB) below
-// bit 16).
+// The same three steps as single instructions, for callers that want to interleave many pairs (stage by stage)
+// so that dependent instructions are far apart in the instruction stream.
 template <int NB, int PR>
-__device__ __forceinline__ uint32_t pair_of(const uint32_t (&w)[kMaxFastNb]) {
+__device__ __forceinline__ uint32_t pair_extract(const uint32_t (&w)[kMaxFastNb]) {      // e = 2*NB bits at pair PR
     constexpr int bit = PR * 2 * NB, d = bit >> 5, s = bit & 31, W = 2 * NB;
-    uint32_t e;
-    if constexpr (s + W <= 32) e = bfe_const<s, W>(w[d]);
-    else e = __builtin_amdgcn_alignbit(w[d + 1], w[d], s) & ((1u << W) - 1u);
-    return shl_or_self<16 - NB>(e);
+    uint32_t r;
+    if constexpr (s + W <= 32) {
+        asm("v_bfe_u32 %0, %1, %2, %3" : "=v"(r) : "v"(w[d]), "n"(s), "n"(W));
+    } else {
+        asm("v_alignbit_b32 %0, %2, %1, %3" : "=v"(r) : "v"(w[d]), "v"(w[d + 1]), "n"(s));
+    }
+    return r;
+}
+template <int NB, int PR>
+__device__ __forceinline__ uint32_t pair_spread(uint32_t e) {                          // (e << (16-NB)) | e, e cleaned first if needed
+    constexpr int bit = PR * 2 * NB, s = bit & 31, W = 2 * NB;
+    uint32_t r;
+    if constexpr (s + W <= 32) {
+        asm("v_lshl_or_b32 %0, %1, %2, %1" : "=v"(r) : "v"(e), "n"(16 - NB));
+    } else {
+        // the window came from v_alignbit_b32 and still has bits above 2*NB: shifting it left by 16-NB puts id b on
+        // bit 16 and pushes the junk above bit 16+NB, OR-ing the unshifted copy adds id a at bit 0 plus junk at
+        // bits >= NB; everything outside the two id fields is removed by the mask of the final step, except bits
+        // 16..16+NB-1 of the unshifted copy, which must be cleared here
+        asm("v_and_b32 %0, %2, %1\n\tv_lshl_or_b32 %0, %0, %3, %0" : "=&v"(r) : "v"(e), "n"((1 << W) - 1), "n"(16 - NB));
+    }
+    return r;
+}
+__device__ __forceinline__ uint32_t and_or3(uint32_t t, uint32_t mask, uint32_t bias) {   // (t & mask) | bias
+    uint32_t r;
+    asm("v_bitop3_b32 %0, %1, %2, %3 bitop3:0xea" : "=v"(r) : "v"(t), "v"(mask), "v"(bias));
+    return r;
 }
 
 // The lane's NB dwords, 4-byte aligned.
@@ -136,6 +163,24 @@ __device__ __forceinline__ float wave_sum(float v) {
     const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
     const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
     return (r0 + r1) + (r2 + r3);
+}
+
+// Sums of four values per lane over the 64 lanes at once: on return lane j (j < 4) holds the total of v[j].
+// Two select-and-exchange steps leave lane l with the quad sum of v[l & 3]; the quads of a 16-lane row are
+// combined with row rotations, the four rows with two cross-lane reads.  Fixed order: bit-reproducible.
+__device__ __forceinline__ float wave_sum4(const float (&v)[4], int lane) {
+    const bool b0 = lane & 1, b1 = lane & 2;
+    const float k01 = b0 ? v[1] : v[0], s01 = b0 ? v[0] : v[1];
+    const float k23 = b0 ? v[3] : v[2], s23 = b0 ? v[2] : v[3];
+    const float r01 = k01 + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(s01), 0xB1, 0xF, 0xF, true));
+    const float r23 = k23 + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(s23), 0xB1, 0xF, 0xF, true));
+    const float kk = b1 ? r23 : r01, ss = b1 ? r01 : r23;
+    float r = kk + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(ss), 0x4E, 0xF, 0xF, true));
+    r += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(r), 0x124, 0xF, 0xF, true));   // row_ror:4
+    r += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(r), 0x128, 0xF, 0xF, true));   // row_ror:8
+    r += __int_as_float(__builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __float_as_int(r)));
+    r += __int_as_float(__builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __float_as_int(r)));
+    return r;
 }
 
 }  // namespace qvb8

@@ -187,55 +187,57 @@ constexpr float kBias = 1024.0f;
 constexpr uint32_t kBiasBits = 0x64006400u;
 
 template <int NB, int PR, int PR_END, int MB>
-__device__ __forceinline__ void dot_pairs(const uint32_t (&w)[kMaxFastNb], const uint32_t (&xr)[MB][16], float (&acc)[MB][2]) {
+__device__ __forceinline__ void dot_pairs(const uint32_t (&w)[kMaxFastNb], const uint32_t (&xr)[MB][16], float (&acc)[MB][2],
+                                          uint32_t mask, uint32_t bias) {
     if constexpr (PR < PR_END) {
-        constexpr uint32_t mask = ((1u << NB) - 1u) * 0x00010001u;
-        const uint32_t bits = and_or(pair_of<NB, PR>(w), mask, kBiasBits);
+        const uint32_t bits = pair_bits<NB, PR>(w, mask, bias);
         const half2_t wv = __builtin_bit_cast(half2_t, bits);
 #pragma unroll
         for (int m = 0; m < MB; ++m)
             acc[m][PR & 1] = __builtin_amdgcn_fdot2(wv, __builtin_bit_cast(half2_t, xr[m][PR]), acc[m][PR & 1], false);
-        dot_pairs<NB, PR + 1, PR_END, MB>(w, xr, acc);
+        dot_pairs<NB, PR + 1, PR_END, MB>(w, xr, acc, mask, bias);
     }
 }
 
+// A lane's slice is NB dwords.  It is fetched as two 16-byte loads whatever NB is: dwords [0, 4) and the LAST
+// four dwords [NB-4, NB) (they overlap for NB < 8), so every row costs the same two in-bounds load
+// instructions and the wait counters of the prefetch pipeline stay exact.
 template <int NB, int MB>
-__device__ __forceinline__ void gemv_item_fast(const uint32_t (&w)[kMaxFastNb], const uint32_t (&xr)[MB][16],
+__device__ __forceinline__ void gemv_item_fast(const uint4& lo, const uint4& hi, const uint32_t (&xr)[MB][16],
                                                const float (&sx)[MB], float (&d)[MB]) {
+    const uint32_t l[4] = {lo.x, lo.y, lo.z, lo.w}, h[4] = {hi.x, hi.y, hi.z, hi.w};
+    uint32_t w[kMaxFastNb];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) w[k] = l[k];
+#pragma unroll
+    for (int k = 4; k < NB; ++k) w[k] = h[k - (NB - 4)];
     float acc[MB][2];
 #pragma unroll
     for (int m = 0; m < MB; ++m) acc[m][0] = acc[m][1] = 0.f;
-    dot_pairs<NB, 0, 16, MB>(w, xr, acc);
+    constexpr uint32_t mask = ((1u << NB) - 1u) * 0x00010001u;
+    dot_pairs<NB, 0, 16, MB>(w, xr, acc, mask, kBiasBits);
 #pragma unroll
     for (int m = 0; m < MB; ++m) d[m] = __builtin_fmaf(-kBias, sx[m], acc[m][0] + acc[m][1]);
 }
 
 template <int MB>
-__device__ __forceinline__ void gemv_compute_fast(int nb, const uint32_t (&w)[kMaxFastNb], const uint32_t (&xr)[MB][16],
+__device__ __forceinline__ void gemv_compute_fast(int nb, const uint4& lo, const uint4& hi, const uint32_t (&xr)[MB][16],
                                                   const float (&sx)[MB], float (&d)[MB]) {
     switch (nb) {
-        case 4: gemv_item_fast<4, MB>(w, xr, sx, d); break;
-        case 5: gemv_item_fast<5, MB>(w, xr, sx, d); break;
-        case 6: gemv_item_fast<6, MB>(w, xr, sx, d); break;
-        case 7: gemv_item_fast<7, MB>(w, xr, sx, d); break;
-        default: gemv_item_fast<8, MB>(w, xr, sx, d); break;
+        case 4: gemv_item_fast<4, MB>(lo, hi, xr, sx, d); break;
+        case 5: gemv_item_fast<5, MB>(lo, hi, xr, sx, d); break;
+        case 6: gemv_item_fast<6, MB>(lo, hi, xr, sx, d); break;
+        case 7: gemv_item_fast<7, MB>(lo, hi, xr, sx, d); break;
+        default: gemv_item_fast<8, MB>(lo, hi, xr, sx, d); break;
     }
 }
 
-__device__ __forceinline__ void gemv_issue_fast(int nb, const uint32_t* __restrict__ p, uint32_t (&w)[kMaxFastNb]) {
-    switch (nb) {
-        case 4: load_slice<4>(p, w); break;
-        case 5: load_slice<5>(p, w); break;
-        case 6: load_slice<6>(p, w); break;
-        case 7: load_slice<7>(p, w); break;
-        default: load_slice<8>(p, w); break;
-    }
-}
+// kind of a row for the GEMV: 0 = metadata points outside the buffer, 1 = dword-sliced, 2 = per element
+struct RowState { int nb; int kind; int64_t bit0; };
 
-// Row state a wave carries between issuing a row's loads and consuming them.
-struct RowState { int nb; int kind; int64_t bit0; };     // kind: 0 = out of bounds, 1 = fast, 2 = per-element
-
-template <int MB, int D>
+// FAST = false: no row can take the dword-sliced path (P % 32 != 0, or a buffer too small to prefetch from);
+// the kernel then contains no prefetch at all.
+template <int MB, int D, bool FAST>
 __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     uint16_t* xh = reinterpret_cast<uint16_t*>(smem);                                // [MB][P] sat-fp16 activations
@@ -249,49 +251,107 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
     const int row0 = blockIdx.x * a.RW;
     const int rows_here = min(a.RW, a.Q - row0);
     const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
-    const bool p32 = (a.P % kFieldsPerLane) == 0;
+    // rows of this wave's group: row0 + g + G*k, k < n_rows (<= 64)
+    const int n_rows = rows_here > g ? (rows_here - g + a.G - 1) / a.G : 0;
 
-    // ---- activations: narrow once per workgroup ----
-    {
-        const int64_t n = (int64_t)MB * a.P;
-        if ((a.P & 7) == 0) {
-            for (int64_t i = (int64_t)tid * 8; i < n; i += (int64_t)blockDim.x * 8) {
-                uint32_t o[4];
-                if (a.x_dtype == QVB8_F32) {
-                    const float4 v0 = *reinterpret_cast<const float4*>((const float*)a.X + i);
-                    const float4 v1 = *reinterpret_cast<const float4*>((const float*)a.X + i + 4);
-                    o[0] = sat_half_bits(v0.x) | (sat_half_bits(v0.y) << 16);
-                    o[1] = sat_half_bits(v0.z) | (sat_half_bits(v0.w) << 16);
-                    o[2] = sat_half_bits(v1.x) | (sat_half_bits(v1.y) << 16);
-                    o[3] = sat_half_bits(v1.z) | (sat_half_bits(v1.w) << 16);
-                } else {
-                    const uint4 v = *reinterpret_cast<const uint4*>((const uint16_t*)a.X + i);
-                    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-                    if (a.x_dtype == QVB8_F16) {
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) o[k] = u[k];      // fp16 -> sat fp16 is the identity (inf stays inf, as the reference's early return)
-                    } else {
-#pragma unroll
-                        for (int k = 0; k < 4; ++k)
-                            o[k] = sat_half_bits(__uint_as_float(u[k] << 16)) | (sat_half_bits(__uint_as_float(u[k] & 0xFFFF0000u)) << 16);
-                    }
-                }
-                *reinterpret_cast<uint4*>(xh + i) = make_uint4(o[0], o[1], o[2], o[3]);
-            }
-        } else {
-            for (int64_t i = tid; i < n; i += blockDim.x) {
-                const float v = load_as_f32(a.X, i, a.x_dtype);
-                xh[i] = a.x_dtype == QVB8_F16 ? ((const uint16_t*)a.X)[i] : (uint16_t)sat_half_bits(v);
-            }
-        }
+    // ---- row metadata of the whole group in one vector load: lane k holds row k's width, kind and bit offset.
+    // kind: 0 = metadata points outside the buffer, 1 = dword-sliced, 2 = per element, 3 = no such row
+    uint32_t my_info = 3u << 8;
+    int64_t my_bit0 = 0;
+    if (lane < n_rows) {
+        const int q = row0 + g + a.G * lane;
+        const int nb = a.nbits[q];
+        my_bit0 = a.bit_off[q];
+        const int64_t row_bits = (int64_t)nb * a.P;
+        const bool ok = nb >= 1 && nb <= 14 && my_bit0 >= 0 && ((my_bit0 + row_bits + 7) >> 3) + 8 <= a.ids_bytes;
+        const int kind = !ok ? 0 : (FAST && (my_bit0 & 31) == 0 && nb >= 4 && nb <= kMaxFastNb) ? 1 : 2;
+        my_info = (uint32_t)nb | ((uint32_t)kind << 8);
     }
-    __syncthreads();
+    uint32_t my_b_lo = (uint32_t)my_bit0, my_b_hi = (uint32_t)((uint64_t)my_bit0 >> 32);
+    // The values are copied once (the copy is where the wait for the metadata happens); reading a lane of them
+    // later never waits on the vector-memory queue again.
+    asm volatile("v_mov_b32 %0, %0\n\tv_mov_b32 %1, %1\n\tv_mov_b32 %2, %2" : "+v"(my_info), "+v"(my_b_lo), "+v"(my_b_hi));
+
+    bool active = false;      // whether this wave has a chunk in the current panel
+    auto row_state = [&](int k) {
+        RowState s;
+        const uint32_t info = (uint32_t)__builtin_amdgcn_readlane((int)my_info, k & 63);
+        const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readlane((int)my_b_lo, k & 63);
+        const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readlane((int)my_b_hi, k & 63);
+        s.nb = (int)(info & 0xFFu);
+        s.kind = (active && k < 64) ? (int)(info >> 8) : 3;
+        s.bit0 = (int64_t)(((uint64_t)b_hi << 32) | b_lo);
+        return s;
+    };
+
+    uint4 wlo[D], whi[D];
+    RowState st[D];
+    int cur_col = 0;          // this lane's first column in the current panel
+    bool cur_live = false;
+    // Requests the two 16-byte pieces of row k's slice.  ALWAYS exactly two loads, never under a branch, from
+    // addresses inside the buffer (rows or lanes that do not use them read the first 32 bytes of `ids`): the
+    // number of loads in flight behind any slot is then the same on every path, which is what lets the
+    // consumer wait for its own slot only.
+    auto issue = [&](int slot, int k) {
+        const RowState s = row_state(k);
+        st[slot] = s;
+        if constexpr (FAST) {
+            const bool row_fast = s.kind == 1;                                   // uniform
+            const unsigned char* rowp = a.ids + (row_fast ? (s.bit0 >> 3) : 0);  // uniform
+            const uint32_t tail = row_fast ? 4u * (uint32_t)(s.nb - 4) : 16u;    // uniform
+            const uint32_t off = (row_fast && cur_live) ? (uint32_t)(cur_col / kFieldsPerLane) * (4u * (uint32_t)s.nb) : 0u;
+            wlo[slot] = *reinterpret_cast<const uint4*>(rowp + (uint64_t)off);
+            whi[slot] = *reinterpret_cast<const uint4*>(rowp + tail + (uint64_t)off);
+        }
+    };
 
     for (int panel = 0; panel < a.panels; ++panel) {
         const int c = panel * a.W + wc;
-        if (c >= a.C || g >= a.G) continue;                  // wave-uniform
-        const int col = c * kChunk + lane * kFieldsPerLane;
-        const bool live = p32 && col < a.P;                   // this lane owns 32 whole ids of the chunk
+        active = c < a.C;                                    // wave-uniform
+        const int n_eff = active ? n_rows : 0;
+        cur_col = c * kChunk + lane * kFieldsPerLane;
+        cur_live = FAST && active && cur_col < a.P;
+#pragma unroll
+        for (int s = 0; s < D; ++s) issue(s, s);
+
+        if (panel == 0) {
+            // ---- activations: narrow once per workgroup (after the first ids are on their way) ----
+            const int64_t n = (int64_t)MB * a.P;
+            if ((a.P & 7) == 0) {
+                for (int64_t i = (int64_t)tid * 8; i < n; i += (int64_t)blockDim.x * 8) {
+                    uint32_t o[4];
+                    if (a.x_dtype == QVB8_F32) {
+                        const float4 v0 = *reinterpret_cast<const float4*>((const float*)a.X + i);
+                        const float4 v1 = *reinterpret_cast<const float4*>((const float*)a.X + i + 4);
+                        o[0] = sat_half_bits(v0.x) | (sat_half_bits(v0.y) << 16);
+                        o[1] = sat_half_bits(v0.z) | (sat_half_bits(v0.w) << 16);
+                        o[2] = sat_half_bits(v1.x) | (sat_half_bits(v1.y) << 16);
+                        o[3] = sat_half_bits(v1.z) | (sat_half_bits(v1.w) << 16);
+                    } else {
+                        const uint4 v = *reinterpret_cast<const uint4*>((const uint16_t*)a.X + i);
+                        const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+                        if (a.x_dtype == QVB8_F16) {
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) o[k] = u[k];      // fp16 input is used as it is (no clamp: inf stays inf)
+                        } else {
+#pragma unroll
+                            for (int k = 0; k < 4; ++k)
+                                o[k] = sat_half_bits(__uint_as_float(u[k] << 16)) | (sat_half_bits(__uint_as_float(u[k] & 0xFFFF0000u)) << 16);
+                        }
+                    }
+                    *reinterpret_cast<uint4*>(xh + i) = make_uint4(o[0], o[1], o[2], o[3]);
+                }
+            } else {
+                for (int64_t i = tid; i < n; i += blockDim.x) {
+                    const float v = load_as_f32(a.X, i, a.x_dtype);
+                    xh[i] = a.x_dtype == QVB8_F16 ? ((const uint16_t*)a.X)[i] : (uint16_t)sat_half_bits(v);
+                }
+            }
+            __syncthreads();
+        }
+
+        const int col = cur_col;
+        const bool live = cur_live;
         // the lane's activations as fp16 pairs, and their sum
         uint32_t xr[MB][16];
         float sx[MB];
@@ -312,14 +372,13 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
             }
             sx[m] = s0 + s1;
         }
-        // chunk sum of x for the epilogue; when P is not a multiple of 32 the lanes' registers are unused and the
-        // sum is taken per element below
+        // chunk sum of x for the epilogue (per element when no lane owns whole slices)
         float sxw[MB];
-        if (p32) {
+        if constexpr (FAST) {
 #pragma unroll
             for (int m = 0; m < MB; ++m) sxw[m] = wave_sum(sx[m]);
         } else {
-            const int col_end = min(a.P, (c + 1) * kChunk);
+            const int col_end = active ? min(a.P, (c + 1) * kChunk) : 0;
 #pragma unroll
             for (int m = 0; m < MB; ++m) {
                 float s = 0.f;
@@ -327,81 +386,46 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
                 sxw[m] = wave_sum(s);
             }
         }
-        if (g == 0 && lane == 0) {
+        if (active && g == 0 && lane == 0) {
 #pragma unroll
             for (int m = 0; m < MB; ++m) sxc[c * MB + m] = sxw[m];
         }
 
-        // rows of this group: row0 + g + G*k
-        const int n_rows = rows_here > g ? (rows_here - g + a.G - 1) / a.G : 0;
-        uint32_t wbuf[D][kMaxFastNb];
-        RowState st[D];
-        // Row metadata is fetched one row ahead of the row whose ids are being requested, with scalar loads, so
-        // that no wait on it ever drains the vector-memory queue that holds the prefetched ids.
-        auto load_meta = [&](int k, int& nb, int64_t& bit0) {
-            const int q = row0 + g + a.G * k;
-            const uintptr_t at = reinterpret_cast<uintptr_t>(a.nbits) + (uintptr_t)q;
-            const uint32_t word = *reinterpret_cast<const uint32_t*>(at & ~(uintptr_t)3);
-            nb = (int)((word >> (8u * (uint32_t)(at & 3u))) & 0xFFu);
-            bit0 = a.bit_off[q];
-        };
-        int nxt_nb = 0;
-        int64_t nxt_bit0 = 0;
-        if (n_rows > 0) load_meta(0, nxt_nb, nxt_bit0);
-        auto issue = [&](int slot, int k) {
-            RowState s;
-            s.nb = nxt_nb;
-            s.bit0 = nxt_bit0;
-            if (k + 1 < n_rows) load_meta(k + 1, nxt_nb, nxt_bit0);
-            const int64_t row_bits = (int64_t)s.nb * a.P;
-            const bool ok = s.nb >= 1 && s.nb <= 14 && s.bit0 >= 0 && ((s.bit0 + row_bits + 7) >> 3) + 8 <= a.ids_bytes;
-            s.kind = !ok ? 0 : (p32 && (s.bit0 & 31) == 0 && s.nb >= 4 && s.nb <= kMaxFastNb) ? 1 : 2;
-            if (s.kind == 1 && live)
-                gemv_issue_fast(s.nb, reinterpret_cast<const uint32_t*>(a.ids + (s.bit0 >> 3)) + (int64_t)(col / kFieldsPerLane) * s.nb, wbuf[slot]);
-            st[slot] = s;
-        };
-        auto consume = [&](int slot, int k) {
+        // id sums of one row for this lane (before the lanes are combined)
+        auto consume = [&](int slot, float (&d)[MB]) {
             const RowState s = st[slot];
-            float d[MB];
-            if (s.kind == 1) {
-                if (live) gemv_compute_fast<MB>(s.nb, wbuf[slot], xr, sx, d);
-                else {
 #pragma unroll
-                    for (int m = 0; m < MB; ++m) d[m] = 0.f;
-                }
+            for (int m = 0; m < MB; ++m) d[m] = 0.f;
+            if (FAST && s.kind == 1) {
+                if (live) gemv_compute_fast<MB>(s.nb, wlo[slot], whi[slot], xr, sx, d);
             } else if (s.kind == 2) {
-#pragma unroll
-                for (int m = 0; m < MB; ++m) d[m] = 0.f;
                 const int col_end = min(a.P, (c + 1) * kChunk);
                 for (int cc = c * kChunk + lane; cc < col_end; cc += kWave) {
                     const float idf = (float)load_field(a.ids, s.bit0 + (int64_t)cc * s.nb, s.nb, clamp_byte);
 #pragma unroll
                     for (int m = 0; m < MB; ++m) d[m] = __builtin_fmaf(f16_bits_to_f32(xh[(size_t)m * a.P + cc]), idf, d[m]);
                 }
-            } else {
+            } else if (s.kind == 0) {
 #pragma unroll
                 for (int m = 0; m < MB; ++m) d[m] = __builtin_nanf("");
             }
-            float tot[MB];
-#pragma unroll
-            for (int m = 0; m < MB; ++m) tot[m] = wave_sum(d[m]);
-            if (lane == 0) {
-                float* dst = part + ((size_t)(g + a.G * k) * a.C + c) * MB;
-#pragma unroll
-                for (int m = 0; m < MB; ++m) dst[m] = tot[m];
-            }
         };
-#pragma unroll
-        for (int s = 0; s < D; ++s)
-            if (s < n_rows) issue(s, s);
-        for (int k0 = 0; k0 < n_rows; k0 += D) {
+        static_assert(D == 4, "the row pipeline combines four rows at a time");
+        const int n_iter = (n_eff + D - 1) / D;
+        for (int it = 0; it < n_iter; ++it) {
+            float d[D][MB];
 #pragma unroll
             for (int s = 0; s < D; ++s) {
-                const int k = k0 + s;
-                if (k < n_rows) {
-                    consume(s, k);
-                    if (k + D < n_rows) issue(s, k + D);
-                }
+                consume(s, d[s]);
+                issue(s, it * D + s + D);
+            }
+            // lanes 0..3 end up with the totals of rows it*4 + 0..3
+            const int k = it * D + (lane & 3);
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                const float v4[4] = {d[0][m], d[1][m], d[2][m], d[3][m]};
+                const float tot = wave_sum4(v4, lane);
+                if (lane < 4 && k < n_eff) part[((size_t)(g + a.G * k) * a.C + c) * MB + m] = tot;
             }
         }
     }
@@ -411,9 +435,9 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
     for (int i = tid; i < rows_here * MB; i += blockDim.x) {
         const int rl = i / MB, m = i - rl * MB;
         double dsum = 0.0, xsum = 0.0;
-        for (int c = 0; c < a.C; ++c) {
-            dsum += (double)part[((size_t)rl * a.C + c) * MB + m];
-            xsum += (double)sxc[c * MB + m];
+        for (int cc = 0; cc < a.C; ++cc) {
+            dsum += (double)part[((size_t)rl * a.C + cc) * MB + m];
+            xsum += (double)sxc[cc * MB + m];
         }
         const int q = row0 + rl;
         a.Y[(size_t)m * a.Q + q] = (float)((double)a.tau_s[q] * dsum + (double)a.min_s[q] * xsum);
@@ -577,17 +601,22 @@ bool plan_gemv(int64_t M, int64_t Q, int64_t P, GemvPlan& pl) {
     return pl.lds <= kGemvLdsLimit;
 }
 
+template <int MB, int D, bool FAST>
+void launch_gemv_as(const GemvArgs& a, const GemvPlan& pl, hipStream_t s) {
+    static bool attr = false;
+    if (!attr) {
+        (void)hipFuncSetAttribute((const void*)gemv_kernel<MB, D, FAST>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvLdsLimit);
+        attr = true;
+    }
+    hipLaunchKernelGGL((gemv_kernel<MB, D, FAST>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s, a);
+}
+
 template <int MB>
 void launch_gemv(const GemvArgs& a, const GemvPlan& pl, hipStream_t s) {
-    if constexpr (MB <= 2) {
-        static bool attr = false;
-        if (!attr) { (void)hipFuncSetAttribute((const void*)gemv_kernel<MB, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvLdsLimit); attr = true; }
-        hipLaunchKernelGGL((gemv_kernel<MB, 2>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s, a);
-    } else {
-        static bool attr = false;
-        if (!attr) { (void)hipFuncSetAttribute((const void*)gemv_kernel<MB, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvLdsLimit); attr = true; }
-        hipLaunchKernelGGL((gemv_kernel<MB, 4>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s, a);
-    }
+    constexpr int D = 4;
+    const bool fast = (a.P % kFieldsPerLane) == 0 && a.ids_bytes >= 32;
+    if (fast) launch_gemv_as<MB, D, true>(a, pl, s);
+    else launch_gemv_as<MB, D, false>(a, pl, s);
 }
 }  // namespace
 

@@ -1,0 +1,517 @@
+// Fused QVB8 decode + small-M GEMM on the matrix cores (gfx950): M = 1..48 rows of X against the packed (Q, P) weight.
+//
+//   Y[t][q] = tau_s[q] * sum_c X[t][c] * id[q][c]  +  min_s[q] * sum_c X[t][c]
+//
+// The id sum is a matrix product with the ids as one MFMA operand.  A tile is 16 weight rows; per step a wave
+// takes 128 columns of the tile: lane l owns the 32 consecutive ids of row l % 16 at columns 32 * (l / 16), which
+// are NB dwords of that row, fetched as two 16-byte loads straight in the MFMA operand layout (16 row streams
+// per wave; measured as fast as fully contiguous loads).  Each pair of ids is turned into two 16-bit floats
+// `bias + id` (exact: 1024 + id in fp16, 128 + id in bf16) with three integer operations, four v_mfma 16x16x32
+// consume the lane's 32 ids against the activations held in registers, and the bias is removed with one more
+// MFMA per step against a matrix of ones (computed once per wave, not per tile).  Activations are used in
+// their own 16-bit format: no conversion anywhere.
+//
+// A workgroup has W waves that share a tile and own T*128 columns each (repeated over `panels` when the row is
+// longer), times G tile groups.  Per-row metadata of the workgroup's rows is staged in LDS once; partial sums
+// meet in LDS and are combined in a fixed order (bit-reproducible, no atomics).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/qvb8_amd.h"
+#include "qvb8_device.h"
+#include "qvb8_host.h"
+
+namespace qvb8 {
+
+typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
+
+constexpr int kTileRows = 16;
+constexpr int kStepCols = 128;          // columns one wave step covers (4 lane groups x 32 ids)
+
+template <bool BF> struct Fmt;
+template <> struct Fmt<false> {          // fp16: 0x6400 | id == 1024 + id for id < 1024
+    static constexpr uint32_t bias_bits = 0x64006400u, one_bits = 0x3C003C00u;
+    static constexpr float bias = 1024.0f;
+    static constexpr int max_nb = 8;
+    static __device__ __forceinline__ v4f_t mfma(const v4u_t& a, const v4u_t& b, const v4f_t& c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h_t, a), __builtin_bit_cast(v8h_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(uint32_t h) { return f16_bits_to_f32(h); }
+};
+template <> struct Fmt<true> {           // bf16: 0x4300 | id == 128 + id for id < 128
+    static constexpr uint32_t bias_bits = 0x43004300u, one_bits = 0x3F803F80u;
+    static constexpr float bias = 128.0f;
+    static constexpr int max_nb = 7;
+    static __device__ __forceinline__ v4f_t mfma(const v4u_t& a, const v4u_t& b, const v4f_t& c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, a), __builtin_bit_cast(v8bf_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(uint32_t h) { return bf16_bits_to_f32(h); }
+};
+
+// Per-row record of the tile kernel, one u64 per row in TILE ORDER (position -> row through `perm`):
+//   bits 0..47 absolute bit offset of the row's first id | bits 48..55 width | bits 56..57 kind
+//   kind 0: the metadata points outside the buffer (the row yields NaN), 1: dword-aligned row of width 4..8
+//   (sliced path), 2: anything else that is in bounds (read element by element), 3: no such row
+constexpr uint64_t kRowOffMask = (1ull << 48) - 1;
+
+struct TileArgs {
+    const uint16_t* X;            // (M, P) fp16 or bf16 bits
+    const uint8_t* ids; const float* min_s; const float* tau_s;
+    const uint64_t* rowinfo;      // [Q] row records in tile order
+    const int32_t* perm;          // position -> row, or null
+    float* Y;                     // (M, Q) fp32
+    int64_t ids_bytes;
+    int M, Q, P;
+    int n_steps;                  // P / 128
+    int W, G, panels;             // waves per tile, tile groups per workgroup, column panels
+    int TW;                       // tiles per workgroup (multiple of G)
+    unsigned long long* dbg;      // DEBUG timestamps
+};
+
+__global__ void __launch_bounds__(256) rowinfo_kernel(const uint8_t* __restrict__ nbits, const int64_t* __restrict__ bit_off,
+                                                      const int32_t* __restrict__ perm, int Q, int P, int64_t ids_bytes,
+                                                      uint64_t* __restrict__ out) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= Q) return;
+    const int q = perm ? perm[i] : i;
+    uint64_t rec = 0;
+    if (q >= 0 && q < Q) {
+        const int nb = nbits[q];
+        const int64_t bit0 = bit_off[q];
+        const int64_t row_bits = (int64_t)nb * P;
+        const bool ok = nb >= 1 && nb <= 14 && bit0 >= 0 && bit0 < (int64_t)kRowOffMask && ((bit0 + row_bits + 7) >> 3) + 8 <= ids_bytes;
+        const uint64_t kind = !ok ? 0 : ((bit0 & 31) == 0 && nb >= 4 && nb <= 8) ? 1 : 2;
+        rec = (ok ? (uint64_t)bit0 : 0) | ((uint64_t)nb << 48) | (kind << 56);
+    }
+    out[i] = rec;
+}
+
+// the 16 pairs of a lane's slice -> 4 operand registers for each of the 4 MFMA steps, stage by stage: all
+// extracts, then all spreads, then all mask-and-bias steps, so that no instruction waits for its predecessor
+template <int NB, int PR>
+__device__ __forceinline__ void stage_extract(const uint32_t (&w)[kMaxFastNb], uint32_t (&e)[16]) {
+    if constexpr (PR < 16) { e[PR] = pair_extract<NB, PR>(w); stage_extract<NB, PR + 1>(w, e); }
+}
+template <int NB, int PR>
+__device__ __forceinline__ void stage_spread(uint32_t (&e)[16]) {
+    if constexpr (PR < 16) { e[PR] = pair_spread<NB, PR>(e[PR]); stage_spread<NB, PR + 1>(e); }
+}
+
+template <int NB>
+__device__ __forceinline__ void slice_pairs(const uint4& lo, const uint4& hi, uint32_t (&e)[16]) {
+    const uint32_t l[4] = {lo.x, lo.y, lo.z, lo.w}, h[4] = {hi.x, hi.y, hi.z, hi.w};
+    uint32_t w[kMaxFastNb];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) w[k] = l[k];
+#pragma unroll
+    for (int k = 4; k < NB; ++k) w[k] = h[k - (NB - 4)];
+    stage_extract<NB, 0>(w, e);
+    stage_spread<NB, 0>(e);
+}
+
+template <int NB, bool BF>
+__device__ __forceinline__ void decode_slice(const uint4& lo, const uint4& hi, v4u_t (&b)[4]) {
+    constexpr int KEEP = (BF && NB > 7) ? 7 : NB;            // bf16 holds 7 id bits next to the bias
+    constexpr uint32_t mask = ((1u << KEEP) - 1u) * 0x00010001u;
+    uint32_t e[16];
+    slice_pairs<NB>(lo, hi, e);
+#pragma unroll
+    for (int p = 0; p < 16; ++p) b[p / 4][p % 4] = and_or3(e[p], mask, Fmt<BF>::bias_bits);
+}
+
+// bf16, width 8: the operand above carries id & 127 (plus the bias); bit 7 goes into a second operand as
+// 2^-63 per set bit (a lone exponent bit), multiplied separately and scaled back in the epilogue.
+constexpr uint32_t kTopBitBits = 0x20002000u;               // bf16 2^-63 in both halves
+constexpr float kTopBitScale = 128.0f * 9223372036854775808.0f;   // 128 * 2^63
+
+__device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& hi, v4u_t (&bt)[4]) {
+    uint32_t e[16];
+    slice_pairs<8>(lo, hi, e);
+#pragma unroll
+    for (int p = 0; p < 16; ++p) bt[p / 4][p % 4] = (e[p] << 6) & kTopBitBits;
+}
+
+// NT = token tiles of 16 (M <= 16 * NT); T = steps of 128 columns a wave owns per panel; BF = bf16 operands
+template <int NT, int T, bool BF>
+__global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
+    using F = Fmt<BF>;
+    constexpr int D = 4;                                   // steps in flight per wave
+    constexpr int TM = 16 * NT;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int rows_cap = a.TW * kTileRows;
+    const int ranges = a.W;                                             // partial-sum slots per row: one per wave of the tile, panels add up in place
+    const int wave_rows = (a.TW / a.G) * kTileRows;                     // rows a wave ever touches
+    const int n_waves = a.W * a.G;
+    // LDS: per-wave copies of the row records, epilogue metadata, column-range sums of x, partial sums
+    uint64_t* s_rec = reinterpret_cast<uint64_t*>(smem);                // [n_waves][wave_rows]
+    int32_t* s_q = reinterpret_cast<int32_t*>(s_rec + (size_t)n_waves * wave_rows);   // [rows_cap] output row or -1
+    float* s_ts = reinterpret_cast<float*>(s_q + rows_cap);
+    float* s_mn = s_ts + rows_cap;
+    float* sxs = s_mn + rows_cap;                                       // [ranges][TM]
+    float* part = sxs + (size_t)ranges * TM;                            // [rows_cap][ranges][TM]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = wave / a.W, wc = wave - g * a.W;
+    const int r = lane & 15, kg = lane >> 4;
+    const int srow0 = blockIdx.x * rows_cap;                            // first position of the workgroup
+    const int rows_here = min(rows_cap, a.Q - srow0);
+    const int tiles_here = (rows_here + kTileRows - 1) / kTileRows;
+    const int n_tiles = tiles_here > g ? (tiles_here - g + a.G - 1) / a.G : 0;    // tiles of this wave's group
+#define TS(k) do { if (a.dbg && tid == 0) a.dbg[blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
+    TS(0);
+
+    // ---- this wave's row records into its own LDS copy (no workgroup barrier: a wave's LDS accesses stay in order) ----
+    uint64_t* my_rec = s_rec + (size_t)wave * wave_rows;
+    for (int i = lane; i < n_tiles * kTileRows; i += kWave) {
+        const int tk = i >> 4, rr = i & 15;
+        const int pos = srow0 + (g + a.G * tk) * kTileRows + rr;
+        my_rec[i] = pos < a.Q ? a.rowinfo[pos] : (3ull << 56);
+    }
+    // ---- epilogue metadata, needed only after the final barrier ----
+    for (int i = tid; i < rows_cap; i += blockDim.x) {
+        int q = -1;
+        float ts = 0.f, mn = 0.f;
+        if (i < rows_here) {
+            q = a.perm ? a.perm[srow0 + i] : srow0 + i;
+            if (q >= 0 && q < a.Q) { ts = a.tau_s[q]; mn = a.min_s[q]; } else q = -1;
+        }
+        s_q[i] = q; s_ts[i] = ts; s_mn[i] = mn;
+    }
+
+    const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
+    uint4 wlo[D], whi[D];
+    uint32_t inf[D];                                     // width | kind << 8 of the lane's row, per slot
+    int step0 = 0;                                       // first global step of this wave in the current panel
+    bool active = false;
+    // Requests the lane's slice of flat step i = tile_k * T + it of the current panel.  Always exactly two
+    // loads, never under a branch, from addresses inside the buffer.
+    auto issue = [&](int slot, int i) {
+        const int tk = i / T, it = i - tk * T;
+        const bool in_range = active && tk < n_tiles && (step0 + it) < a.n_steps;
+        const uint64_t rec = in_range ? my_rec[tk * kTileRows + r] : (3ull << 56);
+        const uint32_t nb = (uint32_t)(rec >> 48) & 0xFFu, kind = (uint32_t)(rec >> 56) & 3u;
+        const bool sliced = kind == 1u && nb <= 8u && (BF || nb <= (uint32_t)F::max_nb);
+        const uint64_t off = sliced ? ((rec & kRowOffMask) >> 3) + (uint64_t)((step0 + it) * 4 + kg) * (4u * nb) : 0;
+        const uint32_t tail = sliced ? 4u * (nb - 4u) : 16u;
+        inf[slot] = nb | ((sliced ? 1u : kind == 1u ? 2u : kind) << 8);
+        wlo[slot] = *reinterpret_cast<const uint4*>(a.ids + off);
+        whi[slot] = *reinterpret_cast<const uint4*>(a.ids + off + tail);
+    };
+
+    for (int panel = 0; panel < a.panels; ++panel) {
+        step0 = (panel * a.W + wc) * T;
+        active = step0 < a.n_steps;                                   // wave-uniform
+        const int range = wc;
+        const bool first_panel = panel == 0;
+
+        // ---- activations of this wave's columns, in MFMA operand layout: lane (t = l % 16, kg) holds
+        //      X[16*nt + t][128*(step0+it) + 32*kg + 8*j + 0..7].  Requested before the ids: they are few and
+        //      everything below waits for them ----
+        v4u_t xa[NT][T][4];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int it = 0; it < T; ++it)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xa[nt][it][j] = v4u_t{0, 0, 0, 0};
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int t = nt * 16 + r;
+#pragma unroll
+            for (int it = 0; it < T; ++it) {
+                if (active && t < a.M && (step0 + it) < a.n_steps) {
+                    const uint16_t* xp = a.X + (size_t)t * a.P + (size_t)(step0 + it) * kStepCols + kg * 32;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint4 v = *reinterpret_cast<const uint4*>(xp + 8 * j);
+                        xa[nt][it][j] = v4u_t{v.x, v.y, v.z, v.w};
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < D; ++s) issue(s, s);
+
+        // sums of x over the wave's columns: the product with a matrix of ones, in the accumulator layout
+        // (lane (row r, token group kg) register e <-> token 4*kg + e; identical for every r)
+        const v4u_t ones = {F::one_bits, F::one_bits, F::one_bits, F::one_bits};
+        v4f_t sx[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            sx[nt] = v4f_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int it = 0; it < T; ++it)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) sx[nt] = F::mfma(xa[nt][it][j], ones, sx[nt]);
+        }
+        if (active && g == 0 && r == 0) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float* dst = sxs + range * TM + nt * 16 + kg * 4 + e;
+                    *dst = first_panel ? sx[nt][e] : *dst + sx[nt][e];
+                }
+        }
+        if (panel == 0) TS(2);
+
+        const int n_flat = active ? n_tiles * T : 0;
+        const int n_iter = (n_flat + D - 1) / D;
+        v4f_t acc[NT], acc_top[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) { acc[nt] = v4f_t{0.f, 0.f, 0.f, 0.f}; acc_top[nt] = v4f_t{0.f, 0.f, 0.f, 0.f}; }
+        for (int itr = 0; itr < n_iter; ++itr) {
+#pragma unroll
+            for (int s = 0; s < D; ++s) {
+                static_assert(D % T == 0, "a slot always holds the same step of a tile");
+                const int i = itr * D + s;
+                const int it = s % T;                              // compile-time after unrolling
+                const int tk = itr * (D / T) + s / T;
+                // ---- decode the slot: one pass per width present in the tile ----
+                const uint32_t info = inf[s];
+                const uint32_t nb = info & 0xFFu;
+                const bool sliced = (info >> 8) == 1u;
+                v4u_t b[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) b[j] = v4u_t{F::bias_bits, F::bias_bits, F::bias_bits, F::bias_bits};
+                const uint4 lo = wlo[s], hi = whi[s];
+                if (__builtin_amdgcn_ballot_w64(sliced && nb == 7)) { if (sliced && nb == 7) decode_slice<7, BF>(lo, hi, b); }
+                if (__builtin_amdgcn_ballot_w64(sliced && nb == 6)) { if (sliced && nb == 6) decode_slice<6, BF>(lo, hi, b); }
+                if (__builtin_amdgcn_ballot_w64(sliced && nb == 5)) { if (sliced && nb == 5) decode_slice<5, BF>(lo, hi, b); }
+                if (__builtin_amdgcn_ballot_w64(sliced && nb == 4)) { if (sliced && nb == 4) decode_slice<4, BF>(lo, hi, b); }
+                const bool any8 = __builtin_amdgcn_ballot_w64(sliced && nb == 8) != 0;
+                if (any8) {
+                    if (sliced && nb == 8) decode_slice<8, BF>(lo, hi, b);
+                    if constexpr (BF) {
+                        v4u_t bt[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) bt[j] = v4u_t{0, 0, 0, 0};
+                        if (sliced && nb == 8) decode_slice8_top(lo, hi, bt);
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) acc_top[nt] = F::mfma(xa[nt][it][j], bt[j], acc_top[nt]);
+                    }
+                }
+                issue(s, i + D);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[nt] = F::mfma(xa[nt][it][j], b[j], acc[nt]);
+                if (it == T - 1 && i < n_flat) {
+                    // ---- tile done for this wave: remove the bias, store into the wave's own LDS slots ----
+                    const int lrow = (g + a.G * tk) * kTileRows + r;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int t = nt * 16 + kg * 4 + e;
+                            float v = __builtin_fmaf(-F::bias, sx[nt][e], acc[nt][e]);
+                            if constexpr (BF) v = __builtin_fmaf(kTopBitScale, acc_top[nt][e], v);
+                            if (t < a.M) {
+                                float* dst = part + ((size_t)lrow * ranges + range) * TM + t;
+                                *dst = first_panel ? v : *dst + v;
+                            }
+                        }
+                        acc[nt] = v4f_t{0.f, 0.f, 0.f, 0.f};
+                        acc_top[nt] = v4f_t{0.f, 0.f, 0.f, 0.f};
+                    }
+                    // rows the sliced path cannot read: redo them element by element
+                    const uint32_t kind_here = (uint32_t)(my_rec[tk * kTileRows + r] >> 56) & 3u;   // of row r of this tile
+                    const uint32_t nb_here = (uint32_t)(my_rec[tk * kTileRows + r] >> 48) & 0xFFu;
+                    uint64_t odd = __builtin_amdgcn_ballot_w64(kg == 0 && (kind_here == 0u || kind_here == 2u || (kind_here == 1u && nb_here > 8u)));
+                    while (odd) {
+                        const int rr = __builtin_ctzll(odd);
+                        odd &= odd - 1;
+                        const int lr2 = (g + a.G * tk) * kTileRows + rr;
+                        const uint64_t rec = my_rec[tk * kTileRows + rr];
+                        const int nb2 = (int)((rec >> 48) & 0xFFu);
+                        const bool readable = ((rec >> 56) & 3u) != 0u;
+                        const int64_t bit0 = (int64_t)(rec & kRowOffMask);
+                        const int c_lo = step0 * kStepCols, c_hi = min(a.P, (step0 + T) * kStepCols);
+                        for (int t = 0; t < a.M; ++t) {
+                            float sacc = 0.f;
+                            if (readable) {
+                                for (int c = c_lo + lane; c < c_hi; c += kWave) {
+                                    const float idf = (float)load_field(a.ids, bit0 + (int64_t)c * nb2, nb2, clamp_byte);
+                                    sacc = __builtin_fmaf(F::to_f32(a.X[(size_t)t * a.P + c]), idf, sacc);
+                                }
+                            } else {
+                                sacc = __builtin_nanf("");
+                            }
+                            const float tot = wave_sum(sacc);
+                            if (lane == 0) {
+                                // the sliced pass stored this wave's value for the row already (zero contribution plus earlier panels): add to it
+                                part[((size_t)lr2 * ranges + range) * TM + t] += tot;
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+    TS(3);
+    __syncthreads();
+    TS(4);
+
+    // ---- epilogue: combine the column ranges of each row in ascending order ----
+    for (int i = tid; i < rows_here * a.M; i += blockDim.x) {
+        const int rl = i / a.M, t = i - rl * a.M;
+        const int q = s_q[rl];
+        if (q < 0) continue;
+        double dsum = 0.0, xsum = 0.0;
+        const int all_ranges = (a.n_steps + T - 1) / T;
+        const int valid_ranges = all_ranges < ranges ? all_ranges : ranges;      // waves without any column never stored
+        for (int w = 0; w < valid_ranges; ++w) {
+            dsum += (double)part[((size_t)rl * ranges + w) * TM + t];
+            xsum += (double)sxs[w * TM + t];
+        }
+        a.Y[(size_t)t * a.Q + q] = (float)((double)s_ts[rl] * dsum + (double)s_mn[rl] * xsum);
+    }
+    TS(5);
+}
+
+// Escape correction for any M: one thread per (output row with escapes, token), ascending order, no atomics.
+template <bool BF>
+__global__ void __launch_bounds__(256) tile_fix_escapes_kernel(const uint16_t* __restrict__ X, int M,
+        const uint8_t* __restrict__ ids, int64_t ids_bytes, const float* __restrict__ min_s, const float* __restrict__ tau_s,
+        const uint8_t* __restrict__ nbits, const int64_t* __restrict__ bit_off, const int64_t* __restrict__ esc_idx,
+        const float* __restrict__ esc_vals, int64_t n_esc, float* __restrict__ Y, int Q, int P) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int t = blockIdx.y;
+    if (i >= n_esc || t >= M) return;
+    const int64_t q = esc_idx[i] / P;
+    if (q < 0 || q >= Q) return;
+    if (i > 0 && esc_idx[i - 1] / P == q) return;
+    const int nb = nbits[q];
+    const int64_t bit0 = bit_off[q];
+    const float ts = tau_s[q], mn = min_s[q];
+    const int64_t clamp_byte = (ids_bytes - 8) & ~(int64_t)3;
+    float acc = 0.f;
+    for (int64_t e = i; e < n_esc && esc_idx[e] / P == q; ++e) {
+        const int c = (int)(esc_idx[e] - q * P);
+        const float banded = __builtin_fmaf((float)load_field(ids, bit0 + (int64_t)c * nb, nb, clamp_byte), ts, mn);
+        acc = __builtin_fmaf(Fmt<BF>::to_f32(X[(size_t)t * P + c]), esc_vals[e] - banded, acc);
+    }
+    Y[(size_t)t * Q + q] += acc;
+}
+
+}  // namespace qvb8
+
+using namespace qvb8;
+
+namespace {
+struct TilePlan { int W, G, panels, TW, threads; size_t lds; unsigned blocks; };
+
+constexpr size_t kTileLdsLimit = 128 * 1024;
+
+bool plan_tile(int NT, int T, int64_t Q, int64_t P, TilePlan& pl) {
+    const int n_steps = (int)(P / kStepCols);
+    const int ranges = (n_steps + T - 1) / T;                 // column ranges of T steps
+    const int max_waves = 8;
+    pl.panels = (ranges + max_waves - 1) / max_waves;
+    pl.W = (ranges + pl.panels - 1) / pl.panels;
+    pl.G = pl.panels == 1 ? max_waves / pl.W : 1;
+    if (pl.G < 1) pl.G = 1;
+    pl.threads = 64 * pl.W * pl.G;
+    const int64_t tiles = (Q + kTileRows - 1) / kTileRows;
+    const int cus = host::device_cus();
+    const int per_cu = host::env_int("QVB8_TILE_WGS_PER_CU", 1);
+    int64_t target = (int64_t)cus * (per_cu > 0 ? per_cu : 1);
+    int64_t tw = (tiles + target - 1) / target;
+    tw = (tw + pl.G - 1) / pl.G * pl.G;
+    if (tw < pl.G) tw = pl.G;
+    const size_t TM = 16 * (size_t)NT, rg = (size_t)pl.W;
+    for (;;) {
+        const size_t rows = (size_t)tw * kTileRows;
+        pl.lds = (size_t)pl.W * pl.G * (tw / pl.G) * kTileRows * 8 + rows * 3 * 4 + rg * TM * 4 + rows * rg * TM * 4;
+        if (pl.lds <= kTileLdsLimit || tw <= pl.G) break;
+        tw -= pl.G;
+    }
+    if (pl.lds > kTileLdsLimit) return false;
+    pl.TW = (int)tw;
+    pl.blocks = (unsigned)((tiles + tw - 1) / tw);
+    return true;
+}
+
+template <int NT, int T, bool BF>
+int launch_tile(TileArgs& a, hipStream_t s) {
+    TilePlan pl;
+    if (!plan_tile(NT, T, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
+    a.W = pl.W; a.G = pl.G; a.panels = pl.panels; a.TW = pl.TW;
+    static bool attr = false;
+    if (!attr) {
+        (void)hipFuncSetAttribute((const void*)tile_kernel<NT, T, BF>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTileLdsLimit);
+        attr = true;
+    }
+    hipLaunchKernelGGL((tile_kernel<NT, T, BF>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s, a);
+    return host::check_launch("qvb8_mma");
+}
+}  // namespace
+
+extern "C" int64_t qvb8_mma_rowinfo_bytes(int64_t Q) { return Q > 0 ? 8 * Q : 0; }
+
+extern "C" int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, const int32_t* perm, int64_t Q, int64_t P,
+                                int64_t ids_bytes, uint64_t* rowinfo, void* stream) {
+    if (Q < 0 || P < 0 || Q > 0x7fffffff || P > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8_mma_prepare: Q or P out of range");
+    if (Q == 0) return QVB8_OK;
+    if (!nbits || !bit_off || !rowinfo) return host::fail(QVB8_ERR_ARG, "qvb8_mma_prepare: null pointer");
+    hipLaunchKernelGGL(rowinfo_kernel, dim3((unsigned)((Q + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       nbits, bit_off, perm, (int)Q, (int)P, ids_bytes, rowinfo);
+    return host::check_launch("qvb8_mma_prepare");
+}
+
+extern "C" int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P) {
+    (void)M; (void)P;
+    return qvb8_mma_rowinfo_bytes(Q);
+}
+
+extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
+                        const uint8_t* ids, int64_t ids_bytes, const float* min_s, const float* tau_s,
+                        const uint8_t* nbits, const int64_t* bit_off, int64_t Q, int64_t P,
+                        const int64_t* esc_idx, const float* esc_vals, int64_t n_esc,
+                        const int32_t* perm, const uint64_t* rowinfo, int flags, float* Y,
+                        void* workspace, int64_t workspace_bytes, void* stream) {
+    (void)flags;
+    if (Q < 0 || P < 0 || Q > 0x7fffffff || P > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8_mma: Q or P out of range");
+    if (M < 1 || M > 48) return host::fail(QVB8_ERR_ARG, "qvb8 mma-multi: M=%lld outside 1..48", (long long)M);
+    if (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16) return host::fail(QVB8_ERR_ARG, "qvb8_mma: X must be fp16 or bf16 (narrow fp32 activations with qvb8_sat_half first)");
+    if ((P % kStepCols) != 0 || (reinterpret_cast<uintptr_t>(ids) & 3u) != 0)
+        return host::fail(QVB8_ERR_ARG, "qvb8 mma-multi: needs P%%128==0 and 4-byte-aligned ids");
+    if (ids_bytes < 32) return host::fail(QVB8_ERR_ARG, "qvb8_mma: ids buffer shorter than 32 bytes");
+    if (n_esc < 0 || (n_esc > 0 && (!esc_idx || !esc_vals))) return host::fail(QVB8_ERR_ARG, "qvb8_mma: bad escape list");
+    if (Q == 0) return QVB8_OK;
+    if (!X || !Y || !ids || !min_s || !tau_s || !nbits || !bit_off) return host::fail(QVB8_ERR_ARG, "qvb8_mma: null pointer");
+    if (reinterpret_cast<uintptr_t>(X) & 15u) return host::fail(QVB8_ERR_ARG, "qvb8_mma: X must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    unsigned long long* dbg = nullptr;
+    if (!rowinfo) {
+        if (!workspace || workspace_bytes < qvb8_mma_rowinfo_bytes(Q))
+            return host::fail(QVB8_ERR_WORKSPACE, "qvb8_mma: without row records the call needs %lld bytes of workspace", (long long)qvb8_mma_rowinfo_bytes(Q));
+        if (int rc = qvb8_mma_prepare(nbits, bit_off, perm, Q, P, ids_bytes, (uint64_t*)workspace, stream)) return rc;
+        rowinfo = (const uint64_t*)workspace;
+    } else if (workspace && workspace_bytes == -1) {
+        dbg = (unsigned long long*)workspace;       // DEBUG
+    }
+    TileArgs a;
+    a.X = (const uint16_t*)X; a.ids = ids; a.min_s = min_s; a.tau_s = tau_s; a.rowinfo = rowinfo;
+    a.perm = perm; a.Y = Y; a.ids_bytes = ids_bytes; a.M = (int)M; a.Q = (int)Q; a.P = (int)P; a.n_steps = (int)(P / kStepCols);
+    a.dbg = dbg;
+    const bool bf = x_dtype == QVB8_BF16;
+    int rc;
+    if (M <= 16) rc = bf ? launch_tile<1, 4, true>(a, s) : launch_tile<1, 4, false>(a, s);
+    else if (M <= 32) rc = bf ? launch_tile<2, 2, true>(a, s) : launch_tile<2, 2, false>(a, s);
+    else rc = bf ? launch_tile<3, 2, true>(a, s) : launch_tile<3, 2, false>(a, s);
+    if (rc) return rc;
+    if (n_esc > 0) {
+        dim3 grid((unsigned)((n_esc + 255) / 256), (unsigned)M);
+        if (bf) hipLaunchKernelGGL(tile_fix_escapes_kernel<true>, grid, dim3(256), 0, s, (const uint16_t*)X, (int)M, ids, ids_bytes, min_s, tau_s, nbits, bit_off, esc_idx, esc_vals, n_esc, Y, (int)Q, (int)P);
+        else hipLaunchKernelGGL(tile_fix_escapes_kernel<false>, grid, dim3(256), 0, s, (const uint16_t*)X, (int)M, ids, ids_bytes, min_s, tau_s, nbits, bit_off, esc_idx, esc_vals, n_esc, Y, (int)Q, (int)P);
+        return host::check_launch("qvb8_mma escapes");
+    }
+    return QVB8_OK;
+}

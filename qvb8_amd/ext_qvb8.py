@@ -143,6 +143,86 @@ def gemv(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
     return gemv_multi(X.reshape(1, int(P)), ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)
 
 
+MMA_MAX_M = 48
+MMA_SATURATE_X = 1
+
+
+def mma_prepare(row_nbits, row_bit_off, P, ids_bytes, perm=None):
+    """Row records (int64 tensor of Q words) for mma_tiles: built once per weight."""
+    lib = _lib.load()
+    _lib.require_cuda(row_nbits, row_bit_off)
+    Q = row_nbits.numel()
+    row_nbits, row_bit_off = row_nbits.contiguous(), row_bit_off.contiguous()
+    if perm is not None and perm.numel():
+        if perm.dtype != torch.int32 or perm.numel() != Q or not perm.is_cuda:
+            raise RuntimeError("qvb8 mma-multi: perm must be an int32 GPU tensor of length Q (or empty)")
+        perm = perm.contiguous()
+    else:
+        perm = None
+    with torch.cuda.device(row_nbits.device):
+        out = torch.empty(Q, dtype=torch.int64, device=row_nbits.device)
+        _lib._check(lib.qvb8_mma_prepare(_lib.ptr(row_nbits), _lib.ptr(row_bit_off), _lib.ptr(perm), Q, int(P),
+                                         int(ids_bytes), _lib.ptr(out), _lib.stream_of(row_nbits)), lib)
+    return out
+
+
+def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm=None, saturate=True,
+              rowinfo=None):
+    """Matrix-core path for 1 <= M <= 48 and P % 128 == 0: X (fp16 or bf16) times the fp32 band value, fp32 (M, Q).
+    `perm` (int32, position -> row) groups rows of equal width into tiles; `rowinfo` = mma_prepare(...) for the
+    same perm (built on the fly when absent); `saturate` makes bf16 activations beyond +-65504 count as
+    +-65504, as every fp16 path of the reference does."""
+    lib = _lib.load()
+    Q = _check_pack(ids, min_s, row_nbits, row_bit_off, tau_s)
+    n_esc = _check_escapes(esc_idx, esc_vals)
+    _lib.require_cuda(X)
+    if X.dim() != 2 or X.shape[1] != int(P):
+        raise RuntimeError(f"X must be (M, {int(P)})")
+    M = X.shape[0]
+    if not 1 <= M <= MMA_MAX_M:
+        raise RuntimeError(f"qvb8 mma-multi: M={M} outside 1..{MMA_MAX_M}")
+    if int(P) % 128 != 0 or ids.data_ptr() % 4 != 0:
+        raise RuntimeError("qvb8 mma-multi: needs P%128==0 and 4-byte-aligned ids")
+    if X.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("qvb8 mma-multi: X must be fp16 or bf16")
+    if perm is not None and perm.numel():
+        if perm.dtype != torch.int32 or perm.numel() != Q or not perm.is_cuda:
+            raise RuntimeError("qvb8 mma-multi: perm must be an int32 GPU tensor of length Q (or empty)")
+        perm = perm.contiguous()
+    else:
+        perm = None
+    if rowinfo is not None and (rowinfo.dtype != torch.int64 or rowinfo.numel() != Q or not rowinfo.is_cuda):
+        raise RuntimeError("qvb8 mma-multi: rowinfo must be the int64 GPU tensor mma_prepare returned")
+    Xc = X.contiguous()
+    ids, min_s, tau_s = ids.contiguous(), min_s.contiguous(), tau_s.contiguous()
+    row_nbits, row_bit_off = row_nbits.contiguous(), row_bit_off.contiguous()
+    with torch.cuda.device(Xc.device):
+        Y = torch.empty((M, Q), dtype=torch.float32, device=Xc.device)
+        ei = esc_idx.contiguous() if n_esc else None
+        ev = esc_vals.contiguous() if n_esc else None
+        ws = None if rowinfo is not None else torch.empty(Q, dtype=torch.int64, device=Xc.device)
+        _lib._check(lib.qvb8_mma(_lib.ptr(Xc), _lib.dtype_code(Xc.dtype), M, _lib.ptr(ids), ids.numel(),
+                                 _lib.ptr(min_s), _lib.ptr(tau_s), _lib.ptr(row_nbits), _lib.ptr(row_bit_off),
+                                 Q, int(P), _lib.ptr(ei), _lib.ptr(ev), n_esc, _lib.ptr(perm),
+                                 None if rowinfo is None else rowinfo.contiguous().data_ptr(),
+                                 MMA_SATURATE_X if saturate else 0, _lib.ptr(Y),
+                                 None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel() * 8,
+                                 _lib.stream_of(Xc)), lib)
+    return Y
+
+
+def mma_multi(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm, tile_nb,
+              bf16=False, esc_starts=None, general=-1):
+    """QVB8 tensor-core multi-row product (M <= 48), bf16.  fp16 mode (bf16=False): X saturated to fp16;
+    bf16 mode: X as bf16, not saturated.  `tile_nb`, `esc_starts` and `general` are launch hints of the
+    reference's kernels and are not needed here."""
+    del tile_nb, esc_starts, general
+    if bf16:
+        Xk = X if X.dtype == torch.bfloat16 else X.to(torch.bfloat16)
+        return mma_tiles(Xk, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm, saturate=False)
+    return mma_tiles(saturating_half(X), ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm)
+
+
 def _forward(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, out_half):
     M = 1 if X.dim() == 1 else X.shape[0]
     if M <= 8:

@@ -1,0 +1,107 @@
+"""GPU parity of the matrix-core path (qvb8_mma through ext.mma_tiles / ext.mma_multi) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qvb8_oracle as O
+from qvb8_amd import ext_qvb8 as ext
+from qvb8_amd.formats.qvb8 import pack as PK
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _x(M, P, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(M, P, generator=g).to(dtype).to(DEV)
+
+
+def _perm_by_width(nbits: torch.Tensor):
+    return torch.argsort(nbits.to(torch.int16), stable=True).to(torch.int32)
+
+
+def _check(d, args, x, y, saturate_ref):
+    ids = H.oracle_ids(d) if "ids_dense" not in d else d["ids_dense"]
+    Wr = O.reconstruct(d["min_s"], d["tau_s"], ids, d["esc_idx"], d["esc_vals"])
+    xs = x.float().cpu().numpy()
+    if saturate_ref:
+        xs = O.sat_half(xs)
+    ref = O.linear_f64(xs, Wr)
+    tol = H.gemv_tolerance(ref, Wr, xs)
+    diff = np.abs(y.cpu().numpy().astype(np.float64) - ref)
+    assert y.dtype == torch.float32 and tuple(y.shape) == ref.shape
+    assert np.all(diff <= tol), (float(diff.max()), float((diff / tol).max()), np.argwhere(diff > tol)[:5])
+    return float((diff / tol).max())
+
+
+@pytest.mark.parametrize("M", [1, 2, 5, 8, 15, 16, 17, 31, 32, 33, 48])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mma_all_m(M, dtype):
+    W = H.synth_weight(272, 4096, seed=M).to(DEV)          # 17 tiles: the last is ragged
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16+bf16")
+    x = _x(M, 4096, dtype, M)
+    perm = _perm_by_width(enc["nbits"])
+    for p in (None, perm):
+        y = ext.mma_tiles(x, *H.pack_args(enc), perm=p, saturate=False)
+        _check(H.oracle_view(enc), None, x, y, saturate_ref=False)
+
+
+@pytest.mark.parametrize("Q,P,tau", [(1024, 4096, 1e-3), (200, 12288, 1e-3), (130, 768, 2e-3), (96, 2048, 2e-3),
+                                     (64, 5120, 2e-3), (40, 17408, 2e-3), (24, 28672, 2e-3), (16, 128, 1e-3), (3, 256, 1e-3)])
+def test_mma_shapes(Q, P, tau):
+    W = H.synth_weight(Q, P, seed=P).to(DEV)
+    enc = PK.encode_tensor(W, tau, restore="fp16+bf16")
+    perm = _perm_by_width(enc["nbits"])
+    for M, dtype in ((1, torch.bfloat16), (16, torch.float16), (24, torch.bfloat16)):
+        x = _x(M, P, dtype, Q)
+        y = ext.mma_tiles(x, *H.pack_args(enc), perm=perm, saturate=False)
+        _check(H.oracle_view(enc), None, x, y, saturate_ref=False)
+
+
+@pytest.mark.parametrize("Q,P,widths", [(40, 2176, [4, 5, 6, 7, 8]), (35, 128, list(range(1, 15))), (33, 4096, [7, 9, 6, 3]),
+                                        (20, 6144, [7, 3, 12]), (64, 1024, [8]), (48, 1024, [4])])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mma_mixed_widths_and_per_element_rows(Q, P, widths, dtype):
+    d = H.mixed_width_pack(Q, P, widths, seed=11)
+    args = H.to_device_args(d, DEV)
+    for M in (1, 7, 20):
+        x = _x(M, P, dtype, 3)
+        for perm in (None, _perm_by_width(args[2])):
+            y = ext.mma_tiles(x, *args, perm=perm, saturate=False)
+            _check(d, None, x, y, saturate_ref=False)
+
+
+def test_mma_escapes_and_determinism():
+    W = H.synth_weight(128, 4096, seed=11).to(DEV)
+    W[3, 17] = 1.5
+    W[3, 4000] = -2.0
+    W[90, 0] = 0.8
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16", max_nbits=7, force_escapes=[5 * 4096 + 9, 5 * 4096 + 10])
+    assert enc["esc_idx"].numel() >= 5
+    for M in (1, 12, 40):
+        x = _x(M, 4096, torch.bfloat16, 5)
+        y1 = ext.mma_tiles(x, *H.pack_args(enc), saturate=False)
+        y2 = ext.mma_tiles(x, *H.pack_args(enc), saturate=False)
+        assert torch.equal(y1, y2)
+        _check(H.oracle_view(enc), None, x, y1, saturate_ref=False)
+
+
+def test_mma_multi_reference_signature():
+    W = H.synth_weight(256, 1024, seed=4).to(DEV)
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16+bf16")
+    perm = _perm_by_width(enc["nbits"])
+    tile_nb = torch.zeros((256 + 15) // 16, dtype=torch.int32, device=DEV)
+    x32 = torch.randn(9, 1024, device=DEV) * 3
+    x32[0, 0] = 1e6                                            # saturates in fp16 mode
+    y = ext.mma_multi(x32, *H.pack_args(enc), perm, tile_nb)
+    _check(H.oracle_view(enc), None, x32, y, saturate_ref=True)
+    xb = x32.bfloat16()
+    yb = ext.mma_multi(xb, *H.pack_args(enc, bf16_table=True), perm, tile_nb, True, None, 0)
+    _check(H.oracle_view(enc, bf16_table=True), None, xb, yb, saturate_ref=False)
+    with pytest.raises(RuntimeError, match="outside 1..48"):
+        ext.mma_multi(torch.randn(49, 1024, device=DEV), *H.pack_args(enc), perm, tile_nb)
+    Wodd = H.synth_weight(16, 192, seed=1).to(DEV)
+    eo = PK.encode_tensor(Wodd, 1e-3)
+    with pytest.raises(RuntimeError, match="P%128==0"):
+        ext.mma_multi(torch.randn(2, 192, device=DEV), *H.pack_args(eo), None, None)
