@@ -95,13 +95,14 @@ enum qvb8_mma_flags {
                                  multiply); without it bf16 X is used as it is (the reference's bf16 mode) */
 };
 
-/* Row records of the matrix-core path: one u64 per row, in tile order (position i describes row perm[i], or row i
- * when perm is NULL).  Built once per weight (at load) and passed to every qvb8_mma call, so that a call never
- * chases perm -> nbits/bit_off before it can request ids.  Counterpart of the per-weight launch metadata the
+/* Row records of the matrix-core path: qvb8_mma_rowinfo_bytes(Q) bytes (24 per row, 8-byte aligned), in tile order
+ * (position i describes row perm[i], or row i when perm is NULL): where the row's ids start and how wide they are,
+ * then tau_s, min_s and the output row.  Built once per weight (at load) and passed to every qvb8_mma call, so that
+ * a call never chases perm -> nbits/bit_off before it can request ids.  Counterpart of the per-weight launch metadata the
  * reference computes once in QVBandLinearV8._mma_order  formats/qvb8/module.py:230-277 (perm, tile_nb). */
 int64_t qvb8_mma_rowinfo_bytes(int64_t Q);
-int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, const int32_t* perm, int64_t Q, int64_t P,
-                     int64_t ids_bytes, uint64_t* rowinfo, void* stream);
+int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, const float* tau_s, const float* min_s,
+                     const int32_t* perm, int64_t Q, int64_t P, int64_t ids_bytes, uint64_t* rowinfo, void* stream);
 
 /* Workspace qvb8_mma needs when it is called WITHOUT row records (it then builds them itself first). */
 int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);

@@ -21,6 +21,9 @@ SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_scatter_e
 
 
 def lib_path() -> str:
+    override = os.environ.get("QVB8_AMD_LIB")          # a differently built library, for experiments
+    if override:
+        return override
     return os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libqvb8_amd.so")
 
 
@@ -56,7 +59,7 @@ def load(build_if_missing: bool = True):
     lib.qvb8_mma_workspace_bytes.restype = i64
     lib.qvb8_mma_rowinfo_bytes.argtypes = [i64]
     lib.qvb8_mma_rowinfo_bytes.restype = i64
-    lib.qvb8_mma_prepare.argtypes = [vp, vp, vp, i64, i64, i64, vp, vp]
+    lib.qvb8_mma_prepare.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, vp]
     lib.qvb8_mma.argtypes = [vp, i32, i64, vp, i64, vp, vp, vp, vp, i64, i64, vp, vp, i64, vp, vp, i32, vp, vp, i64, vp]
     for name in SYMBOLS:
         getattr(lib, name)                           # every declared symbol must be exported

@@ -51,34 +51,39 @@ template <> struct Fmt<true> {           // bf16: 0x4300 | id == 128 + id for id
     static __device__ __forceinline__ float to_f32(uint32_t h) { return bf16_bits_to_f32(h); }
 };
 
-// Per-row record of the tile kernel, one u64 per row in TILE ORDER (position -> row through `perm`):
-//   bits 0..47 absolute bit offset of the row's first id | bits 48..55 width | bits 56..57 kind
-//   kind 0: the metadata points outside the buffer (the row yields NaN), 1: dword-aligned row of width 4..8
-//   (sliced path), 2: anything else that is in bounds (read element by element), 3: no such row
+// Row records of the tile kernel, in TILE ORDER (position -> row through `perm`), two arrays back to back:
+//   loc[pos]  u64   bits 0..47 absolute bit offset of the row's first id | bits 48..55 width | bits 56..57 kind
+//             kind 0: the metadata points outside the buffer (the row yields NaN), 1: dword-aligned row of width
+//             4..8 (sliced path), 2: anything else that is in bounds (read element by element), 3: no such row
+//   fin[pos]  4 x u32   tau_s bits, min_s bits, output row q (or 0xffffffff), 0 -- what the end of a tile needs
+// loc has Q rounded up to even entries, so that fin is 16-byte aligned.
 constexpr uint64_t kRowOffMask = (1ull << 48) - 1;
+__host__ __device__ inline size_t rowinfo_loc_words(int64_t Q) { return (size_t)((Q + 1) & ~(int64_t)1); }
 
 struct TileArgs {
     const uint16_t* X;            // (M, P) fp16 or bf16 bits
-    const uint8_t* ids; const float* min_s; const float* tau_s;
-    const uint64_t* rowinfo;      // [Q] row records in tile order
-    const int32_t* perm;          // position -> row, or null
+    const uint8_t* ids;
+    const uint64_t* loc;          // row records, see above
+    const uint4* fin;
     float* Y;                     // (M, Q) fp32
     int64_t ids_bytes;
     int M, Q, P;
     int n_steps;                  // P / 128
     int W, G, panels;             // waves per tile, tile groups per workgroup, column panels
     int TW;                       // tiles per workgroup (multiple of G)
-    unsigned long long* dbg;      // DEBUG timestamps
 };
 
 __global__ void __launch_bounds__(256) rowinfo_kernel(const uint8_t* __restrict__ nbits, const int64_t* __restrict__ bit_off,
+                                                      const float* __restrict__ tau_s, const float* __restrict__ min_s,
                                                       const int32_t* __restrict__ perm, int Q, int P, int64_t ids_bytes,
-                                                      uint64_t* __restrict__ out) {
+                                                      uint64_t* __restrict__ loc, uint4* __restrict__ fin) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= Q) return;
     const int q = perm ? perm[i] : i;
     uint64_t rec = 0;
+    uint4 f = {0u, 0u, 0xffffffffu, 0u};
     if (q >= 0 && q < Q) {
+        f = uint4{__float_as_uint(tau_s[q]), __float_as_uint(min_s[q]), (uint32_t)q, 0u};
         const int nb = nbits[q];
         const int64_t bit0 = bit_off[q];
         const int64_t row_bits = (int64_t)nb * P;
@@ -86,7 +91,8 @@ __global__ void __launch_bounds__(256) rowinfo_kernel(const uint8_t* __restrict_
         const uint64_t kind = !ok ? 0 : ((bit0 & 31) == 0 && nb >= 4 && nb <= 8) ? 1 : 2;
         rec = (ok ? (uint64_t)bit0 : 0) | ((uint64_t)nb << 48) | (kind << 56);
     }
-    out[i] = rec;
+    loc[i] = rec;
+    fin[i] = f;
 }
 
 // the 16 pairs of a lane's slice -> 4 operand registers for each of the 4 MFMA steps, stage by stage: all
@@ -134,95 +140,90 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
     for (int p = 0; p < 16; ++p) bt[p / 4][p % 4] = (e[p] << 6) & kTopBitBits;
 }
 
-// NT = token tiles of 16 (M <= 16 * NT); T = steps of 128 columns a wave owns per panel; BF = bf16 operands
+// NT = token tiles of 16 (M <= 16 * NT); T = steps of 128 columns a wave owns per panel; BF = bf16 operands.
+//
+// Wave (g, wc) of a workgroup owns column range wc (T steps; further ranges in later panels) of the tiles of group
+// g.  Its activations for that range stay in registers for the whole panel.  Per tile it requests its T slices in
+// one burst (2T loads), turns them into MFMA operands as they arrive, and puts its partial sums into its own LDS
+// slots.  After one barrier the whole workgroup combines the column ranges of each row in a fixed order.
 template <int NT, int T, bool BF>
 __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
     using F = Fmt<BF>;
-    constexpr int D = 4;                                   // steps in flight per wave
     constexpr int TM = 16 * NT;
     extern __shared__ __align__(16) unsigned char smem[];
     const int rows_cap = a.TW * kTileRows;
-    const int ranges = a.W;                                             // partial-sum slots per row: one per wave of the tile, panels add up in place
-    const int wave_rows = (a.TW / a.G) * kTileRows;                     // rows a wave ever touches
+    const int ranges = a.W;                                   // partial-sum slots per row: one per wave of the tile; panels add up in place
+    const int wave_rows = (a.TW / a.G) * kTileRows;           // rows a wave ever touches
     const int n_waves = a.W * a.G;
-    // LDS: per-wave copies of the row records, epilogue metadata, column-range sums of x, partial sums
-    uint64_t* s_rec = reinterpret_cast<uint64_t*>(smem);                // [n_waves][wave_rows]
-    int32_t* s_q = reinterpret_cast<int32_t*>(s_rec + (size_t)n_waves * wave_rows);   // [rows_cap] output row or -1
-    float* s_ts = reinterpret_cast<float*>(s_q + rows_cap);
-    float* s_mn = s_ts + rows_cap;
-    float* sxs = s_mn + rows_cap;                                       // [ranges][TM]
-    float* part = sxs + (size_t)ranges * TM;                            // [rows_cap][ranges][TM]
+    // LDS: per-wave copies of the row records, what the end needs per row, column-range sums of x, partial sums
+    uint4* s_fin = reinterpret_cast<uint4*>(smem);                                       // [rows_cap]
+    uint64_t* s_loc = reinterpret_cast<uint64_t*>(s_fin + rows_cap);                     // [n_waves][wave_rows]
+    float* sxs = reinterpret_cast<float*>(s_loc + (size_t)n_waves * wave_rows);          // [ranges][TM]
+    float* part = sxs + (size_t)ranges * TM;                                             // [rows_cap][ranges][TM]
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = wave / a.W, wc = wave - g * a.W;
     const int r = lane & 15, kg = lane >> 4;
-    const int srow0 = blockIdx.x * rows_cap;                            // first position of the workgroup
-    const int rows_here = min(rows_cap, a.Q - srow0);
-    const int tiles_here = (rows_here + kTileRows - 1) / kTileRows;
+    // The workgroup's local tile lt is global tile lt * gridDim.x + blockIdx.x: at any moment the workgroups of the
+    // grid read neighbouring tiles, so the whole chip walks through memory together (spread over all channels).
+    const int total_tiles = (a.Q + kTileRows - 1) / kTileRows;
+    const int tiles_here = (int)blockIdx.x < total_tiles ? min(a.TW, (total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1) : 0;
+    auto local_to_pos = [&](int lrow) { return ((lrow >> 4) * (int)gridDim.x + (int)blockIdx.x) * kTileRows + (lrow & 15); };
     const int n_tiles = tiles_here > g ? (tiles_here - g + a.G - 1) / a.G : 0;    // tiles of this wave's group
-#define TS(k) do { if (a.dbg && tid == 0) a.dbg[blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
-    TS(0);
 
-    // ---- this wave's row records into its own LDS copy (no workgroup barrier: a wave's LDS accesses stay in order) ----
-    uint64_t* my_rec = s_rec + (size_t)wave * wave_rows;
+    // ---- the records of this wave's rows into its own LDS copy (a wave's LDS accesses stay in order, so the copy
+    //      needs no barrier); a position past Q has no row ----
+    uint64_t* my_loc = s_loc + (size_t)wave * wave_rows;
     for (int i = lane; i < n_tiles * kTileRows; i += kWave) {
-        const int tk = i >> 4, rr = i & 15;
-        const int pos = srow0 + (g + a.G * tk) * kTileRows + rr;
-        my_rec[i] = pos < a.Q ? a.rowinfo[pos] : (3ull << 56);
+        const int pos = local_to_pos((g + a.G * (i >> 4)) * kTileRows + (i & 15));
+        my_loc[i] = pos < a.Q ? a.loc[pos] : (3ull << 56);
     }
-    // ---- epilogue metadata, needed only after the final barrier ----
-    for (int i = tid; i < rows_cap; i += blockDim.x) {
-        int q = -1;
-        float ts = 0.f, mn = 0.f;
-        if (i < rows_here) {
-            q = a.perm ? a.perm[srow0 + i] : srow0 + i;
-            if (q >= 0 && q < a.Q) { ts = a.tau_s[q]; mn = a.min_s[q]; } else q = -1;
-        }
-        s_q[i] = q; s_ts[i] = ts; s_mn[i] = mn;
-    }
+    // ---- what the end needs for row `tid`: requested now, parked in registers, put in LDS before the barrier ----
+    uint4 e_fin = {0u, 0u, 0xffffffffu, 0u};
+    if (tid < tiles_here * kTileRows && local_to_pos(tid) < a.Q) e_fin = a.fin[local_to_pos(tid)];
 
     const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
-    uint4 wlo[D], whi[D];
-    uint32_t inf[D];                                     // width | kind << 8 of the lane's row, per slot
-    int step0 = 0;                                       // first global step of this wave in the current panel
-    bool active = false;
-    // Requests the lane's slice of flat step i = tile_k * T + it of the current panel.  Always exactly two
-    // loads, never under a branch, from addresses inside the buffer.
-    auto issue = [&](int slot, int i) {
-        const int tk = i / T, it = i - tk * T;
-        const bool in_range = active && tk < n_tiles && (step0 + it) < a.n_steps;
-        const uint64_t rec = in_range ? my_rec[tk * kTileRows + r] : (3ull << 56);
+    int step0 = 0;                                            // first global step of this wave in the current panel
+    // Requests the lane's slices of all T steps of the wave's tile number tk: 2T loads, none under a branch, all from
+    // addresses inside the buffer (lanes whose row is not sliced, and steps past the end of the row, read the first
+    // 32 bytes of `ids`).  Returns width | 1 << 8 for a sliced row, 0 otherwise.
+    auto issue_tile = [&](int tk, uint4 (&wlo)[T], uint4 (&whi)[T]) -> uint32_t {
+        const uint64_t rec = my_loc[tk * kTileRows + r];
         const uint32_t nb = (uint32_t)(rec >> 48) & 0xFFu, kind = (uint32_t)(rec >> 56) & 3u;
-        const bool sliced = kind == 1u && nb <= 8u && (BF || nb <= (uint32_t)F::max_nb);
-        const uint64_t off = sliced ? ((rec & kRowOffMask) >> 3) + (uint64_t)((step0 + it) * 4 + kg) * (4u * nb) : 0;
-        const uint32_t tail = sliced ? 4u * (nb - 4u) : 16u;
-        inf[slot] = nb | ((sliced ? 1u : kind == 1u ? 2u : kind) << 8);
-        wlo[slot] = *reinterpret_cast<const uint4*>(a.ids + off);
-        whi[slot] = *reinterpret_cast<const uint4*>(a.ids + off + tail);
+        const bool row_sliced = kind == 1u;
+        const uint64_t row_off = ((rec & kRowOffMask) >> 3) + (uint64_t)(step0 * 4 + kg) * (4u * nb);
+        const uint32_t step_bytes = 16u * nb;
+        const uint32_t tail = row_sliced ? 4u * (nb - 4u) : 16u;
+#pragma unroll
+        for (int it = 0; it < T; ++it) {
+            const bool use = row_sliced && (step0 + it) < a.n_steps;
+            const uint64_t off = use ? row_off + (uint64_t)it * step_bytes : 0;
+            wlo[it] = *reinterpret_cast<const uint4*>(a.ids + off);
+            whi[it] = *reinterpret_cast<const uint4*>(a.ids + off + tail);
+        }
+        return row_sliced ? (nb | (1u << 8)) : 0u;
     };
 
     for (int panel = 0; panel < a.panels; ++panel) {
         step0 = (panel * a.W + wc) * T;
-        active = step0 < a.n_steps;                                   // wave-uniform
+        const bool active = step0 < a.n_steps;                          // wave-uniform
         const int range = wc;
         const bool first_panel = panel == 0;
+        const int n_mine = active ? n_tiles : 0;
 
+        uint4 wlo[T], whi[T];
+        uint32_t info = 0;
         // ---- activations of this wave's columns, in MFMA operand layout: lane (t = l % 16, kg) holds
-        //      X[16*nt + t][128*(step0+it) + 32*kg + 8*j + 0..7].  Requested before the ids: they are few and
-        //      everything below waits for them ----
+        //      X[16*nt + t][128*(step0+it) + 32*kg + 8*j + 0..7] ----
         v4u_t xa[NT][T][4];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int it = 0; it < T; ++it)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) xa[nt][it][j] = v4u_t{0, 0, 0, 0};
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             const int t = nt * 16 + r;
 #pragma unroll
             for (int it = 0; it < T; ++it) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xa[nt][it][j] = v4u_t{0, 0, 0, 0};
                 if (active && t < a.M && (step0 + it) < a.n_steps) {
                     const uint16_t* xp = a.X + (size_t)t * a.P + (size_t)(step0 + it) * kStepCols + kg * 32;
 #pragma unroll
@@ -233,9 +234,6 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
                 }
             }
         }
-#pragma unroll
-        for (int s = 0; s < D; ++s) issue(s, s);
-
         // sums of x over the wave's columns: the product with a matrix of ones, in the accumulator layout
         // (lane (row r, token group kg) register e <-> token 4*kg + e; identical for every r)
         const v4u_t ones = {F::one_bits, F::one_bits, F::one_bits, F::one_bits};
@@ -257,122 +255,122 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
                     *dst = first_panel ? sx[nt][e] : *dst + sx[nt][e];
                 }
         }
-        if (panel == 0) TS(2);
+        // The first tile's ids are requested only now: the few activation requests above must not queue up behind
+        // the flood of id requests of the whole chip (measured: asking for the ids first costs about a microsecond).
+        if (n_mine > 0) info = issue_tile(0, wlo, whi);
 
-        const int n_flat = active ? n_tiles * T : 0;
-        const int n_iter = (n_flat + D - 1) / D;
-        v4f_t acc[NT], acc_top[NT];
+        for (int tk = 0; tk < n_mine; ++tk) {
+            v4f_t acc[NT], acc_top[NT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) { acc[nt] = v4f_t{0.f, 0.f, 0.f, 0.f}; acc_top[nt] = v4f_t{0.f, 0.f, 0.f, 0.f}; }
-        for (int itr = 0; itr < n_iter; ++itr) {
+            for (int nt = 0; nt < NT; ++nt) { acc[nt] = v4f_t{0.f, 0.f, 0.f, 0.f}; acc_top[nt] = v4f_t{0.f, 0.f, 0.f, 0.f}; }
+            const uint32_t nb = info & 0xFFu;
+            const bool sliced = (info >> 8) == 1u;
+            const uint32_t info0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
+            const bool uniform = __builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u && !(BF && (info0 & 0xFFu) == 8u);
 #pragma unroll
-            for (int s = 0; s < D; ++s) {
-                static_assert(D % T == 0, "a slot always holds the same step of a tile");
-                const int i = itr * D + s;
-                const int it = s % T;                              // compile-time after unrolling
-                const int tk = itr * (D / T) + s / T;
-                // ---- decode the slot: one pass per width present in the tile ----
-                const uint32_t info = inf[s];
-                const uint32_t nb = info & 0xFFu;
-                const bool sliced = (info >> 8) == 1u;
+            for (int it = 0; it < T; ++it) {
                 v4u_t b[4];
+                const uint4 lo = wlo[it], hi = whi[it];
+                if (uniform) {
+                    switch (info0 & 0xFFu) {
+                        case 7: decode_slice<7, BF>(lo, hi, b); break;
+                        case 6: decode_slice<6, BF>(lo, hi, b); break;
+                        case 5: decode_slice<5, BF>(lo, hi, b); break;
+                        case 4: decode_slice<4, BF>(lo, hi, b); break;
+                        default: decode_slice<8, BF>(lo, hi, b); break;
+                    }
+                } else {
+                    // mixed tile: one pass per width present; lanes without a sliced row multiply id 0
 #pragma unroll
-                for (int j = 0; j < 4; ++j) b[j] = v4u_t{F::bias_bits, F::bias_bits, F::bias_bits, F::bias_bits};
-                const uint4 lo = wlo[s], hi = whi[s];
-                if (__builtin_amdgcn_ballot_w64(sliced && nb == 7)) { if (sliced && nb == 7) decode_slice<7, BF>(lo, hi, b); }
-                if (__builtin_amdgcn_ballot_w64(sliced && nb == 6)) { if (sliced && nb == 6) decode_slice<6, BF>(lo, hi, b); }
-                if (__builtin_amdgcn_ballot_w64(sliced && nb == 5)) { if (sliced && nb == 5) decode_slice<5, BF>(lo, hi, b); }
-                if (__builtin_amdgcn_ballot_w64(sliced && nb == 4)) { if (sliced && nb == 4) decode_slice<4, BF>(lo, hi, b); }
-                const bool any8 = __builtin_amdgcn_ballot_w64(sliced && nb == 8) != 0;
-                if (any8) {
-                    if (sliced && nb == 8) decode_slice<8, BF>(lo, hi, b);
-                    if constexpr (BF) {
-                        v4u_t bt[4];
+                    for (int j = 0; j < 4; ++j) b[j] = v4u_t{F::bias_bits, F::bias_bits, F::bias_bits, F::bias_bits};
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 7)) { if (sliced && nb == 7) decode_slice<7, BF>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 6)) { if (sliced && nb == 6) decode_slice<6, BF>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 5)) { if (sliced && nb == 5) decode_slice<5, BF>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 4)) { if (sliced && nb == 4) decode_slice<4, BF>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 8)) {
+                        if (sliced && nb == 8) decode_slice<8, BF>(lo, hi, b);
+                        if constexpr (BF) {
+                            v4u_t bt[4];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) bt[j] = v4u_t{0, 0, 0, 0};
-                        if (sliced && nb == 8) decode_slice8_top(lo, hi, bt);
+                            for (int j = 0; j < 4; ++j) bt[j] = v4u_t{0, 0, 0, 0};
+                            if (sliced && nb == 8) decode_slice8_top(lo, hi, bt);
 #pragma unroll
-                        for (int nt = 0; nt < NT; ++nt)
+                            for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) acc_top[nt] = F::mfma(xa[nt][it][j], bt[j], acc_top[nt]);
+                                for (int j = 0; j < 4; ++j) acc_top[nt] = F::mfma(xa[nt][it][j], bt[j], acc_top[nt]);
+                        }
                     }
                 }
-                issue(s, i + D);
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) acc[nt] = F::mfma(xa[nt][it][j], b[j], acc[nt]);
-                if (it == T - 1 && i < n_flat) {
-                    // ---- tile done for this wave: remove the bias, store into the wave's own LDS slots ----
-                    const int lrow = (g + a.G * tk) * kTileRows + r;
+            }
+            // the next tile's ids are requested before this tile's sums are put away
+            if (tk + 1 < n_mine) info = issue_tile(tk + 1, wlo, whi);
+
+            // ---- tile done for this wave: remove the bias, store into the wave's own LDS slots ----
+            const int lt = g + a.G * tk;                                // the workgroup's local tile
+            const int lrow = lt * kTileRows + r;
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
+            for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int t = nt * 16 + kg * 4 + e;
-                            float v = __builtin_fmaf(-F::bias, sx[nt][e], acc[nt][e]);
-                            if constexpr (BF) v = __builtin_fmaf(kTopBitScale, acc_top[nt][e], v);
-                            if (t < a.M) {
-                                float* dst = part + ((size_t)lrow * ranges + range) * TM + t;
-                                *dst = first_panel ? v : *dst + v;
-                            }
-                        }
-                        acc[nt] = v4f_t{0.f, 0.f, 0.f, 0.f};
-                        acc_top[nt] = v4f_t{0.f, 0.f, 0.f, 0.f};
+                for (int e = 0; e < 4; ++e) {
+                    const int t = nt * 16 + kg * 4 + e;
+                    float v = __builtin_fmaf(-F::bias, sx[nt][e], acc[nt][e]);
+                    if constexpr (BF) v = __builtin_fmaf(kTopBitScale, acc_top[nt][e], v);
+                    if (t < a.M) {
+                        float* dst = part + ((size_t)lrow * ranges + range) * TM + t;
+                        *dst = first_panel ? v : *dst + v;
                     }
-                    // rows the sliced path cannot read: redo them element by element
-                    const uint32_t kind_here = (uint32_t)(my_rec[tk * kTileRows + r] >> 56) & 3u;   // of row r of this tile
-                    const uint32_t nb_here = (uint32_t)(my_rec[tk * kTileRows + r] >> 48) & 0xFFu;
-                    uint64_t odd = __builtin_amdgcn_ballot_w64(kg == 0 && (kind_here == 0u || kind_here == 2u || (kind_here == 1u && nb_here > 8u)));
-                    while (odd) {
-                        const int rr = __builtin_ctzll(odd);
-                        odd &= odd - 1;
-                        const int lr2 = (g + a.G * tk) * kTileRows + rr;
-                        const uint64_t rec = my_rec[tk * kTileRows + rr];
-                        const int nb2 = (int)((rec >> 48) & 0xFFu);
-                        const bool readable = ((rec >> 56) & 3u) != 0u;
-                        const int64_t bit0 = (int64_t)(rec & kRowOffMask);
-                        const int c_lo = step0 * kStepCols, c_hi = min(a.P, (step0 + T) * kStepCols);
-                        for (int t = 0; t < a.M; ++t) {
-                            float sacc = 0.f;
-                            if (readable) {
-                                for (int c = c_lo + lane; c < c_hi; c += kWave) {
-                                    const float idf = (float)load_field(a.ids, bit0 + (int64_t)c * nb2, nb2, clamp_byte);
-                                    sacc = __builtin_fmaf(F::to_f32(a.X[(size_t)t * a.P + c]), idf, sacc);
-                                }
-                            } else {
-                                sacc = __builtin_nanf("");
-                            }
-                            const float tot = wave_sum(sacc);
-                            if (lane == 0) {
-                                // the sliced pass stored this wave's value for the row already (zero contribution plus earlier panels): add to it
-                                part[((size_t)lr2 * ranges + range) * TM + t] += tot;
-                            }
+                }
+            }
+            // rows the sliced path cannot read: redo them element by element
+            const uint32_t kind_here = (uint32_t)(my_loc[tk * kTileRows + r] >> 56) & 3u;
+            uint64_t odd = __builtin_amdgcn_ballot_w64(kg == 0 && (kind_here == 0u || kind_here == 2u));
+            while (odd) {
+                const int rr = __builtin_ctzll(odd);
+                odd &= odd - 1;
+                const int lr2 = lt * kTileRows + rr;
+                const uint64_t rec = my_loc[tk * kTileRows + rr];
+                const int nb2 = (int)((rec >> 48) & 0xFFu);
+                const bool readable = ((rec >> 56) & 3u) != 0u;
+                const int64_t bit0 = (int64_t)(rec & kRowOffMask);
+                const int c_lo = step0 * kStepCols, c_hi = min(a.P, (step0 + T) * kStepCols);
+                for (int t = 0; t < a.M; ++t) {
+                    float sacc = 0.f;
+                    if (readable) {
+                        for (int c = c_lo + lane; c < c_hi; c += kWave) {
+                            const float idf = (float)load_field(a.ids, bit0 + (int64_t)c * nb2, nb2, clamp_byte);
+                            sacc = __builtin_fmaf(F::to_f32(a.X[(size_t)t * a.P + c]), idf, sacc);
                         }
+                    } else {
+                        sacc = __builtin_nanf("");
                     }
+                    const float tot = wave_sum(sacc);
+                    // the sliced pass stored this wave's value for the row already (zero contribution plus earlier panels)
+                    if (lane == 0) part[((size_t)lr2 * ranges + range) * TM + t] += tot;
                 }
             }
         }
     }
-    TS(3);
+    if (tid < rows_cap) s_fin[tid] = e_fin;
     __syncthreads();
-    TS(4);
 
-    // ---- epilogue: combine the column ranges of each row in ascending order ----
-    for (int i = tid; i < rows_here * a.M; i += blockDim.x) {
+    // ---- combine the column ranges of each row in ascending order ----
+    const int all_ranges = (a.n_steps + T - 1) / T;
+    const int valid_ranges = all_ranges < ranges ? all_ranges : ranges;      // waves without any column never stored
+    for (int i = tid; i < tiles_here * kTileRows * a.M; i += blockDim.x) {
         const int rl = i / a.M, t = i - rl * a.M;
-        const int q = s_q[rl];
-        if (q < 0) continue;
+        const uint4 f = s_fin[rl];
+        if (f.z >= (uint32_t)a.Q) continue;
         double dsum = 0.0, xsum = 0.0;
-        const int all_ranges = (a.n_steps + T - 1) / T;
-        const int valid_ranges = all_ranges < ranges ? all_ranges : ranges;      // waves without any column never stored
         for (int w = 0; w < valid_ranges; ++w) {
             dsum += (double)part[((size_t)rl * ranges + w) * TM + t];
             xsum += (double)sxs[w * TM + t];
         }
-        a.Y[(size_t)t * a.Q + q] = (float)((double)s_ts[rl] * dsum + (double)s_mn[rl] * xsum);
+        a.Y[(size_t)t * a.Q + f.z] = (float)((double)__uint_as_float(f.x) * dsum + (double)__uint_as_float(f.y) * xsum);
     }
-    TS(5);
 }
 
 // Escape correction for any M: one thread per (output row with escapes, token), ascending order, no atomics.
@@ -425,10 +423,11 @@ bool plan_tile(int NT, int T, int64_t Q, int64_t P, TilePlan& pl) {
     int64_t tw = (tiles + target - 1) / target;
     tw = (tw + pl.G - 1) / pl.G * pl.G;
     if (tw < pl.G) tw = pl.G;
+    while (tw > pl.G && tw * kTileRows > pl.threads) tw -= pl.G;     // the end needs one thread per row of the workgroup
     const size_t TM = 16 * (size_t)NT, rg = (size_t)pl.W;
     for (;;) {
         const size_t rows = (size_t)tw * kTileRows;
-        pl.lds = (size_t)pl.W * pl.G * (tw / pl.G) * kTileRows * 8 + rows * 3 * 4 + rg * TM * 4 + rows * rg * TM * 4;
+        pl.lds = rows * 16 + (size_t)pl.W * pl.G * (tw / pl.G) * kTileRows * 8 + rg * TM * 4 + rows * rg * TM * 4;
         if (pl.lds <= kTileLdsLimit || tw <= pl.G) break;
         tw -= pl.G;
     }
@@ -453,15 +452,16 @@ int launch_tile(TileArgs& a, hipStream_t s) {
 }
 }  // namespace
 
-extern "C" int64_t qvb8_mma_rowinfo_bytes(int64_t Q) { return Q > 0 ? 8 * Q : 0; }
+extern "C" int64_t qvb8_mma_rowinfo_bytes(int64_t Q) { return Q > 0 ? (int64_t)(rowinfo_loc_words(Q) * 8 + (size_t)Q * 16) : 0; }
 
-extern "C" int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, const int32_t* perm, int64_t Q, int64_t P,
-                                int64_t ids_bytes, uint64_t* rowinfo, void* stream) {
+extern "C" int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, const float* tau_s, const float* min_s,
+                                const int32_t* perm, int64_t Q, int64_t P, int64_t ids_bytes, uint64_t* rowinfo, void* stream) {
     if (Q < 0 || P < 0 || Q > 0x7fffffff || P > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8_mma_prepare: Q or P out of range");
     if (Q == 0) return QVB8_OK;
-    if (!nbits || !bit_off || !rowinfo) return host::fail(QVB8_ERR_ARG, "qvb8_mma_prepare: null pointer");
+    if (!nbits || !bit_off || !tau_s || !min_s || !rowinfo) return host::fail(QVB8_ERR_ARG, "qvb8_mma_prepare: null pointer");
     hipLaunchKernelGGL(rowinfo_kernel, dim3((unsigned)((Q + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       nbits, bit_off, perm, (int)Q, (int)P, ids_bytes, rowinfo);
+                       nbits, bit_off, tau_s, min_s, perm, (int)Q, (int)P, ids_bytes, rowinfo,
+                       reinterpret_cast<uint4*>(rowinfo + rowinfo_loc_words(Q)));
     return host::check_launch("qvb8_mma_prepare");
 }
 
@@ -488,19 +488,15 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     if (!X || !Y || !ids || !min_s || !tau_s || !nbits || !bit_off) return host::fail(QVB8_ERR_ARG, "qvb8_mma: null pointer");
     if (reinterpret_cast<uintptr_t>(X) & 15u) return host::fail(QVB8_ERR_ARG, "qvb8_mma: X must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
-    unsigned long long* dbg = nullptr;
     if (!rowinfo) {
         if (!workspace || workspace_bytes < qvb8_mma_rowinfo_bytes(Q))
             return host::fail(QVB8_ERR_WORKSPACE, "qvb8_mma: without row records the call needs %lld bytes of workspace", (long long)qvb8_mma_rowinfo_bytes(Q));
-        if (int rc = qvb8_mma_prepare(nbits, bit_off, perm, Q, P, ids_bytes, (uint64_t*)workspace, stream)) return rc;
+        if (int rc = qvb8_mma_prepare(nbits, bit_off, tau_s, min_s, perm, Q, P, ids_bytes, (uint64_t*)workspace, stream)) return rc;
         rowinfo = (const uint64_t*)workspace;
-    } else if (workspace && workspace_bytes == -1) {
-        dbg = (unsigned long long*)workspace;       // DEBUG
     }
     TileArgs a;
-    a.X = (const uint16_t*)X; a.ids = ids; a.min_s = min_s; a.tau_s = tau_s; a.rowinfo = rowinfo;
-    a.perm = perm; a.Y = Y; a.ids_bytes = ids_bytes; a.M = (int)M; a.Q = (int)Q; a.P = (int)P; a.n_steps = (int)(P / kStepCols);
-    a.dbg = dbg;
+    a.X = (const uint16_t*)X; a.ids = ids; a.loc = rowinfo; a.fin = reinterpret_cast<const uint4*>(rowinfo + rowinfo_loc_words(Q));
+    a.Y = Y; a.ids_bytes = ids_bytes; a.M = (int)M; a.Q = (int)Q; a.P = (int)P; a.n_steps = (int)(P / kStepCols);
     const bool bf = x_dtype == QVB8_BF16;
     int rc;
     if (M <= 16) rc = bf ? launch_tile<1, 4, true>(a, s) : launch_tile<1, 4, false>(a, s);

@@ -147,12 +147,13 @@ MMA_MAX_M = 48
 MMA_SATURATE_X = 1
 
 
-def mma_prepare(row_nbits, row_bit_off, P, ids_bytes, perm=None):
-    """Row records (int64 tensor of Q words) for mma_tiles: built once per weight."""
+def mma_prepare(row_nbits, row_bit_off, tau_s, min_s, P, ids_bytes, perm=None):
+    """Row records (int64 tensor of qvb8_mma_rowinfo_bytes(Q) bytes) for mma_tiles: built once per weight."""
     lib = _lib.load()
-    _lib.require_cuda(row_nbits, row_bit_off)
+    _lib.require_cuda(row_nbits, row_bit_off, tau_s, min_s)
     Q = row_nbits.numel()
     row_nbits, row_bit_off = row_nbits.contiguous(), row_bit_off.contiguous()
+    tau_s, min_s = tau_s.contiguous(), min_s.contiguous()
     if perm is not None and perm.numel():
         if perm.dtype != torch.int32 or perm.numel() != Q or not perm.is_cuda:
             raise RuntimeError("qvb8 mma-multi: perm must be an int32 GPU tensor of length Q (or empty)")
@@ -160,8 +161,9 @@ def mma_prepare(row_nbits, row_bit_off, P, ids_bytes, perm=None):
     else:
         perm = None
     with torch.cuda.device(row_nbits.device):
-        out = torch.empty(Q, dtype=torch.int64, device=row_nbits.device)
-        _lib._check(lib.qvb8_mma_prepare(_lib.ptr(row_nbits), _lib.ptr(row_bit_off), _lib.ptr(perm), Q, int(P),
+        out = torch.empty(lib.qvb8_mma_rowinfo_bytes(Q) // 8, dtype=torch.int64, device=row_nbits.device)
+        _lib._check(lib.qvb8_mma_prepare(_lib.ptr(row_nbits), _lib.ptr(row_bit_off), _lib.ptr(tau_s), _lib.ptr(min_s),
+                                         _lib.ptr(perm), Q, int(P),
                                          int(ids_bytes), _lib.ptr(out), _lib.stream_of(row_nbits)), lib)
     return out
 
@@ -191,7 +193,8 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
         perm = perm.contiguous()
     else:
         perm = None
-    if rowinfo is not None and (rowinfo.dtype != torch.int64 or rowinfo.numel() != Q or not rowinfo.is_cuda):
+    if rowinfo is not None and (rowinfo.dtype != torch.int64 or rowinfo.numel() * 8 != lib.qvb8_mma_rowinfo_bytes(Q)
+                                or not rowinfo.is_cuda):
         raise RuntimeError("qvb8 mma-multi: rowinfo must be the int64 GPU tensor mma_prepare returned")
     Xc = X.contiguous()
     ids, min_s, tau_s = ids.contiguous(), min_s.contiguous(), tau_s.contiguous()
@@ -200,7 +203,8 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
         Y = torch.empty((M, Q), dtype=torch.float32, device=Xc.device)
         ei = esc_idx.contiguous() if n_esc else None
         ev = esc_vals.contiguous() if n_esc else None
-        ws = None if rowinfo is not None else torch.empty(Q, dtype=torch.int64, device=Xc.device)
+        ws = None if rowinfo is not None else torch.empty(lib.qvb8_mma_workspace_bytes(M, Q, int(P)) // 8,
+                                                          dtype=torch.int64, device=Xc.device)
         _lib._check(lib.qvb8_mma(_lib.ptr(Xc), _lib.dtype_code(Xc.dtype), M, _lib.ptr(ids), ids.numel(),
                                  _lib.ptr(min_s), _lib.ptr(tau_s), _lib.ptr(row_nbits), _lib.ptr(row_bit_off),
                                  Q, int(P), _lib.ptr(ei), _lib.ptr(ev), n_esc, _lib.ptr(perm),
