@@ -91,8 +91,10 @@ int qvb8_gemv(const void* X, int x_dtype, int64_t M,
 /* ---- fused decode + small-M GEMM on the matrix cores, M = 1..48 ------------------------------------------- */
 
 enum qvb8_mma_flags {
-    QVB8_MMA_SATURATE_X = 1   /* bf16 X: values beyond +-65504 count as +-65504 (what the fp16 paths of the reference
-                                 multiply); without it bf16 X is used as it is (the reference's bf16 mode) */
+    QVB8_MMA_SATURATE_X = 1   /* bf16 X is narrowed as saturating_half does (clamp to +-65504, round to fp16, NaN kept) while
+                                 it is loaded, and the product runs on fp16 operands: what the fp16 paths of the reference
+                                 multiply.  Without it bf16 X is used as it is, on bf16 operands (the reference's bf16
+                                 mode).  No effect on fp16 X. */
 };
 
 /* Row records of the matrix-core path: qvb8_mma_rowinfo_bytes(Q) bytes (24 per row, 8-byte aligned), in tile order

@@ -51,6 +51,21 @@ template <> struct Fmt<true> {           // bf16: 0x4300 | id == 128 + id for id
     static __device__ __forceinline__ float to_f32(uint32_t h) { return bf16_bits_to_f32(h); }
 };
 
+// How the kernels read an activation.  XC = false: X is already in the operand format (fp16 for Fmt<false>, bf16 for
+// Fmt<true>).  XC = true (fp16 operands only): X is bf16 in memory and is narrowed on the way in exactly as
+// saturating_half does it -- clamp to +-65504, round to fp16, NaN kept -- so a bf16 caller gets what the fp16 paths of
+// the reference multiply without a separate pass over X.
+template <bool BF, bool XC> struct XIn {
+    static __device__ __forceinline__ float scalar(uint32_t bits) {
+        if constexpr (XC) return f16_bits_to_f32(sat_half_bits(bf16_bits_to_f32(bits)));
+        else return Fmt<BF>::to_f32(bits);
+    }
+    static __device__ __forceinline__ uint32_t pair(uint32_t w) {        // two activations in one dword
+        if constexpr (XC) return sat_half_bits(__uint_as_float(w << 16)) | (sat_half_bits(__uint_as_float(w & 0xFFFF0000u)) << 16);
+        else return w;
+    }
+};
+
 // Row records of the tile kernel, in TILE ORDER (position -> row through `perm`), two arrays back to back:
 //   loc[pos]  u64   bits 0..47 absolute bit offset of the row's first id | bits 48..55 width | bits 56..57 kind
 //             kind 0: the metadata points outside the buffer (the row yields NaN), 1: dword-aligned row of width
@@ -146,9 +161,11 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
 // g.  Its activations for that range stay in registers for the whole panel.  Per tile it requests its T slices in
 // one burst (2T loads), turns them into MFMA operands as they arrive, and puts its partial sums into its own LDS
 // slots.  After one barrier the whole workgroup combines the column ranges of each row in a fixed order.
-template <int NT, int T, bool BF>
+template <int NT, int T, bool BF, bool XC>
 __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
+    static_assert(!(BF && XC), "narrowing on the way in exists for fp16 operands only");
     using F = Fmt<BF>;
+    using XI = XIn<BF, XC>;
     constexpr int TM = 16 * NT;
     extern __shared__ __align__(16) unsigned char smem[];
     const int rows_cap = a.TW * kTileRows;
@@ -229,7 +246,7 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const uint4 v = *reinterpret_cast<const uint4*>(xp + 8 * j);
-                        xa[nt][it][j] = v4u_t{v.x, v.y, v.z, v.w};
+                        xa[nt][it][j] = v4u_t{XI::pair(v.x), XI::pair(v.y), XI::pair(v.z), XI::pair(v.w)};
                     }
                 }
             }
@@ -342,7 +359,7 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
                     if (readable) {
                         for (int c = c_lo + lane; c < c_hi; c += kWave) {
                             const float idf = (float)load_field(a.ids, bit0 + (int64_t)c * nb2, nb2, clamp_byte);
-                            sacc = __builtin_fmaf(F::to_f32(a.X[(size_t)t * a.P + c]), idf, sacc);
+                            sacc = __builtin_fmaf(XI::scalar(a.X[(size_t)t * a.P + c]), idf, sacc);
                         }
                     } else {
                         sacc = __builtin_nanf("");
@@ -374,7 +391,7 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
 }
 
 // Escape correction for any M: one thread per (output row with escapes, token), ascending order, no atomics.
-template <bool BF>
+template <bool BF, bool XC>
 __global__ void __launch_bounds__(256) tile_fix_escapes_kernel(const uint16_t* __restrict__ X, int M,
         const uint8_t* __restrict__ ids, int64_t ids_bytes, const float* __restrict__ min_s, const float* __restrict__ tau_s,
         const uint8_t* __restrict__ nbits, const int64_t* __restrict__ bit_off, const int64_t* __restrict__ esc_idx,
@@ -393,7 +410,7 @@ __global__ void __launch_bounds__(256) tile_fix_escapes_kernel(const uint16_t* _
     for (int64_t e = i; e < n_esc && esc_idx[e] / P == q; ++e) {
         const int c = (int)(esc_idx[e] - q * P);
         const float banded = __builtin_fmaf((float)load_field(ids, bit0 + (int64_t)c * nb, nb, clamp_byte), ts, mn);
-        acc = __builtin_fmaf(Fmt<BF>::to_f32(X[(size_t)t * P + c]), esc_vals[e] - banded, acc);
+        acc = __builtin_fmaf(XIn<BF, XC>::scalar(X[(size_t)t * P + c]), esc_vals[e] - banded, acc);
     }
     Y[(size_t)t * Q + q] += acc;
 }
@@ -437,17 +454,20 @@ bool plan_tile(int NT, int T, int64_t Q, int64_t P, TilePlan& pl) {
     return true;
 }
 
-template <int NT, int T, bool BF>
+template <int NT, int T, bool BF, bool XC>
 int launch_tile(TileArgs& a, hipStream_t s) {
     TilePlan pl;
     if (!plan_tile(NT, T, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
     a.W = pl.W; a.G = pl.G; a.panels = pl.panels; a.TW = pl.TW;
-    static bool attr = false;
-    if (!attr) {
-        (void)hipFuncSetAttribute((const void*)tile_kernel<NT, T, BF>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTileLdsLimit);
-        attr = true;
+    static bool attr[64] = {false};                           // per device: the attribute belongs to the device's copy of the kernel
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: no current device");
+    if (!attr[dev]) {
+        if (hipFuncSetAttribute((const void*)tile_kernel<NT, T, BF, XC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTileLdsLimit) != hipSuccess)
+            return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: cannot raise the kernel's LDS limit");
+        attr[dev] = true;
     }
-    hipLaunchKernelGGL((tile_kernel<NT, T, BF>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s, a);
+    hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s, a);
     return host::check_launch("qvb8_mma");
 }
 }  // namespace
@@ -476,7 +496,6 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
                         const int64_t* esc_idx, const float* esc_vals, int64_t n_esc,
                         const int32_t* perm, const uint64_t* rowinfo, int flags, float* Y,
                         void* workspace, int64_t workspace_bytes, void* stream) {
-    (void)flags;
     if (Q < 0 || P < 0 || Q > 0x7fffffff || P > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8_mma: Q or P out of range");
     if (M < 1 || M > 48) return host::fail(QVB8_ERR_ARG, "qvb8 mma-multi: M=%lld outside 1..48", (long long)M);
     if (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16) return host::fail(QVB8_ERR_ARG, "qvb8_mma: X must be fp16 or bf16 (narrow fp32 activations with qvb8_sat_half first)");
@@ -497,16 +516,22 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     TileArgs a;
     a.X = (const uint16_t*)X; a.ids = ids; a.loc = rowinfo; a.fin = reinterpret_cast<const uint4*>(rowinfo + rowinfo_loc_words(Q));
     a.Y = Y; a.ids_bytes = ids_bytes; a.M = (int)M; a.Q = (int)Q; a.P = (int)P; a.n_steps = (int)(P / kStepCols);
-    const bool bf = x_dtype == QVB8_BF16;
+    // mode 0: fp16 X, fp16 operands; 1: bf16 X narrowed to saturated fp16 on the way in, fp16 operands; 2: bf16 operands
+    const int mode = x_dtype == QVB8_F16 ? 0 : (flags & QVB8_MMA_SATURATE_X) ? 1 : 2;
     int rc;
-    if (M <= 16) rc = bf ? launch_tile<1, 4, true>(a, s) : launch_tile<1, 4, false>(a, s);
-    else if (M <= 32) rc = bf ? launch_tile<2, 2, true>(a, s) : launch_tile<2, 2, false>(a, s);
-    else rc = bf ? launch_tile<3, 2, true>(a, s) : launch_tile<3, 2, false>(a, s);
+#define QVB8_TILE_LAUNCH(NT_, T_) (mode == 0 ? launch_tile<NT_, T_, false, false>(a, s) : mode == 1 ? launch_tile<NT_, T_, false, true>(a, s) : launch_tile<NT_, T_, true, false>(a, s))
+    if (M <= 16) rc = QVB8_TILE_LAUNCH(1, 4);
+    else if (M <= 32) rc = QVB8_TILE_LAUNCH(2, 2);
+    else rc = QVB8_TILE_LAUNCH(3, 2);
+#undef QVB8_TILE_LAUNCH
     if (rc) return rc;
     if (n_esc > 0) {
         dim3 grid((unsigned)((n_esc + 255) / 256), (unsigned)M);
-        if (bf) hipLaunchKernelGGL(tile_fix_escapes_kernel<true>, grid, dim3(256), 0, s, (const uint16_t*)X, (int)M, ids, ids_bytes, min_s, tau_s, nbits, bit_off, esc_idx, esc_vals, n_esc, Y, (int)Q, (int)P);
-        else hipLaunchKernelGGL(tile_fix_escapes_kernel<false>, grid, dim3(256), 0, s, (const uint16_t*)X, (int)M, ids, ids_bytes, min_s, tau_s, nbits, bit_off, esc_idx, esc_vals, n_esc, Y, (int)Q, (int)P);
+#define QVB8_FIX_ARGS grid, dim3(256), 0, s, (const uint16_t*)X, (int)M, ids, ids_bytes, min_s, tau_s, nbits, bit_off, esc_idx, esc_vals, n_esc, Y, (int)Q, (int)P
+        if (mode == 0) hipLaunchKernelGGL((tile_fix_escapes_kernel<false, false>), QVB8_FIX_ARGS);
+        else if (mode == 1) hipLaunchKernelGGL((tile_fix_escapes_kernel<false, true>), QVB8_FIX_ARGS);
+        else hipLaunchKernelGGL((tile_fix_escapes_kernel<true, false>), QVB8_FIX_ARGS);
+#undef QVB8_FIX_ARGS
         return host::check_launch("qvb8_mma escapes");
     }
     return QVB8_OK;

@@ -172,8 +172,9 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
               rowinfo=None):
     """Matrix-core path for 1 <= M <= 48 and P % 128 == 0: X (fp16 or bf16) times the fp32 band value, fp32 (M, Q).
     `perm` (int32, position -> row) groups rows of equal width into tiles; `rowinfo` = mma_prepare(...) for the
-    same perm (built on the fly when absent); `saturate` makes bf16 activations beyond +-65504 count as
-    +-65504, as every fp16 path of the reference does."""
+    same perm (built on the fly when absent).  `saturate` (bf16 X only): X is narrowed like saturating_half while it
+    is loaded and the product runs on fp16 operands, as every fp16 path of the reference does; without it bf16 X is
+    multiplied as it is on bf16 operands."""
     lib = _lib.load()
     Q = _check_pack(ids, min_s, row_nbits, row_bit_off, tau_s)
     n_esc = _check_escapes(esc_idx, esc_vals)
@@ -224,7 +225,8 @@ def mma_multi(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
     if bf16:
         Xk = X if X.dtype == torch.bfloat16 else X.to(torch.bfloat16)
         return mma_tiles(Xk, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm, saturate=False)
-    return mma_tiles(saturating_half(X), ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm)
+    Xk = X if X.dtype in (torch.float16, torch.bfloat16) else saturating_half(X)
+    return mma_tiles(Xk, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm, saturate=True)
 
 
 def _forward(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, out_half):

@@ -26,6 +26,7 @@ _MAGIC = b"QVBD"
 _VERSION = 1
 _CALC_FORMULA = 0
 _CALC_TABLE = 1
+CALC_FORMULA, CALC_TABLE = _CALC_FORMULA, _CALC_TABLE
 _SOURCE_CODES = {"bf16": 0, "fp8_block": 1, "q4_block": 2, "fp32": 3}
 _SOURCE_NAMES = {v: k for k, v in _SOURCE_CODES.items()}
 _ESC32_WIDTH = {"bf16": 2, "fp8_block": 2, "q4_block": 2, "fp32": 4}
@@ -87,9 +88,9 @@ def pack_formula(*, Q: int, P: int, tau: float, max_err: float, min_s, tau_s, nb
                      np.zeros(int(Q), "<f4").tobytes()])
 
 
-def unpack_formula(blob: bytes, *, fp16_list=None, where: str = "") -> dict:
+def unpack_formula(blob: bytes, *, skip_bit_decode: bool = True, fp16_list=None, where: str = "") -> dict:
     """Parse a QVBD formula pack.  The ids stay packed (`buf`): they are decoded on the
-    GPU.  esc_idx/esc_vals merge both pools ascending by flat index; esc_idx_fp16 /
+    GPU, whatever `skip_bit_decode` says (accepted for call-site compatibility; `codes` is always None).  esc_idx/esc_vals merge both pools ascending by flat index; esc_idx_fp16 /
     esc_vals_fp16 is the fp16 table (the same list for an fp16 pack, a subset chosen
     by `fp16_list` for an fp16+bf16 pack, None when that list is missing)."""
     Q, P, tau, max_err, source, calc, restore = _unpack_header(blob)

@@ -1,0 +1,114 @@
+"""GPU tests of QVBandLinearV8 (the operator the model adapters call): every dispatch branch against the CPU oracle."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import qvb8_oracle as O
+from qvb8_amd.formats.qvb8 import pack as PK
+from qvb8_amd.formats.qvb8.module import QVBandLinearV8, enable_bf16_gemm, footprint_report
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _ref(enc, x, saturate, bf16_table=False, narrow=None):
+    d = H.oracle_view(enc, bf16_table=bf16_table)
+    Wr = O.reconstruct(d["min_s"], d["tau_s"], H.oracle_ids(d), d["esc_idx"], d["esc_vals"])
+    if narrow == "fp16":
+        Wr = O.narrow_fp16(Wr)
+    elif narrow == "bf16":
+        Wr = O.narrow_bf16(Wr)
+    xs = x.float().cpu().numpy().reshape(-1, x.shape[-1])
+    if saturate:
+        xs = O.sat_half(xs)
+    return O.linear_f64(xs, Wr), Wr, xs
+
+
+def _close(y, ref, Wr, xs, out_dtype):
+    tol = H.gemv_tolerance(ref, Wr, xs)
+    if out_dtype != torch.float32:                       # one more rounding, to the caller's 16-bit dtype
+        eps = 2.0 ** -8 if out_dtype == torch.bfloat16 else 2.0 ** -11
+        tol = tol + eps * np.abs(ref)
+    diff = np.abs(y.float().cpu().numpy().astype(np.float64).reshape(ref.shape) - ref)
+    assert np.all(diff <= tol), (float(diff.max()), float((diff / tol).max()))
+
+
+@pytest.mark.parametrize("M", [1, 4, 8, 16, 48, 60, 96])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_linear_small_m(M, dtype):
+    W = H.synth_weight(200, 1024, seed=3).to(DEV)
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16", force_escapes=[0, 1024 * 7 + 5, 1024 * 199 + 1023])
+    bias = torch.linspace(-1, 1, 200, device=DEV)
+    lin = QVBandLinearV8.from_encoded(enc, bias=bias)
+    g = torch.Generator().manual_seed(M)
+    x = torch.randn(2, M // 2, 1024, generator=g).to(dtype).to(DEV) if M % 2 == 0 else torch.randn(M, 1024, generator=g).to(dtype).to(DEV)
+    y = lin(x)
+    assert y.dtype == dtype and y.shape == (*x.shape[:-1], 200)
+    ref, Wr, xs = _ref(enc, x, saturate=True)
+    _close(y, ref + bias.double().cpu().numpy(), Wr, xs, dtype)
+
+
+def test_linear_without_matrix_core_shape_and_large_m():
+    """P % 128 != 0: GEMV for M <= 8, dense restore + library GEMM above (fp16 restore for fp16 callers)."""
+    W = H.synth_weight(96, 200, seed=5).to(DEV)
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16")
+    lin = QVBandLinearV8.from_encoded(enc)
+    assert lin._mma_order() is None
+    for M, dtype in ((3, torch.bfloat16), (20, torch.float32), (20, torch.float16), (150, torch.bfloat16)):
+        x = torch.randn(M, 200, generator=torch.Generator().manual_seed(M)).to(dtype).to(DEV)
+        y = lin(x)
+        narrow = "fp16" if M > 8 else None                 # above 8 rows the weight is restored to fp16 first
+        ref, Wr, xs = _ref(enc, x, saturate=True, narrow=narrow)
+        _close(y, ref, Wr, xs, dtype)
+    W2 = H.synth_weight(64, 1024, seed=6).to(DEV)
+    lin2 = QVBandLinearV8.from_encoded(PK.encode_tensor(W2, 1e-3, restore="fp16"))
+    x = torch.randn(130, 1024, generator=torch.Generator().manual_seed(1)).to(torch.float16).to(DEV)
+    ref, Wr, xs = _ref(PK.encode_tensor(W2, 1e-3, restore="fp16"), x, saturate=True, narrow="fp16")
+    _close(lin2(x), ref, Wr, xs, torch.float16)
+
+
+def test_bf16_certified_pack_modes():
+    W = H.synth_weight(128, 1024, seed=9).to(DEV)
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16+bf16")
+    lin = QVBandLinearV8.from_encoded(enc)
+    assert lin.bf16_certified and enable_bf16_gemm(lin) == (1, 1)
+    x = torch.randn(16, 1024, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).to(DEV)
+    ref, Wr, xs = _ref(enc, x, saturate=False, bf16_table=True)
+    _close(lin(x), ref, Wr, xs, torch.bfloat16)             # bf16 operands, bf16 escape table
+    xl = torch.randn(128, 1024, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(DEV)
+    ref, Wr, xs = _ref(enc, xl, saturate=False, bf16_table=True, narrow="bf16")
+    _close(lin(xl), ref, Wr, xs, torch.bfloat16)            # M > 96: bf16 restore + one bf16 GEMM
+    rep = footprint_report(lin)
+    assert rep["linears"] == 1 and rep["params"] == 128 * 1024 and rep["bytes_per_param"] < 1.2
+
+
+def test_row_subset_and_dtype_cast_keep_metadata():
+    W = H.synth_weight(300, 512, seed=11).to(DEV)
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16", force_escapes=[512 * 17 + 3, 512 * 250 + 9])
+    lin = QVBandLinearV8.from_encoded(enc)
+    rows = torch.tensor([250, 3, 17, 299, 100], device=DEV)
+    sub = lin.row_subset(rows)
+    assert sub.ids.data_ptr() == lin.ids.data_ptr() and sub.out_features == 5
+    x = torch.randn(2, 512, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16).to(DEV)
+    assert torch.equal(sub(x), lin(x)[:, rows])
+    before = lin.tau_s.clone()
+    lin.to(torch.bfloat16)
+    assert lin.tau_s.dtype == torch.float32 and torch.equal(lin.tau_s, before) and lin.esc_vals.dtype == torch.float32
+
+
+def test_from_packfile_roundtrip(tmp_path):
+    W = H.synth_weight(64, 256, seed=13).to(DEV)
+    for restore, name in (("fp16", "a.qvband"), ("fp16+bf16", "b.qvband"), ("fp16", "c.qvb8")):
+        enc = PK.encode_tensor(W, 1e-3, restore=restore, force_escapes=[5, 256 * 63 + 255])
+        path = os.path.join(tmp_path, name)
+        PK.write_pack(path, enc)
+        lin = QVBandLinearV8.from_packfile(path, device=DEV)
+        ref = QVBandLinearV8.from_encoded(enc)
+        assert lin.bf16_certified == (restore == "fp16+bf16") and not lin.fp16_table_missing
+        for k in ("tau_s", "min_s", "nbits", "bit_off", "ids", "esc_idx", "esc_vals", "esc_idx_bf16", "esc_vals_bf16"):
+            assert torch.equal(getattr(lin, k), getattr(ref, k)), k
+        x = torch.randn(3, 256, generator=torch.Generator().manual_seed(5)).to(torch.float16).to(DEV)
+        assert torch.equal(lin(x), ref(x))

@@ -105,3 +105,25 @@ def test_mma_multi_reference_signature():
     eo = PK.encode_tensor(Wodd, 1e-3)
     with pytest.raises(RuntimeError, match="P%128==0"):
         ext.mma_multi(torch.randn(2, 192, device=DEV), *H.pack_args(eo), None, None)
+
+
+@pytest.mark.parametrize("M", [1, 7, 16, 20, 40])
+def test_mma_bf16_activations_narrowed_on_load(M):
+    """bf16 X with saturate=True: the kernel narrows X like saturating_half (clamp to +-65504, fp16, NaN kept) in
+    registers; the oracle does the same narrowing on the CPU and multiplies the fp32 band value."""
+    W = H.synth_weight(150, 2048, seed=40 + M).to(DEV)
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16", force_escapes=[5, 2048 * 3 + 17, 2048 * 149 + 2047])
+    x = _x(M, 2048, torch.bfloat16, 90 + M)
+    x[0, 3] = 3.0e5                                            # clamps to 65504
+    x[M - 1, 100] = -1.0e30                                    # clamps to -65504
+    x[0, 7] = 1.0e-6                                           # an fp16 subnormal after narrowing
+    perm = _perm_by_width(enc["nbits"])
+    y = ext.mma_tiles(x, *H.pack_args(enc), perm=perm, saturate=True)
+    _check(H.oracle_view(enc), None, x, y, saturate_ref=True)
+    # the unsaturated mode sees the huge activations as they are: the two modes must differ there
+    y2 = ext.mma_tiles(x, *H.pack_args(enc), perm=perm, saturate=False)
+    assert not torch.allclose(y[0], y2[0])
+    xn = x.clone()
+    xn[0, 11] = float("nan")
+    yn = ext.mma_tiles(xn, *H.pack_args(enc), perm=perm, saturate=True)
+    assert torch.isnan(yn[0]).all() and (M == 1 or not torch.isnan(yn[1:]).any())
