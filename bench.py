@@ -27,6 +27,9 @@ HBM_PEAK_GBS = 8000.0
 LAYER_9B = (("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
             ("gate", 12288, 4096), ("up", 12288, 4096), ("down", 4096, 12288))
 TAU = 1e-3
+# HBM bytes per launch of the tile kernel from hardware counters (FETCH_SIZE scaled by 2.0 against a plain 1 GiB pass,
+# plus WRITE_SIZE), as recorded in profiles/tile_kernel_9b_decode_step_hbm_traffic.md: {workgroups: bytes}
+MEASURED_TRAFFIC = {256: (2 * 16078.3 + 39.8) * 1024, 64: (2 * 2014.4 + 4.9) * 1024}
 MMA_FLAGS = int(os.environ.get("QVB8_BENCH_MMA_FLAGS", "1"))     # 1 = QVB8_MMA_SATURATE_X: the operator's default for bf16 x
 
 
@@ -66,8 +69,7 @@ def cpu_baseline(layers, x_by_p, budget_s=12.0):
     import numpy as np
     import torch
     from oracle import qvb8_oracle as O
-    t0 = time.perf_counter()
-    nbytes, done = 0, []
+    nbytes, done, dt = 0, [], 0.0
     for enc in (e for lay in layers for e in lay):
         d = {k: enc[k].cpu().numpy() for k in ("min_s", "tau_s", "nbits", "bit_off", "ids", "esc_idx", "esc_vals")}
         x = x_by_p[enc["P"]].float().cpu()
@@ -76,12 +78,11 @@ def cpu_baseline(layers, x_by_p, budget_s=12.0):
         Wr = O.reconstruct(d["min_s"], d["tau_s"], ids, d["esc_idx"], d["esc_vals"])
         y = x @ torch.from_numpy(Wr).T
         assert y.shape == (1, enc["Q"])
-        t0 += t1 - t0 if not done else 0.0               # the clock starts at the first restore, after the copies to host
+        dt += time.perf_counter() - t1                   # restore + product only: the copies to host are not CPU work of the path
         nbytes += algorithmic_bytes(enc, 1)
         done.append(enc["name"])
-        if time.perf_counter() - t0 >= budget_s:
+        if dt >= budget_s:
             break
-    dt = time.perf_counter() - t0
     return {"value": round(nbytes / dt / 1e9, 6), "unit": "GB/s", "cores": int(torch.get_num_threads()), "kind": "port",
             "sample": "numpy restore + torch fp32 matmul (M=1) of the first %d projections of the workload (%s; %.1f MB "
                       "packed) in %.1f s; the restore is single-threaded numpy, the matmul uses torch's threads"
@@ -95,6 +96,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain elementwise pass over 1 GiB in and 1 GiB out (torch.add on 2^28 floats): the "
+                         "known-size kernel that hardware byte counters of a profiler run are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU (no collectives are part of it); run with --gpus 1", file=sys.stderr)
@@ -127,6 +131,13 @@ def main():
             if rc != 0:
                 raise RuntimeError(lib.qvb8_last_error().decode())
 
+    if args.copy_probe:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     step()
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
@@ -161,7 +172,9 @@ def main():
                    "launches_per_step": n_launch, "bytes_per_step": step_bytes, "escapes": esc,
                    "bits_per_weight": round(8.0 * sum(e["ids"].numel() for e in flat) / sum(e["Q"] * e["P"] for e in flat), 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": (round(sum(MEASURED_TRAFFIC[256 if e["Q"] >= 4096 else 64] for e in flat) / n_launch)
+                                 if MMA_FLAGS == 1 else None),
                      "kernel": "qvb8::tile_kernel<1,4,false,true>", "bytes_per_launch": step_bytes // n_launch,
                      "launch_us": round(launch_us, 3)},
     }
