@@ -112,3 +112,38 @@ def test_from_packfile_roundtrip(tmp_path):
             assert torch.equal(getattr(lin, k), getattr(ref, k)), k
         x = torch.randn(3, 256, generator=torch.Generator().manual_seed(5)).to(torch.float16).to(DEV)
         assert torch.equal(lin(x), ref(x))
+
+
+def test_same_input_fusion_is_bit_identical():
+    import torch.nn as nn
+    from qvb8_amd.formats.qvb8.fuse import FusedMember, concat_linears, fuse_same_input
+    lins, encs = [], []
+    for i, Q in enumerate((96, 40, 33)):
+        W = H.synth_weight(Q, 512, seed=20 + i).to(DEV)
+        enc = PK.encode_tensor(W, 1e-3, restore="fp16", force_escapes=[3 + i, 512 * (Q - 1) + 500])
+        encs.append(enc)
+        lins.append(QVBandLinearV8.from_encoded(enc, bias=torch.full((Q,), 0.5 * i, device=DEV) if i != 1 else None))
+    fused, splits = concat_linears(lins)
+    assert splits == [96, 136] and fused.out_features == 169 and fused.ids.data_ptr() % 16 == 0
+    for M, dtype in ((1, torch.bfloat16), (12, torch.float16), (70, torch.bfloat16), (120, torch.float16)):
+        x = torch.randn(M, 512, generator=torch.Generator().manual_seed(M)).to(dtype).to(DEV)
+        parts = torch.tensor_split(fused(x), splits, -1)
+        for part, lin in zip(parts, lins):
+            assert torch.equal(part, lin(x)), (M, dtype)
+
+    class Attn(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj, self.k_proj, self.v_proj = lins
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.self_attn = Attn()
+    blk = Block()
+    x = torch.randn(2, 512, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(DEV)
+    want = [lin(x) for lin in lins]
+    assert fuse_same_input(blk) == 1 and isinstance(blk.self_attn.k_proj, FusedMember)
+    got = [blk.self_attn.q_proj(x), blk.self_attn.k_proj(x), blk.self_attn.v_proj(x)]
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    assert blk.self_attn._qvb8_fused._x is None           # every member took its part: nothing is held
