@@ -213,11 +213,12 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
     if (tid < tiles_here * kTileRows && local_to_pos(tid) < a.Q) e_fin = a.fin[local_to_pos(tid)];
 
     const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
-    int step0 = 0;                                            // first global step of this wave in the current panel
+    uint4 wlo[T], whi[T];
+    uint32_t info = 0;
     // Requests the lane's slices of all T steps of the wave's tile number tk: 2T loads, none under a branch, all from
     // addresses inside the buffer (lanes whose row is not sliced, and steps past the end of the row, read the first
     // 32 bytes of `ids`).  Returns width | 1 << 8 for a sliced row, 0 otherwise.
-    auto issue_tile = [&](int tk, uint4 (&wlo)[T], uint4 (&whi)[T]) -> uint32_t {
+    auto issue_tile = [&](int tk, int step0, uint4 (&wlo)[T], uint4 (&whi)[T]) -> uint32_t {
         const uint64_t rec = my_loc[tk * kTileRows + r];
         const uint32_t nb = (uint32_t)(rec >> 48) & 0xFFu, kind = (uint32_t)(rec >> 56) & 3u;
         const bool row_sliced = kind == 1u;
@@ -235,14 +236,13 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
     };
 
     for (int panel = 0; panel < a.panels; ++panel) {
-        step0 = (panel * a.W + wc) * T;
+        const int step0 = (panel * a.W + wc) * T;             // first global step of this wave in this panel
         const bool active = step0 < a.n_steps;                          // wave-uniform
         const int range = wc;
         const bool first_panel = panel == 0;
         const int n_mine = active ? n_tiles : 0;
-
-        uint4 wlo[T], whi[T];
-        uint32_t info = 0;
+        const int step0_next = step0 + a.W * T;
+        const bool more = n_mine > 0 && panel + 1 < a.panels && step0_next < a.n_steps;
         // ---- activations of this wave's columns, in MFMA operand layout: lane (t = l % 16, kg) holds
         //      X[16*nt + t][128*(step0+it) + 32*kg + 8*j + 0..7] ----
         v4u_t xa[NT][T][4];
@@ -296,7 +296,8 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
         }
         // The first tile's ids are requested only now: the few activation requests above must not queue up behind
         // the flood of id requests of the whole chip (measured: asking for the ids first costs about a microsecond).
-        if (n_mine > 0) info = issue_tile(0, wlo, whi);
+        // Later panels' first ids are in flight already (requested at the end of the panel before).
+        if (n_mine > 0 && first_panel) info = issue_tile(0, step0, wlo, whi);
 
         for (int tk = 0; tk < n_mine; ++tk) {
             v4f_t acc[NT], acc_top[NT];
@@ -345,8 +346,10 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) acc[nt] = F::mfma(xa[nt][it][j], b[j], acc[nt]);
             }
-            // the next tile's ids are requested before this tile's sums are put away
-            if (tk + 1 < n_mine) info = issue_tile(tk + 1, wlo, whi);
+            // the next tile's ids (after the last tile: the next panel's first) are requested before this tile's sums
+            // are put away
+            if (tk + 1 < n_mine) info = issue_tile(tk + 1, step0, wlo, whi);
+            else if (more) info = issue_tile(0, step0_next, wlo, whi);
 
             // ---- tile done for this wave: remove the bias, store into the wave's own LDS slots ----
             const int lt = g + a.G * tk;                                // the workgroup's local tile
