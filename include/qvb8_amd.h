@@ -126,6 +126,33 @@ int qvb8_mma(const void* X, int x_dtype, int64_t M,
              const int32_t* perm, const uint64_t* rowinfo, int flags, float* Y,
              void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- routed MoE expert stack (decode: a few tokens, top-k experts each) ---------------------------------------- */
+
+enum qvb8_moe_act {
+    QVB8_MOE_SILU_GATED = 0,  /* up rows = gate (first half) then up: H[i] = silu(Y[i]) * Y[I + i], Q_up == 2 * P_dn */
+    QVB8_MOE_RELU2 = 1        /* non-gated: H[i] = max(Y[i], 0)^2, Q_up == P_dn */
+};
+
+/* Bytes of workspace qvb8_moe_experts needs (routing plan + fp32 H (pairs, P_dn) + fp32 Yd (pairs, Q_dn)). */
+int64_t qvb8_moe_workspace_bytes(int64_t tokens, int64_t topk, int64_t n_experts, int64_t Q_up, int64_t P_dn, int64_t Q_dn);
+
+/* out[t] = sum_j w[t][j] * W_dn[e] . act(W_up[e] . sat_half(X[t])),  e = idx[t][j]; out is (tokens, Q_dn) in out_dtype.
+ * Stacked layout of the reference (QVBandExpertsV8.build_stack, formats/qvb8/backends_experts.py:145-195): per
+ * projection ONE ids buffer (16-byte aligned, every expert's ids concatenated) and (n_experts, Q) row metadata with
+ * bit offsets made global; experts carry no escapes.  idx i64 (tokens, topk), w f32 (tokens, topk), X (tokens, P_up)
+ * in x_dtype; P_up and P_dn multiples of 32; Q_dn == P_up.  An expert selected by several tokens is read once for up
+ * to 8 of them.  An index outside 0..n_experts-1 turns the whole output into NaN.  Four launches, no host round trip.
+ * Replaces: ext.moe_experts  qvb8_moe_experts_forward qvb8_cuda.cu:937-992 (kernels qvb8_moe_gemv :860-907,
+ * qvb8_moe_act :910-918, qvb8_moe_combine :924-935) with act QVB8_MOE_SILU_GATED, and ext.moe_experts_relu2
+ * qvb8_moe_experts_relu2_forward :1002-1055 with QVB8_MOE_RELU2. */
+int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, const int64_t* idx, const float* w, int64_t topk,
+                     int64_t n_experts,
+                     const uint8_t* up_ids, int64_t up_ids_bytes, const float* up_min, const float* up_tau,
+                     const uint8_t* up_nb, const int64_t* up_off, int64_t Q_up, int64_t P_up,
+                     const uint8_t* dn_ids, int64_t dn_ids_bytes, const float* dn_min, const float* dn_tau,
+                     const uint8_t* dn_nb, const int64_t* dn_off, int64_t Q_dn, int64_t P_dn,
+                     int act, void* out, int out_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -17,7 +17,8 @@ _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 # every symbol include/qvb8_amd.h declares
 SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_scatter_escapes", "qvb8_certify",
-           "qvb8_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma")
+           "qvb8_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma",
+           "qvb8_moe_workspace_bytes", "qvb8_moe_experts")
 
 
 def lib_path() -> str:
@@ -61,6 +62,10 @@ def load(build_if_missing: bool = True):
     lib.qvb8_mma_rowinfo_bytes.restype = i64
     lib.qvb8_mma_prepare.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, vp]
     lib.qvb8_mma.argtypes = [vp, i32, i64, vp, i64, vp, vp, vp, vp, i64, i64, vp, vp, i64, vp, vp, i32, vp, vp, i64, vp]
+    lib.qvb8_moe_workspace_bytes.argtypes = [i64] * 6
+    lib.qvb8_moe_workspace_bytes.restype = i64
+    lib.qvb8_moe_experts.argtypes = ([vp, i32, i64, vp, vp, i64, i64] + [vp, i64, vp, vp, vp, vp, i64, i64] * 2
+                                     + [i32, vp, i32, vp, i64, vp])
     for name in SYMBOLS:
         getattr(lib, name)                           # every declared symbol must be exported
     _LIB = lib

@@ -1,0 +1,389 @@
+// Routed MoE expert stack on packed QVB8 experts (decode: a few tokens, top-k experts each), gfx950.
+//
+//   pair p = (token t, j-th choice), expert e = idx[t][j]
+//   gated (act 0):   Y = W_gu[e] . x_t ;  H[p][i] = silu(Y[i]) * Y[I + i]      (gate = first half of the rows)
+//   relu2 (act 1):   Y = W_up[e] . x_t ;  H[p][i] = max(Y[i], 0)^2
+//   Yd[p] = W_dn[e] . H[p] ;  out[t] = sum_j w[t][j] * Yd[t * k + j]           (j ascending, fused multiply-add)
+//
+// Three steps on the caller's stream: a one-workgroup routing plan (pairs grouped by expert, no host round trip), the
+// up projection with the activation fused into its epilogue, the down projection, and the weighted combine.  The
+// grouped products run over the experts that were actually selected, and an expert chosen by several tokens is read
+// ONCE for all of them (up to 8 pairs share every decoded id): the bytes touched are those of the unique experts.
+//
+// Arithmetic: x is narrowed like saturating_half and widened again (what the reference multiplies), H stays fp32.
+// A row's product is  tau_s * sum(x * id) + min_s * sum(x)  with fp32 fused multiply-adds per lane, a fixed-order wave
+// sum, and the two terms joined in double: reproducible, and within rounding of  sum(x * fmaf(id, tau_s, min_s)).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <type_traits>
+
+#include "../../include/qvb8_amd.h"
+#include "qvb8_device.h"
+#include "qvb8_host.h"
+
+namespace qvb8 {
+
+constexpr int kMoeMB = 8;              // pairs that share one pass over an expert's rows
+constexpr int kMoeThreads = 256;
+
+// Workspace layout (bytes from the start): plan | H | Yd
+//   plan: i32 n_bad (+3 pad), int4 slot[n_slots] = {expert, first pair, end pair, 0} for the experts that have pairs
+//   (end == first for unused slots), i32 order[npairs] (pair numbers grouped by expert)
+struct MoePlan {
+    int32_t* n_bad; int4* slot; int32_t* order;
+};
+__host__ __device__ inline int64_t moe_slots(int64_t E, int64_t npairs) { return E < npairs ? E : npairs; }
+__host__ __device__ inline size_t moe_plan_bytes(int64_t E, int64_t npairs) {
+    return (size_t)(16 + moe_slots(E, npairs) * 16 + npairs * 4 + 255) & ~(size_t)255;
+}
+__host__ __device__ inline MoePlan moe_plan_at(void* ws, int64_t E, int64_t npairs) {
+    unsigned char* p = reinterpret_cast<unsigned char*>(ws);
+    return MoePlan{reinterpret_cast<int32_t*>(p), reinterpret_cast<int4*>(p + 16),
+                   reinterpret_cast<int32_t*>(p + 16 + moe_slots(E, npairs) * 16)};
+}
+
+// One workgroup: pairs grouped by expert (counting sort), list of the experts that have pairs.
+__global__ void __launch_bounds__(kMoeThreads) moe_plan_kernel(const int64_t* __restrict__ idx, int npairs, int E, MoePlan pl) {
+    extern __shared__ int32_t s_cnt[];                        // [E] counts, then cursors
+    for (int e = threadIdx.x; e < E; e += blockDim.x) s_cnt[e] = 0;
+    if (threadIdx.x == 0) { *pl.n_bad = 0; }
+    __syncthreads();
+    int bad = 0;
+    for (int p = threadIdx.x; p < npairs; p += blockDim.x) {
+        const int64_t e = idx[p];
+        if (e >= 0 && e < E) atomicAdd(&s_cnt[(int)e], 1); else ++bad;
+    }
+    if (bad) atomicAdd(pl.n_bad, bad);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0, na = 0;
+        const int n_slots = E < npairs ? E : npairs;
+        for (int e = 0; e < E; ++e) {
+            const int c = s_cnt[e];
+            if (c > 0) pl.slot[na++] = int4{e, run, run + c, 0};
+            s_cnt[e] = run;                                    // becomes the expert's cursor
+            run += c;
+        }
+        for (; na < n_slots; ++na) pl.slot[na] = int4{0, 0, 0, 0};
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < npairs; p += blockDim.x) {
+        const int64_t e = idx[p];
+        if (e >= 0 && e < E) pl.order[atomicAdd(&s_cnt[(int)e], 1)] = p;
+    }
+}
+
+struct MoeGemvArgs {
+    const void* X;                 // stage 0: (tokens, P) activations in x_dtype; stage 1: H (npairs, P) f32
+    const uint8_t* ids; int64_t ids_bytes;
+    const float* min_s; const float* tau_s; const uint8_t* nbits; const int64_t* bit_off;   // (E, Q) each
+    float* out;                    // stage 0: H (npairs, n_units); stage 1: Yd (npairs, Q)
+    MoePlan plan;
+    int Q, P, topk, x_dtype, act;  // act: 0 gated silu, 1 relu2 (stage 0 only)
+    int units;                     // output columns per pair: stage 0 gated Q/2, relu2 Q; stage 1 Q
+    int units_per_block;
+    int x_rows;                    // activation rows a workgroup stages at a time: min(kMoeMB, tokens)
+};
+
+template <int NB, int J>
+__device__ __forceinline__ void moe_fields(const uint32_t (&w)[kMaxFastNb], float (&idf)[32]) {
+    if constexpr (J < 32) { idf[J] = (float)field_of<NB, J>(w); moe_fields<NB, J + 1>(w, idf); }
+}
+
+// acc[mb] += x[mb][c0 + j] * id_j over the lane's 32 consecutive ids, given as the first and the last four dwords of
+// its NB-dword slice
+template <int NB, typename XT>
+__device__ __forceinline__ void moe_chunk(const uint4& lo, const uint4& hi, const XT* __restrict__ xs, int P, int c0, int n,
+                                          float (&acc)[kMoeMB]) {
+    uint32_t w[kMaxFastNb];
+    const uint32_t l[4] = {lo.x, lo.y, lo.z, lo.w}, h[4] = {hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) w[k] = l[k];
+#pragma unroll
+    for (int k = 4; k < NB; ++k) w[k] = h[k - (NB - 4)];
+    float idf[32];
+    moe_fields<NB, 0>(w, idf);
+#pragma unroll
+    for (int mb = 0; mb < kMoeMB; ++mb) {
+        if (mb >= n) break;                                             // wave-uniform
+        float a = acc[mb];
+        if constexpr (sizeof(XT) == 4) {
+            const float4* xp = reinterpret_cast<const float4*>(xs + (size_t)mb * P + c0);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float4 xv = xp[k];
+                a = __builtin_fmaf(xv.x, idf[4 * k + 0], a);
+                a = __builtin_fmaf(xv.y, idf[4 * k + 1], a);
+                a = __builtin_fmaf(xv.z, idf[4 * k + 2], a);
+                a = __builtin_fmaf(xv.w, idf[4 * k + 3], a);
+            }
+        } else {
+            typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+            const v8h* xp = reinterpret_cast<const v8h*>(xs + (size_t)mb * P + c0);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const v8h xv = xp[k];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) a = __builtin_fmaf((float)xv[j], idf[8 * k + j], a);
+            }
+        }
+        acc[mb] = a;
+    }
+}
+
+template <typename XT>
+__device__ __forceinline__ void moe_chunk_any(int nb, const uint4& lo, const uint4& hi, const XT* xs, int P, int c0, int n,
+                                              float (&acc)[kMoeMB]) {
+    switch (nb) {
+        case 4: moe_chunk<4>(lo, hi, xs, P, c0, n, acc); break;
+        case 5: moe_chunk<5>(lo, hi, xs, P, c0, n, acc); break;
+        case 6: moe_chunk<6>(lo, hi, xs, P, c0, n, acc); break;
+        case 7: moe_chunk<7>(lo, hi, xs, P, c0, n, acc); break;
+        default: moe_chunk<8>(lo, hi, xs, P, c0, n, acc); break;
+    }
+}
+
+// Row record a workgroup keeps in LDS for each of its rows: flags = width | ok << 8 | fast << 9
+struct MoeRow { int64_t bit0; float ts, mn; int flags; int pad; };
+
+// STAGE 0: up projection + activation -> H.  STAGE 1: down projection -> Yd.
+// grid = (unit blocks, expert slots); a workgroup serves `units_per_block` output units of one selected expert for
+// all pairs routed to it, kMoeMB pairs at a time, with those pairs' activation rows staged in LDS as fp32.  A wave
+// walks through its rows with the next row's ids already requested while it multiplies the current one.
+template <int STAGE>
+__global__ void __launch_bounds__(kMoeThreads) moe_gemv_kernel(MoeGemvArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int rpu = (STAGE == 0 && a.act == 0) ? 2 : 1;             // rows per output unit (gate and up)
+    // stage 0 multiplies activations that were narrowed to fp16: they are kept as fp16 (half the LDS and LDS traffic)
+    using XT = std::conditional_t<STAGE == 0, _Float16, float>;
+    XT* xs = reinterpret_cast<XT*>(smem);                           // [x_rows][P]
+    float* sxs = reinterpret_cast<float*>(smem + (((size_t)a.x_rows * a.P * sizeof(XT) + 15) & ~(size_t)15));   // [kMoeMB] sums of the staged rows
+    float* red = sxs + kMoeMB;                                      // [kMoeMB][waves]
+    MoeRow* s_row = reinterpret_cast<MoeRow*>(red + kMoeMB * (kMoeThreads / 64));   // [units_per_block * rpu]
+    const int4 slot = a.plan.slot[blockIdx.y];
+    const int e = slot.x, p_begin = slot.y, p_end = slot.z;
+    if (p_begin >= p_end) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
+    const int u_begin = blockIdx.x * a.units_per_block, u_end = min(a.units, u_begin + a.units_per_block);
+    const int gate_rows = a.Q / 2;
+    const int n_rows_blk = (u_end - u_begin) * rpu;
+    // local row lr -> row of the expert: unit u_begin + lr / rpu; in gated mode the even local rows are gate rows (u),
+    // the odd ones the matching up rows (Q/2 + u)
+    for (int lr = tid; lr < n_rows_blk; lr += blockDim.x) {
+        const int u = u_begin + lr / rpu;
+        const size_t mi = (size_t)e * a.Q + ((rpu == 2 && (lr & 1)) ? gate_rows + u : u);
+        const int nb = a.nbits[mi];
+        const int64_t bit0 = a.bit_off[mi];
+        const bool ok = nb >= 1 && nb <= 14 && bit0 >= 0 && ((bit0 + (int64_t)nb * a.P + 7) >> 3) + 8 <= a.ids_bytes;
+        const bool fast = ok && nb >= 4 && nb <= 8 && (bit0 & 31) == 0;
+        s_row[lr] = MoeRow{ok ? bit0 : 0, a.tau_s[mi], a.min_s[mi], nb | (ok ? 256 : 0) | (fast ? 512 : 0), 0};
+    }
+    const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
+    const int n_items = ((u_end - u_begin - wave + n_waves - 1) / n_waves) * rpu;   // rows this wave walks through
+    auto local_row = [&](int i) { return ((wave + (i / rpu) * n_waves) * rpu) + (i % rpu); };
+    // the lane's slice of the first 2048 columns of a row (fast rows; other lanes / rows read the buffer's first bytes)
+    auto request = [&](const MoeRow& r, uint4& lo, uint4& hi) {
+        const int nb = r.flags & 255;
+        const bool use = (r.flags & 512) && lane * 32 < a.P;
+        const uint8_t* p = a.ids + (use ? (r.bit0 >> 3) + (int64_t)lane * 4 * nb : 0);
+        lo = *reinterpret_cast<const uint4*>(p);
+        hi = *reinterpret_cast<const uint4*>(p + (use ? 4 * (nb - 4) : 16));
+    };
+
+    for (int pc = p_begin; pc < p_end; pc += a.x_rows) {
+        const int n = min(a.x_rows, p_end - pc);                    // x_rows <= kMoeMB
+        __syncthreads();                                            // the previous chunk's rows are no longer read; s_row is written
+        uint4 lo, hi;
+        MoeRow cur;
+        if (n_items > 0) { cur = s_row[local_row(0)]; request(cur, lo, hi); }
+        // ---- stage the chunk's activation rows and their sums ----
+        for (int mb = 0; mb < n; ++mb) {
+            const int p = a.plan.order[pc + mb];
+            float part = 0.f;
+            for (int c = tid; c < a.P; c += blockDim.x) {
+                float v;
+                if constexpr (STAGE == 0) {
+                    const uint32_t hb = sat_half_bits(load_as_f32(a.X, (int64_t)(p / a.topk) * a.P + c, a.x_dtype));
+                    v = f16_bits_to_f32(hb);
+                    xs[(size_t)mb * a.P + c] = __builtin_bit_cast(XT, (uint16_t)hb);
+                } else {
+                    v = reinterpret_cast<const float*>(a.X)[(size_t)p * a.P + c];
+                    xs[(size_t)mb * a.P + c] = v;
+                }
+                part += v;
+            }
+            part = wave_sum(part);
+            if (lane == 0) red[mb * n_waves + wave] = part;
+        }
+        __syncthreads();
+        if (tid < n) {
+            float s = 0.f;
+            for (int w = 0; w < n_waves; ++w) s += red[tid * n_waves + w];
+            sxs[tid] = s;
+        }
+        __syncthreads();
+        // ---- rows: the next row's slice is requested before the current one is multiplied ----
+        float y_gate[kMoeMB];
+#pragma unroll
+        for (int mb = 0; mb < kMoeMB; ++mb) y_gate[mb] = 0.f;
+        for (int i = 0; i < n_items; ++i) {
+            uint4 lo_n = lo, hi_n = hi;
+            MoeRow nxt = cur;
+            if (i + 1 < n_items) { nxt = s_row[local_row(i + 1)]; request(nxt, lo_n, hi_n); }
+            const int nb = cur.flags & 255;
+            float acc[kMoeMB];
+#pragma unroll
+            for (int mb = 0; mb < kMoeMB; ++mb) acc[mb] = 0.f;
+            if (cur.flags & 512) {
+                if (lane * 32 < a.P) moe_chunk_any(nb, lo, hi, xs, a.P, lane * 32, n, acc);
+                for (int c0 = (kWave + lane) * 32; c0 < a.P; c0 += kWave * 32) {          // rows longer than 2048 columns
+                    const uint8_t* p = a.ids + (cur.bit0 >> 3) + (int64_t)(c0 >> 5) * 4 * nb;
+                    moe_chunk_any(nb, *reinterpret_cast<const uint4*>(p), *reinterpret_cast<const uint4*>(p + 4 * (nb - 4)), xs, a.P, c0, n, acc);
+                }
+            } else if (cur.flags & 256) {
+                for (int c = lane; c < a.P; c += kWave) {
+                    const float idf = (float)load_field(a.ids, cur.bit0 + (int64_t)c * nb, nb, clamp_byte);
+#pragma unroll
+                    for (int mb = 0; mb < kMoeMB; ++mb)
+                        if (mb < n) acc[mb] = __builtin_fmaf((float)xs[(size_t)mb * a.P + c], idf, acc[mb]);
+                }
+            }
+            float y[kMoeMB];
+#pragma unroll
+            for (int mb = 0; mb < kMoeMB; ++mb) {
+                y[mb] = 0.f;
+                if (mb < n) {                                                            // wave-uniform
+                    const float sum = wave_sum(acc[mb]);
+                    y[mb] = (cur.flags & 256) ? (float)((double)cur.ts * (double)sum + (double)cur.mn * (double)sxs[mb]) : __builtin_nanf("");
+                }
+            }
+            const bool unit_done = (i % rpu) == rpu - 1;
+            if (unit_done) {
+                const int u = u_begin + wave + (i / rpu) * n_waves;
+                if (lane < n) {
+                    float v = 0.f;
+#pragma unroll
+                    for (int mb = 0; mb < kMoeMB; ++mb) {           // lane mb takes result mb (no dynamic register index)
+                        if (lane == mb) {
+                            if constexpr (STAGE == 0) {
+                                if (a.act == 0) v = (y_gate[mb] / (1.0f + __expf(-y_gate[mb]))) * y[mb];
+                                else { const float r = fmaxf(y[mb], 0.f); v = r * r; }
+                            } else {
+                                v = y[mb];
+                            }
+                        }
+                    }
+                    a.out[(size_t)a.plan.order[pc + lane] * a.units + u] = v;
+                }
+            } else {
+#pragma unroll
+                for (int mb = 0; mb < kMoeMB; ++mb) y_gate[mb] = y[mb];
+            }
+            cur = nxt; lo = lo_n; hi = hi_n;
+        }
+    }
+}
+
+template <int DT>
+__global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restrict__ Yd, const float* __restrict__ w, void* __restrict__ out,
+                                                          int topk, int D, int tokens, const int32_t* __restrict__ n_bad) {
+    const int t = blockIdx.y;
+    const int d = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= tokens || d >= D) return;
+    float acc = 0.f;
+    for (int j = 0; j < topk; ++j) acc = __builtin_fmaf(w[t * topk + j], Yd[((size_t)t * topk + j) * D + d], acc);
+    if (*n_bad != 0) acc = __builtin_nanf("");                      // an expert index outside the stack: fail loudly
+    store_from_f32<DT>(out, (int64_t)t * D + d, acc);
+}
+
+}  // namespace qvb8
+
+using namespace qvb8;
+
+namespace {
+constexpr size_t kMoeLdsLimit = 144 * 1024;
+
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+int launch_moe_gemv(int stage, MoeGemvArgs a, int64_t slots, hipStream_t s) {
+    // enough workgroups to fill the chip four times over the selected experts, at least one unit per wave
+    const int waves = kMoeThreads / 64;
+    const int64_t target_blocks = ((int64_t)host::env_int("QVB8_MOE_WGS_PER_CU", 4) * host::device_cus() + slots - 1) / slots;
+    int64_t upb = (a.units + target_blocks - 1) / target_blocks;
+    upb = (upb + waves - 1) / waves * waves;
+    a.units_per_block = (int)upb;
+    const size_t lds = (((size_t)a.x_rows * a.P * (stage == 0 ? 2 : 4) + 15) & ~(size_t)15) + (kMoeMB + kMoeMB * (kMoeThreads / 64)) * 4
+                       + (size_t)upb * 2 * sizeof(MoeRow);
+    if (lds > kMoeLdsLimit) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_moe_experts: P=%d does not fit the workgroup's LDS", a.P);
+    static bool attr[2][64] = {{false}};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_moe_experts: no current device");
+    if (!attr[stage][dev]) {
+        const void* f = stage == 0 ? (const void*)moe_gemv_kernel<0> : (const void*)moe_gemv_kernel<1>;
+        if (hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMoeLdsLimit) != hipSuccess)
+            return host::fail(QVB8_ERR_LAUNCH, "qvb8_moe_experts: cannot raise the kernel's LDS limit");
+        attr[stage][dev] = true;
+    }
+    dim3 grid((unsigned)((a.units + upb - 1) / upb), (unsigned)slots);
+    if (stage == 0) hipLaunchKernelGGL(moe_gemv_kernel<0>, grid, dim3(kMoeThreads), lds, s, a);
+    else hipLaunchKernelGGL(moe_gemv_kernel<1>, grid, dim3(kMoeThreads), lds, s, a);
+    return host::check_launch("qvb8_moe_experts");
+}
+}  // namespace
+
+extern "C" int64_t qvb8_moe_workspace_bytes(int64_t tokens, int64_t topk, int64_t n_experts, int64_t Q_up, int64_t P_dn, int64_t Q_dn) {
+    (void)Q_up;
+    if (tokens <= 0 || topk <= 0 || n_experts <= 0 || P_dn <= 0 || Q_dn <= 0) return 0;
+    const int64_t np = tokens * topk;
+    return (int64_t)(moe_plan_bytes(n_experts, np) + align256((size_t)np * P_dn * 4) + align256((size_t)np * Q_dn * 4));
+}
+
+extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, const int64_t* idx, const float* w, int64_t topk, int64_t n_experts,
+                                const uint8_t* up_ids, int64_t up_ids_bytes, const float* up_min, const float* up_tau,
+                                const uint8_t* up_nb, const int64_t* up_off, int64_t Q_up, int64_t P_up,
+                                const uint8_t* dn_ids, int64_t dn_ids_bytes, const float* dn_min, const float* dn_tau,
+                                const uint8_t* dn_nb, const int64_t* dn_off, int64_t Q_dn, int64_t P_dn,
+                                int act, void* out, int out_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+    if (tokens < 0 || topk < 1 || n_experts < 1 || n_experts > 8192) return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: bad token / top-k / expert count");
+    if (act != 0 && act != 1) return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: act must be 0 (gated SiLU) or 1 (ReLU squared)");
+    if (Q_up <= 0 || P_up <= 0 || Q_dn <= 0 || P_dn <= 0 || Q_up > 0x7fffffff || P_up > 0x7fffffff || Q_dn > 0x7fffffff || P_dn > 0x7fffffff)
+        return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: bad shape");
+    if (act == 0 ? (Q_up % 2 != 0 || Q_up / 2 != P_dn) : (Q_up != P_dn)) return host::fail(QVB8_ERR_ARG, "moe: gate_up/down shapes disagree");
+    if (Q_dn != P_up) return host::fail(QVB8_ERR_ARG, "moe: down must map back to the hidden size");
+    if (P_up % 32 != 0 || P_dn % 32 != 0) return host::fail(QVB8_ERR_UNSUPPORTED, "moe: P must be a multiple of 32");
+    if (x_dtype < QVB8_F32 || x_dtype > QVB8_BF16 || out_dtype < QVB8_F32 || out_dtype > QVB8_BF16) return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: bad dtype");
+    if (tokens == 0) return QVB8_OK;
+    if (tokens * topk > 0x7fffffff / 4) return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: too many pairs");
+    if (!X || !idx || !w || !up_ids || !up_min || !up_tau || !up_nb || !up_off || !dn_ids || !dn_min || !dn_tau || !dn_nb || !dn_off || !out)
+        return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: null pointer");
+    if ((reinterpret_cast<uintptr_t>(up_ids) & 15u) || (reinterpret_cast<uintptr_t>(dn_ids) & 15u)) return host::fail(QVB8_ERR_ARG, "moe: ids must be 16-byte aligned");
+    if (up_ids_bytes < 32 || dn_ids_bytes < 32) return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: ids buffer shorter than 32 bytes");
+    const int64_t need = qvb8_moe_workspace_bytes(tokens, topk, n_experts, Q_up, P_dn, Q_dn);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u))
+        return host::fail(QVB8_ERR_WORKSPACE, "qvb8_moe_experts: needs %lld bytes of 16-byte aligned workspace", (long long)need);
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t np = tokens * topk;
+    unsigned char* ws = (unsigned char*)workspace;
+    MoePlan pl = moe_plan_at(ws, n_experts, np);
+    float* H = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np));
+    float* Yd = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np) + align256((size_t)np * P_dn * 4));
+
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)n_experts * 4, s, idx, (int)np, (int)n_experts, pl);
+    if (int rc = host::check_launch("qvb8_moe_experts plan")) return rc;
+    const int64_t slots = moe_slots(n_experts, np);
+
+    MoeGemvArgs a;
+    a.X = X; a.ids = up_ids; a.ids_bytes = up_ids_bytes; a.min_s = up_min; a.tau_s = up_tau; a.nbits = up_nb; a.bit_off = up_off;
+    a.out = H; a.plan = pl; a.Q = (int)Q_up; a.P = (int)P_up; a.topk = (int)topk; a.x_dtype = x_dtype; a.act = act;
+    a.units = (int)P_dn; a.units_per_block = 0; a.x_rows = (int)(tokens < kMoeMB ? tokens : kMoeMB);
+    if (int rc = launch_moe_gemv(0, a, slots, s)) return rc;
+    a.X = H; a.ids = dn_ids; a.ids_bytes = dn_ids_bytes; a.min_s = dn_min; a.tau_s = dn_tau; a.nbits = dn_nb; a.bit_off = dn_off;
+    a.out = Yd; a.Q = (int)Q_dn; a.P = (int)P_dn; a.x_dtype = QVB8_F32; a.units = (int)Q_dn;
+    if (int rc = launch_moe_gemv(1, a, slots, s)) return rc;
+
+    dim3 grid((unsigned)((Q_dn + 255) / 256), (unsigned)tokens);
+    if (out_dtype == QVB8_F32) hipLaunchKernelGGL(moe_combine_kernel<0>, grid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
+    else if (out_dtype == QVB8_F16) hipLaunchKernelGGL(moe_combine_kernel<1>, grid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
+    else hipLaunchKernelGGL(moe_combine_kernel<2>, grid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
+    return host::check_launch("qvb8_moe_experts combine");
+}

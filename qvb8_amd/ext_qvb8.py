@@ -249,3 +249,49 @@ def forward(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
 def forward_half(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
     """As forward, but the M > 8 GEMM stores fp16."""
     return _forward(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, True)
+
+
+def _moe(act, X, idx, w, up_ids, up_min, up_tau, up_nb, up_off, Qup, Pup, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn):
+    lib = _lib.load()
+    _lib.require_cuda(X, idx, w, up_ids, up_min, up_tau, up_nb, up_off, dn_ids, dn_min, dn_tau, dn_nb, dn_off)
+    if X.dim() != 2 or X.shape[1] != int(Pup):
+        raise RuntimeError("moe: bad X")
+    if idx.dtype != torch.int64 or w.dtype != torch.float32 or idx.dim() != 2 or tuple(w.shape) != tuple(idx.shape):
+        raise RuntimeError("moe: idx must be int64 and w float32, both (tokens, topk)")
+    if idx.shape[0] != X.shape[0]:
+        raise RuntimeError("moe: one routing row per token")
+    if up_min.dim() != 2 or up_min.shape[1] != int(Qup) or dn_min.dim() != 2 or dn_min.shape[1] != int(Qdn) \
+            or dn_min.shape[0] != up_min.shape[0]:
+        raise RuntimeError("moe: row metadata must be (experts, Q)")
+    for t, dt in ((up_ids, torch.uint8), (up_nb, torch.uint8), (up_off, torch.int64), (up_min, torch.float32),
+                  (up_tau, torch.float32), (dn_ids, torch.uint8), (dn_nb, torch.uint8), (dn_off, torch.int64),
+                  (dn_min, torch.float32), (dn_tau, torch.float32)):
+        if t.dtype != dt:
+            raise RuntimeError(f"moe: expected {dt}, got {t.dtype}")
+    T, k, E = X.shape[0], idx.shape[1], up_min.shape[0]
+    Xc, idxc, wc = X.contiguous(), idx.contiguous(), w.contiguous()
+    tens = [t.contiguous() for t in (up_ids, up_min, up_tau, up_nb, up_off, dn_ids, dn_min, dn_tau, dn_nb, dn_off)]
+    with torch.cuda.device(Xc.device):
+        out = torch.empty((T, int(Qdn)), dtype=Xc.dtype, device=Xc.device)
+        if T == 0:
+            return out
+        nws = lib.qvb8_moe_workspace_bytes(T, k, E, int(Qup), int(Pdn), int(Qdn))
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=Xc.device)
+        u, d = tens[:5], tens[5:]
+        _lib._check(lib.qvb8_moe_experts(
+            _lib.ptr(Xc), _lib.dtype_code(Xc.dtype), T, _lib.ptr(idxc), _lib.ptr(wc), k, E,
+            _lib.ptr(u[0]), u[0].numel(), _lib.ptr(u[1]), _lib.ptr(u[2]), _lib.ptr(u[3]), _lib.ptr(u[4]), int(Qup), int(Pup),
+            _lib.ptr(d[0]), d[0].numel(), _lib.ptr(d[1]), _lib.ptr(d[2]), _lib.ptr(d[3]), _lib.ptr(d[4]), int(Qdn), int(Pdn),
+            act, _lib.ptr(out), _lib.dtype_code(out.dtype), _lib.ptr(ws), ws.numel(), _lib.stream_of(Xc)), lib)
+    return out
+
+
+def moe_experts(X, idx, w, gu_ids, gu_min, gu_tau, gu_nb, gu_off, Qgu, Pgu, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn):
+    """Routed gated-SiLU expert stack on the stacked layout (reference: qvb8_cuda.cu:937-992); returns (tokens, Qdn)
+    in X's dtype."""
+    return _moe(0, X, idx, w, gu_ids, gu_min, gu_tau, gu_nb, gu_off, Qgu, Pgu, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn)
+
+
+def moe_experts_relu2(X, idx, w, up_ids, up_min, up_tau, up_nb, up_off, Qup, Pup, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn):
+    """Non-gated expert stack with H = relu(up(x))^2 (reference: qvb8_cuda.cu:1002-1055)."""
+    return _moe(1, X, idx, w, up_ids, up_min, up_tau, up_nb, up_off, Qup, Pup, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn)

@@ -1,0 +1,129 @@
+"""GPU parity of the routed MoE expert stack (qvb8_moe_experts through ext.moe_experts / QVBandExpertsV8) against the
+CPU oracle's per-token loop over restored weights."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import qvb8_oracle as O
+from qvb8_amd import ext_qvb8 as ext
+from qvb8_amd.formats.qvb8 import pack as PK
+from qvb8_amd.formats.qvb8.backends_experts import QVBandExpertsV8
+from qvb8_amd.formats.qvb8.module import QVBandLinearV8
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _experts(E, hidden, inter, tau, seed, gated=True):
+    gu, dn, Wgu, Wdn = [], [], [], []
+    for e in range(E):
+        for lst, Wl, (Q, P) in ((gu, Wgu, ((2 if gated else 1) * inter, hidden)), (dn, Wdn, (hidden, inter))):
+            W = H.synth_weight(Q, P, seed=seed + 2 * e + len(lst)).to(DEV)
+            enc = PK.encode_tensor(W, tau, restore="fp16")
+            assert enc["esc_idx"].numel() == 0
+            lst.append(QVBandLinearV8.from_encoded(enc))
+            d = H.oracle_view(enc)
+            Wl.append(O.reconstruct(d["min_s"], d["tau_s"], H.oracle_ids(d), d["esc_idx"], d["esc_vals"]))
+    return gu, dn, Wgu, Wdn
+
+
+def _route(T, E, k, seed):
+    rng = np.random.default_rng(seed)
+    idx, w = O.router_topk(rng.normal(size=(T, E)), k)
+    return idx, w
+
+
+def _check(out, ref, out_dtype, roundings=1):
+    """`roundings`: how many times intermediate results pass through out_dtype (the per-expert loop rounds the up
+    output, the activation product, the down output and the weighted sum)."""
+    eps = {torch.float32: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[out_dtype] * roundings
+    got = out.float().cpu().numpy().astype(np.float64)
+    scale = np.sqrt(np.mean(ref ** 2)) + 1e-30
+    tol = (1e-3 + eps) * np.abs(ref) + (2e-3 + eps * (roundings > 1)) * scale
+    diff = np.abs(got - ref)
+    assert np.all(diff <= tol), (float(diff.max()), float((diff / tol).max()))
+
+
+@pytest.mark.parametrize("T,k,dtype", [(1, 2, torch.bfloat16), (3, 4, torch.float16), (8, 2, torch.float32), (20, 3, torch.bfloat16)])
+def test_moe_small_stack(T, k, dtype):
+    E, hidden, inter = 8, 256, 96
+    gu, dn, Wgu, Wdn = _experts(E, hidden, inter, 2e-3, seed=100)
+    idx, w = _route(T, E, k, seed=T)
+    x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(dtype)
+    mod = QVBandExpertsV8(gu, dn, num_experts=E)
+    out = mod(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
+    assert mod._stk not in (None, False) and out.dtype == dtype and out.shape == (T, hidden)
+    ref = O.moe_reference(x.float().numpy(), idx, w, Wgu, Wdn)
+    _check(out, ref, dtype)
+    # the per-expert loop over the same (now stacked) modules agrees
+    loop = mod._forward_loop(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV).to(dtype))
+    _check(loop, ref, dtype if dtype != torch.float32 else torch.float16, roundings=4)
+    # an expert index outside the stack poisons the output instead of reading somewhere else
+    bad = torch.from_numpy(idx).to(DEV).clone()
+    bad[0, 0] = E
+    assert torch.isnan(mod(x.to(DEV), bad, torch.from_numpy(w).to(DEV)).float()).all()
+
+
+def test_moe_config4_shape():
+    """Qwen-35B-A3B-shape layer, fewer experts resident: hidden 2048, gate/up 2048->768, top-8, 1 and 8 tokens."""
+    E, hidden, inter = 16, 2048, 768
+    gu, dn, Wgu, Wdn = _experts(E, hidden, inter, 2e-3, seed=500)
+    mod = QVBandExpertsV8(gu, dn, num_experts=E)
+    for T in (1, 8):
+        idx, w = _route(T, E, 8, seed=10 + T)
+        x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(torch.bfloat16)
+        out = mod(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
+        _check(out, O.moe_reference(x.float().numpy(), idx, w, Wgu, Wdn), torch.bfloat16)
+        again = mod(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
+        assert torch.equal(out, again)                       # reproducible run to run
+
+
+def test_moe_relu2_and_odd_widths():
+    """Non-gated ReLU^2 stack on hand-made packs whose rows use every width 1..14 (the per-element path included)."""
+    E, hidden, inter = 3, 128, 64
+    ups, dns, Wup, Wdn = [], [], [], []
+    for e in range(E):
+        for lst, Wl, (Q, P), widths in ((ups, Wup, (inter, hidden), list(range(1, 15))), (dns, Wdn, (hidden, inter), [4, 5, 6, 7, 8])):
+            d = H.mixed_width_pack(Q, P, widths, seed=7 * e + len(lst))
+            d["tau_s"] = d["tau_s"] * (1.0 / (1 << 6))            # keep products of wide rows in range
+            a = H.to_device_args(d, DEV)
+            lst.append(dict(ids=a[0], min_s=a[1], nbits=a[2], bit_off=a[3], tau_s=a[5]))
+            Wl.append(O.reconstruct(d["min_s"], d["tau_s"], d["ids_dense"], d["esc_idx"], d["esc_vals"]))
+
+    def stack(lst):
+        offs, total = [], 0
+        for t in lst:
+            offs.append(total)
+            total += (t["ids"].numel() + 15) // 16 * 16
+        ids = torch.zeros(total + 64, dtype=torch.uint8, device=DEV)
+        for o, t in zip(offs, lst):
+            ids[o:o + t["ids"].numel()] = t["ids"]
+        return (ids, torch.stack([t["min_s"] for t in lst]), torch.stack([t["tau_s"] for t in lst]),
+                torch.stack([t["nbits"] for t in lst]), torch.stack([t["bit_off"] + 8 * o for t, o in zip(lst, offs)]))
+    T, k = 5, 2
+    idx, w = _route(T, E, k, seed=3)
+    x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(1)).to(torch.float16)
+    out = ext.moe_experts_relu2(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV),
+                                *stack(ups), inter, hidden, *stack(dns), hidden, inter)
+    _check(out, O.moe_reference(x.float().numpy(), idx, w, Wup, Wdn, act="relu2"), torch.float16)
+
+
+def test_moe_refusals():
+    E, hidden, inter = 2, 128, 32
+    gu, dn, _, _ = _experts(E, hidden, inter, 2e-3, seed=900)
+    mod = QVBandExpertsV8(gu, dn, num_experts=E, act_fn=nn.GELU())
+    assert mod.build_stack() is False                        # unknown activation: the loop path serves it
+    x = torch.randn(2, hidden).to(torch.bfloat16).to(DEV)
+    idx = torch.tensor([[0, 1], [1, 0]], device=DEV)
+    w = torch.full((2, 2), 0.5, device=DEV)
+    assert mod(x, idx, w).shape == (2, hidden)
+    with pytest.raises(ValueError):
+        QVBandExpertsV8(gu[:1], dn, num_experts=E)
+    g = QVBandExpertsV8(gu, dn, num_experts=E)
+    assert g.build_stack()
+    s, d = g._stk
+    with pytest.raises(RuntimeError):                        # gate_up / down shapes disagree
+        ext.moe_experts(x, idx, w, s["ids"], s["min_s"], s["tau_s"], s["nbits"], s["bit_off"], s["Q"], s["P"],
+                        d["ids"], d["min_s"], d["tau_s"], d["nbits"], d["bit_off"], d["Q"], d["P"] + 32)
