@@ -153,6 +153,47 @@ int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, const int64_t* 
                      const uint8_t* dn_nb, const int64_t* dn_off, int64_t Q_dn, int64_t P_dn,
                      int act, void* out, int out_dtype, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- QVB8R: the same band ids, rANS-coded (32 interleaved streams per tile) ---------------------------------------- */
+
+/* What every QVB8R kernel walks ("core" of the reference: qvb8r_cuda.cu:333-344), all device pointers:
+ *   words     u32[n_words]   the streams of all tiles back to back, then >= 2048 zero words (n_words counts the pad)
+ *   tile_off  i64[n_tiles+1] first word of each tile            states  u64[n_tiles][32]  initial rANS states
+ *   tiles     i64[n_tiles][3] class, first sorted row, rows     blocks  i32[n_blocks][3]  class, first tile, tiles (<= 8)
+ *   tab       u32[n_classes][4096] slot tables: symbol | offset << 11 | (freq - 1) << 22
+ *   perm      i32[Q] sorted row -> original row                 min_s, tau_s f32[Q], drow i32[Q]  by original row
+ * id = symbol + drow[row]; value = fmaf((float)id, tau_s[row], min_s[row]).  P % 128 == 0. */
+typedef struct qvb8r_core {
+    const uint32_t* words; int64_t n_words;
+    const int64_t* tile_off; const uint64_t* states; const int64_t* tiles; int64_t n_tiles;
+    const int32_t* blocks; int64_t n_blocks;
+    const uint32_t* tab; int64_t n_classes;
+    const int32_t* perm; const float* min_s; const float* tau_s; const int32_t* drow;
+    int64_t Q, P;
+} qvb8r_core;
+
+/* Dense rows of blocks [b0, b0 + nb): out_dtype 0 fp32 / 1 fp16 / 2 bf16 values (rounded once), 3 the ids as int16.
+ * row_base < 0: a row lands at its ORIGINAL index (out is the whole (Q, P) weight); row_base >= 0: at its sorted
+ * position - row_base (a contiguous block range fills a compact chunk).  out has out_rows rows of P.  Escapes are not
+ * applied.  max_tile_rows = most rows in any tile (the file's T).  Bit-exact with the QVB8 restore of the same ids.
+ * Replaces: ext.decode  qvb8r_decode qvb8r_cuda.cu:279-306 (wrapper :398-424) and ext.ids (:426-444). */
+int qvb8r_decode(const qvb8r_core* core, int64_t max_tile_rows, int out_dtype, int64_t b0, int64_t nb, int64_t row_base,
+                 void* out, int64_t out_rows, void* stream);
+
+/* Bytes of workspace qvb8r_gemv needs (the activations transposed to (P, 1|2|4|8|16) fp32). */
+int64_t qvb8r_gemv_workspace_bytes(int64_t M, int64_t P);
+
+/* Y[m, q] = sum_c X[m, c] * value(q, c) for M = 1..16, X (M, P) in x_dtype used in fp32 as it is (no narrowing), fp32
+ * accumulate, Y f32 (M, Q) row-major, every row written.  Escapes are NOT corrected (qvb8r_fix_escapes).
+ * Replaces: ext.gemv  qvb8r_gemv qvb8r_cuda.cu:88-131, ext.multi  qvb8r_multi :153-194 and, for 9..16 rows, ext.tc
+ * qvb8r_tc :199-272 (which multiplies fp16-rounded weights; this one keeps the fp32 band value). */
+int qvb8r_gemv(const void* X, int x_dtype, int64_t M, const qvb8r_core* core, int64_t max_tile_rows, float* Y,
+               void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Y[m, uq[u]] += sum_{e in [ptr[u], ptr[u+1])} X[m, ec[e]] * ed[e]: one thread per (m, u), stored order, no atomics.
+ * Replaces: ext.fix_escapes  qvb8r_fix_escapes qvb8r_cuda.cu:311-320. */
+int qvb8r_fix_escapes(const void* X, int x_dtype, int64_t M, const int64_t* uq, const int64_t* ptr, const int64_t* ec,
+                      const float* ed, int64_t U, float* Y, int64_t Q, int64_t P, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -18,7 +18,8 @@ _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 # every symbol include/qvb8_amd.h declares
 SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_scatter_escapes", "qvb8_certify",
            "qvb8_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma",
-           "qvb8_moe_workspace_bytes", "qvb8_moe_experts")
+           "qvb8_moe_workspace_bytes", "qvb8_moe_experts",
+           "qvb8r_decode", "qvb8r_gemv_workspace_bytes", "qvb8r_gemv", "qvb8r_fix_escapes")
 
 
 def lib_path() -> str:
@@ -66,10 +67,24 @@ def load(build_if_missing: bool = True):
     lib.qvb8_moe_workspace_bytes.restype = i64
     lib.qvb8_moe_experts.argtypes = ([vp, i32, i64, vp, vp, i64, i64] + [vp, i64, vp, vp, vp, vp, i64, i64] * 2
                                      + [i32, vp, i32, vp, i64, vp])
+    lib.qvb8r_decode.argtypes = [vp, i64, i32, i64, i64, i64, vp, i64, vp]
+    lib.qvb8r_gemv_workspace_bytes.argtypes = [i64, i64]
+    lib.qvb8r_gemv_workspace_bytes.restype = i64
+    lib.qvb8r_gemv.argtypes = [vp, i32, i64, vp, i64, vp, vp, i64, vp]
+    lib.qvb8r_fix_escapes.argtypes = [vp, i32, i64, vp, vp, vp, vp, i64, vp, i64, i64, vp]
     for name in SYMBOLS:
         getattr(lib, name)                           # every declared symbol must be exported
     _LIB = lib
     return lib
+
+
+class RCore(ctypes.Structure):
+    """qvb8r_core of include/qvb8_amd.h."""
+    _fields_ = [("words", ctypes.c_void_p), ("n_words", ctypes.c_int64), ("tile_off", ctypes.c_void_p),
+                ("states", ctypes.c_void_p), ("tiles", ctypes.c_void_p), ("n_tiles", ctypes.c_int64),
+                ("blocks", ctypes.c_void_p), ("n_blocks", ctypes.c_int64), ("tab", ctypes.c_void_p),
+                ("n_classes", ctypes.c_int64), ("perm", ctypes.c_void_p), ("min_s", ctypes.c_void_p),
+                ("tau_s", ctypes.c_void_p), ("drow", ctypes.c_void_p), ("Q", ctypes.c_int64), ("P", ctypes.c_int64)]
 
 
 def _check(rc: int, lib):

@@ -85,13 +85,14 @@ def _pack_rows(ids: torch.Tensor, nb: torch.Tensor, P: int):
 
 @torch.no_grad()
 def encode_tensor(W: torch.Tensor, tau: float, *, restore: str = "fp16", source: str | None = None,
-                  max_nbits: int = L.MAX_CERTIFIED_NBITS, force_escapes=None) -> dict:
+                  max_nbits: int = L.MAX_CERTIFIED_NBITS, force_escapes=None, keep_ids: bool = False) -> dict:
     """Encode a (Q, P) weight.  Returns torch tensors on W's device:
     min_s, tau_s (f32), nbits (u8), bit_off (i64), ids (u8 payload + 8 pad bytes),
     esc_idx/esc_vals (the fp16 table: every decode that keeps fp32 or rounds to fp16),
     esc_idx_bf16/esc_vals_bf16 (all escapes: decodes that round to bf16), plus Q, P, tau,
     max_err (over both restore precisions the pack certifies), restore, source.
-    `force_escapes`: flat positions stored as escapes whatever the band says."""
+    `force_escapes`: flat positions stored as escapes whatever the band says.  `keep_ids`: also return the unpacked
+    ids as `ids_dense` (Q, P) int16 (what the entropy coder of the QVB8R format starts from)."""
     if restore not in ("fp16", "fp16+bf16"):
         raise Qvb8Error(f"restore must be 'fp16' or 'fp16+bf16', not {restore!r}")
     if W.dim() != 2:
@@ -164,7 +165,8 @@ def encode_tensor(W: torch.Tensor, tau: float, *, restore: str = "fp16", source:
         max_err = max(max_err, float(eb.max()))
     buf, bit_off = _pack_rows(ids, nb, P)
     same = esc_all.numel() == esc_16.numel()
-    return dict(Q=Q, P=P, tau=float(tau), max_err=max_err, restore=restore, source=source,
+    extra = dict(ids_dense=ids.to(torch.int16)) if keep_ids else {}
+    return dict(**extra, Q=Q, P=P, tau=float(tau), max_err=max_err, restore=restore, source=source,
                 min_s=min_s32, tau_s=ts32, nbits=nb.to(torch.uint8), bit_off=bit_off, ids=buf,
                 esc_idx=esc_16, esc_vals=vals_16,
                 esc_idx_bf16=esc_16 if same else esc_all, esc_vals_bf16=vals_16 if same else vals_all)

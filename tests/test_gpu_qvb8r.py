@@ -1,0 +1,117 @@
+"""GPU parity of the QVB8R path (walk + dense restore, fused product, escape correction, module) against the oracle:
+restored weights bit-exact with the QVB8 restore of the same ids, products within the GEMV tolerance."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import qvb8_oracle as O
+from oracle import qvb8r_oracle as R
+from qvb8_amd import ext_qvb8 as ext8
+from qvb8_amd import ext_qvb8r as ext
+from qvb8_amd.formats.qvb8 import pack as PK
+from qvb8_amd.formats.qvb8r import pack as RP
+from qvb8_amd.formats.qvb8r.module import QVBandLinearV8R
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _make(Q, P, tau, seed, restore="fp16", force=None, **kw):
+    W = H.synth_weight(Q, P, seed=seed).to(DEV)
+    enc = PK.encode_tensor(W, tau, restore=restore, force_escapes=force, keep_ids=True)
+    d = RP.transcode(enc, **kw)
+    return W, enc, d
+
+
+@pytest.mark.parametrize("Q,P,kw", [(64, 512, dict(rows_per_tile=3, n_classes=2)), (37, 128, dict(rows_per_tile=1)),
+                                     (300, 1024, dict()), (20, 5120, dict(rows_per_tile=2)), (9, 8192, dict())])
+def test_restore_bit_exact_and_ids(Q, P, kw):
+    W, enc, d = _make(Q, P, 2e-3, seed=Q + P, force=[3, P * (Q - 1) + 77], **kw)
+    lin = QVBandLinearV8R(d, device=DEV)
+    want_ids = enc["ids_dense"].cpu().numpy().astype(np.int64)
+    assert np.array_equal(R.ids(d), want_ids)                                  # the oracle's walk reads the stream back
+    got_ids = ext.ids(P, *lin._core(), T=lin.T).cpu().numpy().astype(np.int64)
+    assert np.array_equal(got_ids, want_ids)
+    v8 = H.oracle_view(enc)
+    for dt, narrow, tab in ((torch.float32, lambda a: a, False), (torch.float16, O.narrow_fp16, False), (torch.bfloat16, O.narrow_bf16, True)):
+        ei, ev = (enc["esc_idx_bf16"], enc["esc_vals_bf16"]) if tab else (enc["esc_idx"], enc["esc_vals"])
+        ref = narrow(O.reconstruct(v8["min_s"], v8["tau_s"], want_ids, ei.cpu().numpy(), ev.cpu().numpy()))
+        got = lin.dense(dt).float().cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), ref.astype(np.float32).view(np.uint32)), dt
+    # the certificate carries over: re-checked on the GPU against the original weights
+    max_err, bad = ext8.certify(lin.dense(torch.float16), W, 2e-3)
+    assert bad == 0 and max_err < 2e-3
+    # compact chunk of a block range
+    blocks = lin.blocks8.cpu().numpy()
+    if len(blocks) > 1:
+        b0, nb = 1, len(blocks) - 1
+        t0 = int(blocks[b0, 1])
+        base = int(lin.tiles[t0, 1])
+        rows = Q - base
+        Wc = ext.decode(*lin._core(), P, 2, b0, nb, base, rows, T=lin.T).cpu().numpy()
+        full = lin.dense(torch.float32).cpu().numpy()
+        band = O.reconstruct(v8["min_s"], v8["tau_s"], want_ids, np.zeros(0, np.int64), np.zeros(0, np.float32))
+        assert np.array_equal(Wc.view(np.uint32), band[d["perm"][base:base + rows]].view(np.uint32))
+        assert full.shape == (Q, P)
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 7, 8, 9, 16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_product_small_m(M, dtype):
+    Q, P = 150, 1024
+    W, enc, d = _make(Q, P, 2e-3, seed=5, force=[10, P * 149 + 1023, P * 77 + 512], rows_per_tile=3)
+    lin = QVBandLinearV8R(d, device=DEV)
+    x = torch.randn(M, P, generator=torch.Generator().manual_seed(M)).to(dtype).to(DEV)
+    x[0, 5] = 1.0e5                                                           # no narrowing on this path: used as it is
+    y = lin(x)
+    assert y.dtype == dtype and y.shape == (M, Q)
+    Wr = R.reconstruct(d, enc["esc_idx"].cpu().numpy(), enc["esc_vals"].cpu().numpy())
+    xs = x.float().cpu().numpy()
+    ref = O.linear_f64(xs, Wr)
+    tol = H.gemv_tolerance(ref, Wr, xs) + (2.0 ** -8 * np.abs(ref) if dtype == torch.bfloat16 else 0.0)
+    diff = np.abs(y.float().cpu().numpy().astype(np.float64) - ref)
+    assert np.all(diff <= tol), (float(diff.max()), float((diff / tol).max()))
+    assert torch.equal(y, lin(x))                                             # reproducible
+
+
+def test_module_large_m_paths_and_packfile(tmp_path):
+    Q, P = 96, 512
+    W, enc, d = _make(Q, P, 2e-3, seed=8, force=[1, P * 50 + 3], rows_per_tile=4, n_classes=2)
+    path = str(tmp_path / "t.qvb8r")
+    RP.write_pack(path, d)
+    bias = torch.linspace(-1, 1, Q)
+    lin = QVBandLinearV8R.from_packfile(path, bias=bias, device=DEV)
+    lin.CHUNK_BYTES = 2 * P * 40                                             # force several chunks
+    lin.__init__(dict(RP.container.read(path)), bias=bias, device=DEV, path=path)
+    assert len(lin.chunks) > 1
+    Wr = R.reconstruct(d, enc["esc_idx"].cpu().numpy(), enc["esc_vals"].cpu().numpy())
+    for M, dtype in ((30, torch.bfloat16), (70, torch.float16), (70, torch.float32)):
+        x = torch.randn(M, P, generator=torch.Generator().manual_seed(M)).to(dtype).to(DEV)
+        y = lin(x)
+        xs = x.float().cpu().numpy()
+        Wm = O.narrow_fp16(Wr) if M > 48 else Wr
+        if M > 48:
+            xs = O.sat_half(xs)
+        ref = O.linear_f64(xs, Wm) + bias.double().numpy()
+        eps = {torch.float32: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+        tol = H.gemv_tolerance(ref, Wm, xs) + eps * np.abs(ref)
+        diff = np.abs(y.float().cpu().numpy().astype(np.float64) - ref)
+        assert np.all(diff <= tol), (M, dtype, float((diff / tol).max()))
+    before = lin.tau_s.clone()
+    lin.to(torch.bfloat16)
+    assert lin.tau_s.dtype == torch.float32 and torch.equal(lin.tau_s, before)
+
+
+def test_argument_errors():
+    W, enc, d = _make(16, 256, 2e-3, seed=2)
+    lin = QVBandLinearV8R(d, device=DEV)
+    with pytest.raises(RuntimeError):
+        ext.multi(torch.zeros(17, 256, device=DEV), *lin._core(), T=lin.T)
+    with pytest.raises(RuntimeError):
+        ext.multi(torch.zeros(2, 256), *lin._core(), T=lin.T)               # host tensor
+    with pytest.raises(RuntimeError):
+        ext.decode(*lin._core(), 256, 2, 0, 99, -1, 0, T=lin.T)             # block range outside the schedule
+    short = lin.words[:100].contiguous()
+    with pytest.raises(RuntimeError):
+        ext.gemv(torch.zeros(256, device=DEV), short, *lin._core()[1:], T=lin.T)   # stream without its pad

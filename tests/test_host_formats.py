@@ -133,7 +133,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     from qvb8_amd import _lib
     header = open(os.path.join(ROOT, "include", "qvb8_amd.h")).read()
     body = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
-    declared = set(re.findall(r"\b(qvb8_[a-z0-9_]+)\s*\(", body))
+    declared = set(re.findall(r"\b(qvb8r?_[a-z0-9_]+)\s*\(", body))
     assert declared and declared == set(_lib.SYMBOLS)
     path = _lib.lib_path()
     if not os.path.exists(path):
