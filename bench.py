@@ -8,7 +8,8 @@ the clock starts (5+ GB of distinct buffers, so nothing is served from cache).  
 HIP graph and replayed; `value` is the algorithmic bytes of a step (packed ids + row metadata + escapes + activations
 in and out) divided by the measured time per step.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers 32] [--no-cpu] [--no-fuse] [--copy-probe]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--no-cpu] [--no-fuse] [--copy-probe]
+                    [--workload decode9b|moe|qvb8r] [--tokens T]
 
 Prints ONE JSON line.  `roofline` covers the dominant kernel (the tile kernel, every launch of the step):
 algorithmic bytes per launch / average launch time, timed with HIP events on the launch stream over the timed region.
@@ -112,12 +113,160 @@ def cpu_baseline(layers, x_by_p, budget_s=12.0):
                       % (len(done), ",".join(done), nbytes / 1e6, dt)}
 
 
+def time_graph(step, steps, warmup):
+    """Captures `step` (launches on torch's current stream) in a HIP graph, replays it `warmup` + `steps` times; returns
+    (ms per step by HIP events on the replay stream, ms per step by the host clock)."""
+    import torch
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return e0.elapsed_time(e1) / steps, wall * 1e3 / steps
+
+
+def bench_moe(args, dev):
+    """Config 4: Qwen-35B-A3B-shape MoE layer (hidden 2048, 128 experts of gate/up 2048->768 and down 768->2048, top-8
+    routing from softmax of N(0,1) logits), QVB8 at tau = 2e-3, `--tokens` tokens.  A step = the expert stacks of
+    `--layers` distinct layers through qvb8_moe_experts; bytes = packed ids + row metadata of the UNIQUE selected experts."""
+    import numpy as np
+    import torch
+    from oracle import qvb8_oracle as O                      # router_topk only: builds the synthetic routing, not timed
+    from qvb8_amd import _lib
+    from qvb8_amd.formats.qvb8 import pack as PK
+    from qvb8_amd.formats.qvb8.backends_experts import QVBandExpertsV8
+    from qvb8_amd.formats.qvb8.module import QVBandLinearV8
+    lib = _lib.load()
+    E, hidden, inter, k, T = 128, 2048, 768, 8, args.tokens
+    stacks = []
+    for l in range(args.layers):
+        gu, dn = [], []
+        for e in range(E):
+            g = torch.Generator(device=dev).manual_seed(100000 * l + e)
+            Wg = (0.02 * torch.randn(2 * inter, hidden, device=dev, generator=g)).to(torch.bfloat16)
+            Wd = (0.02 * torch.randn(hidden, inter, device=dev, generator=g)).to(torch.bfloat16)
+            gu.append(QVBandLinearV8.from_encoded(PK.encode_tensor(Wg, 2e-3)))
+            dn.append(QVBandLinearV8.from_encoded(PK.encode_tensor(Wd, 2e-3)))
+        m = QVBandExpertsV8(gu, dn, num_experts=E)
+        assert m.build_stack()
+        stacks.append(m._stk)
+    rng = np.random.default_rng(7)
+    x = torch.randn(T, hidden, device=dev, generator=torch.Generator(device=dev).manual_seed(7)).to(torch.bfloat16)
+    out = torch.empty(T, hidden, dtype=torch.bfloat16, device=dev)
+    ws = torch.empty(lib.qvb8_moe_workspace_bytes(T, k, E, 2 * inter, inter, hidden), dtype=torch.uint8, device=dev)
+    routes, step_bytes = [], 0
+    for g_, d_ in stacks:
+        idx, w = O.router_topk(rng.normal(size=(T, E)), k)
+        routes.append((torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)))
+        per_expert = (g_["ids"].numel() + d_["ids"].numel()) // E + 17 * (g_["Q"] + d_["Q"])
+        step_bytes += len(np.unique(idx)) * per_expert + 2 * T * hidden * 2
+
+    def step():
+        s = torch.cuda.current_stream().cuda_stream
+        for (g_, d_), (idx, w) in zip(stacks, routes):
+            rc = lib.qvb8_moe_experts(x.data_ptr(), 2, T, idx.data_ptr(), w.data_ptr(), k, E,
+                                      g_["ids"].data_ptr(), g_["ids"].numel(), g_["min_s"].data_ptr(), g_["tau_s"].data_ptr(),
+                                      g_["nbits"].data_ptr(), g_["bit_off"].data_ptr(), g_["Q"], g_["P"],
+                                      d_["ids"].data_ptr(), d_["ids"].numel(), d_["min_s"].data_ptr(), d_["tau_s"].data_ptr(),
+                                      d_["nbits"].data_ptr(), d_["bit_off"].data_ptr(), d_["Q"], d_["P"],
+                                      0, out.data_ptr(), 2, ws.data_ptr(), ws.numel(), s)
+            if rc != 0:
+                raise RuntimeError(lib.qvb8_last_error().decode())
+    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
+    ms = max(ev_ms, wall_ms)
+    gbs = step_bytes / (ms * 1e-3) / 1e9
+    per_layer_us = ev_ms * 1e3 / args.layers
+    return {"metric": "expert-gathered fused decode-GEMV GB/s on the bytes of the unique selected experts, 35B-A3B-shape MoE "
+                      "layer, 1 MI355X",
+            "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16 activations narrowed to fp16 x fp32 band value, fp32 accumulate", "data": "synthetic",
+            "config": {"workload": "MoE layer: hidden 2048, 128 experts gate/up 2048->768 + down 768->2048, top-8, QVB8 "
+                                   "tau=2e-3, %d token(s), %d layers" % (T, args.layers),
+                       "bytes_per_step": step_bytes, "us_per_layer": round(per_layer_us, 2)},
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                         "kernel": "qvb8::moe_plan_kernel + moe_gemv_kernel<0> + moe_gemv_kernel<1> + moe_combine_kernel "
+                                   "(one layer = 4 launches)",
+                         "bytes_per_launch": step_bytes // args.layers, "launch_us": round(per_layer_us, 3)},
+            "cpu_baseline": None}
+
+
+def bench_qvb8r(args, dev):
+    """Config 5 (27B-class shapes): hidden 5120, FFN 17408, QVB8R at tau = 2e-3, `--tokens` rows (1..16).  A step = gate,
+    up (17408 x 5120) and down (5120 x 17408) of `--layers` layers through qvb8r_gemv; bytes = coded words + states +
+    slot tables + row metadata."""
+    import ctypes
+    import torch
+    from qvb8_amd import _lib, ext_qvb8r
+    from qvb8_amd.formats.qvb8 import pack as PK
+    from qvb8_amd.formats.qvb8r import pack as RP
+    from qvb8_amd.formats.qvb8r.module import QVBandLinearV8R
+    lib = _lib.load()
+    M = args.tokens
+    units, step_bytes, n_sym = [], 0, 0
+    for l in range(args.layers):
+        for pi, (Q, P) in enumerate(((17408, 5120), (17408, 5120), (5120, 17408))):
+            g = torch.Generator(device=dev).manual_seed(5000 + 10 * l + pi)
+            W = (0.02 * torch.randn(Q, P, device=dev, generator=g)).to(torch.bfloat16)
+            d = RP.transcode(PK.encode_tensor(W, 2e-3, keep_ids=True))
+            del W
+            lin = QVBandLinearV8R(d, device=dev)
+            core, _, _ = ext_qvb8r._core(*lin._core(), P)
+            x = torch.randn(M, P, device=dev, generator=g).to(torch.bfloat16)
+            units.append(dict(lin=lin, core=core, x=x, Y=torch.empty(M, Q, dtype=torch.float32, device=dev),
+                              ws=torch.empty(lib.qvb8r_gemv_workspace_bytes(M, P), dtype=torch.uint8, device=dev)))
+            step_bytes += 4 * len(d["words"]) + 8 * 32 * len(d["tiles"]) + 4 * 4096 * d["K"] + 12 * Q + 8 * Q + 2 * M * (P + Q)
+            n_sym += Q * P
+
+    def step():
+        s = torch.cuda.current_stream().cuda_stream
+        for u in units:
+            rc = lib.qvb8r_gemv(u["x"].data_ptr(), 2, M, ctypes.byref(u["core"]), u["lin"].T, u["Y"].data_ptr(),
+                                u["ws"].data_ptr(), u["ws"].numel(), s)
+            if rc != 0:
+                raise RuntimeError(lib.qvb8_last_error().decode())
+    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
+    ms = max(ev_ms, wall_ms)
+    gbs = step_bytes / (ms * 1e-3) / 1e9
+    launch_us = ev_ms * 1e3 / len(units)
+    mb = 1 if M <= 1 else 2 if M <= 2 else 4 if M <= 4 else 8 if M <= 8 else 16
+    return {"metric": "QVB8R fused entropy-decode + GEMV GB/s on coded bytes, 27B-class FFN shapes, 1 MI355X",
+            "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16 activations as fp32 x fp32 band value, fp32 accumulate", "data": "synthetic",
+            "config": {"workload": "QVB8R tau=2e-3, hidden 5120 / FFN 17408 (gate, up, down), M=%d, %d layers" % (M, args.layers),
+                       "bytes_per_step": step_bytes, "bits_per_weight": round(8.0 * step_bytes / n_sym, 3),
+                       "symbols_per_s": round(n_sym / (ms * 1e-3), 1)},
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                         "kernel": "qvb8::r_gemv_kernel<%d> (+ r_transpose_kernel)" % mb,
+                         "bytes_per_launch": step_bytes // len(units), "launch_us": round(launch_us, 3),
+                         "note": "the walk is bound by dependent LDS lookups and a 64-bit multiply per symbol, not by HBM"},
+            "cpu_baseline": None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--layers", type=int, default=None, help="layers of distinct packs (default 32; moe 4; qvb8r 2)")
+    ap.add_argument("--workload", choices=("decode9b", "moe", "qvb8r"), default="decode9b",
+                    help="decode9b (default, the headline metric): 9B-shape decode step; moe: 35B-A3B-shape expert stack; "
+                         "qvb8r: entropy-coded 27B-class FFN shapes")
+    ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-fuse", action="store_true",
                     help="one launch per projection (7 per layer) instead of one per same-input group (q+k+v, gate+up: 4)")
@@ -137,6 +286,11 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     lib = _lib.load()                                       # raises when the HIP library is missing: no fallback
+    if args.layers is None:
+        args.layers = {"decode9b": 32, "moe": 4, "qvb8r": 2}[args.workload]
+    if args.workload != "decode9b":
+        print(json.dumps(bench_moe(args, dev) if args.workload == "moe" else bench_qvb8r(args, dev)))
+        return 0
     layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse)
     g = torch.Generator(device=dev).manual_seed(7)
     x_by_p = {P: torch.randn(1, P, device=dev, generator=g).to(torch.bfloat16) for P in (4096, 12288)}
@@ -164,23 +318,8 @@ def main():
             torch.add(src, 1.0, out=dst)
         torch.cuda.synchronize()
         del src, dst
-    step()
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        step()
-    for _ in range(args.warmup):
-        graph.replay()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()                                             # the graph replays on this (the current) stream
-    for _ in range(args.steps):
-        graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ev_ms = e0.elapsed_time(e1)
+    ev_per_step, wall_per_step = time_graph(step, args.steps, args.warmup)
+    ev_ms, wall = ev_per_step * args.steps, wall_per_step * args.steps * 1e-3
     ms_per_step = max(wall * 1e3, ev_ms) / args.steps
     gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
     launch_us = ev_ms * 1e3 / (args.steps * n_launch)
