@@ -30,8 +30,9 @@ LAYER_9B = (("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096,
             ("gate", 12288, 4096), ("up", 12288, 4096), ("down", 4096, 12288))
 TAU = 1e-3
 # HBM bytes per launch of the tile kernel from hardware counters (FETCH_SIZE scaled by 2.0 against a plain 1 GiB pass,
-# plus WRITE_SIZE), as recorded in profiles/tile_kernel_9b_decode_step_hbm_traffic.md: {workgroups: bytes}
-MEASURED_TRAFFIC = {256: (2 * 16078.3 + 39.8) * 1024, 64: (2 * 2014.4 + 4.9) * 1024}
+# plus WRITE_SIZE), as recorded in profiles/tile_kernel_9b_decode_step_hbm_traffic.md, by launch class
+MEASURED_TRAFFIC = {"q+k+v": (2 * 11039.5 + 33.2) * 1024, "fused-other": (2 * 24263.0 + 59.7) * 1024,      # default
+                    256: (2 * 16078.3 + 39.8) * 1024, 64: (2 * 2014.4 + 4.9) * 1024}                        # --no-fuse
 MMA_FLAGS = int(os.environ.get("QVB8_BENCH_MMA_FLAGS", "1"))     # 1 = QVB8_MMA_SATURATE_X: the operator's default for bf16 x
 
 
@@ -339,8 +340,9 @@ def main():
                    "bits_per_weight": round(8.0 * sum(u["lin"].ids.numel() for u in units) / sum(e["Q"] * e["P"] for e in flat), 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": (round(sum(MEASURED_TRAFFIC[256 if e["Q"] >= 4096 else 64] for e in flat) / n_launch)
-                                 if MMA_FLAGS == 1 and args.no_fuse else None),
+                     "traffic": (None if MMA_FLAGS != 1 else
+                                 round(sum(MEASURED_TRAFFIC[256 if e["Q"] >= 4096 else 64] for e in flat) / n_launch) if args.no_fuse
+                                 else round(sum(MEASURED_TRAFFIC["q+k+v" if u["name"] == "q+k+v" else "fused-other"] for u in units) / n_launch)),
                      "kernel": "qvb8::tile_kernel<1,4,false,true>", "bytes_per_launch": step_bytes // n_launch,
                      "launch_us": round(launch_us, 3)},
     }
