@@ -42,32 +42,53 @@ __host__ __device__ inline MoePlan moe_plan_at(void* ws, int64_t E, int64_t npai
                    reinterpret_cast<int32_t*>(p + 16 + moe_slots(E, npairs) * 16)};
 }
 
-// One workgroup: pairs grouped by expert (counting sort), list of the experts that have pairs.
+// One workgroup: pairs grouped by expert (counting sort), table of the experts that have pairs.  The two running
+// sums over the experts (pairs before expert e, selected experts before e) are a workgroup scan, 256 experts per round.
 __global__ void __launch_bounds__(kMoeThreads) moe_plan_kernel(const int64_t* __restrict__ idx, int npairs, int E, MoePlan pl) {
-    extern __shared__ int32_t s_cnt[];                        // [E] counts, then cursors
-    for (int e = threadIdx.x; e < E; e += blockDim.x) s_cnt[e] = 0;
-    if (threadIdx.x == 0) { *pl.n_bad = 0; }
+    extern __shared__ int32_t s_cnt[];                        // [E] counts, then cursors; [E .. E + 8) scan scratch
+    int32_t* s_scan = s_cnt + E;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int e = tid; e < E; e += blockDim.x) s_cnt[e] = 0;
+    if (tid == 0) *pl.n_bad = 0;
     __syncthreads();
     int bad = 0;
-    for (int p = threadIdx.x; p < npairs; p += blockDim.x) {
+    for (int p = tid; p < npairs; p += blockDim.x) {
         const int64_t e = idx[p];
         if (e >= 0 && e < E) atomicAdd(&s_cnt[(int)e], 1); else ++bad;
     }
     if (bad) atomicAdd(pl.n_bad, bad);
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int run = 0, na = 0;
-        const int n_slots = E < npairs ? E : npairs;
-        for (int e = 0; e < E; ++e) {
-            const int c = s_cnt[e];
-            if (c > 0) pl.slot[na++] = int4{e, run, run + c, 0};
-            s_cnt[e] = run;                                    // becomes the expert's cursor
-            run += c;
+    const int n_slots = E < npairs ? E : npairs;
+    int run_pairs = 0, run_active = 0;                        // totals of the rounds before this one (same in every thread)
+    for (int e0 = 0; e0 < E; e0 += blockDim.x) {
+        const int e = e0 + tid;
+        const int c = e < E ? s_cnt[e] : 0;
+        // inclusive scan of (c, c > 0) packed as pairs * 2^16 + active: both stay below 2^15 per round... pairs can be
+        // larger, so scan them separately
+        int sc = c, sa = c > 0 ? 1 : 0;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int tc = __shfl_up(sc, o, 64), ta = __shfl_up(sa, o, 64);
+            if (lane >= o) { sc += tc; sa += ta; }
         }
-        for (; na < n_slots; ++na) pl.slot[na] = int4{0, 0, 0, 0};
+        if (lane == 63) { s_scan[wave] = sc; s_scan[4 + wave] = sa; }
+        __syncthreads();
+        int base_c = run_pairs, base_a = run_active, tot_c = 0, tot_a = 0;
+        for (int w = 0; w < (int)(blockDim.x >> 6); ++w) {
+            if (w < wave) { base_c += s_scan[w]; base_a += s_scan[4 + w]; }
+            tot_c += s_scan[w]; tot_a += s_scan[4 + w];
+        }
+        const int first = base_c + sc - c;                    // pairs before expert e
+        if (e < E) {
+            if (c > 0) pl.slot[base_a + sa - 1] = int4{e, first, first + c, 0};
+            s_cnt[e] = first;                                 // becomes the expert's cursor
+        }
+        run_pairs += tot_c; run_active += tot_a;
+        __syncthreads();
     }
+    for (int i = run_active + tid; i < n_slots; i += blockDim.x) pl.slot[i] = int4{0, 0, 0, 0};
     __syncthreads();
-    for (int p = threadIdx.x; p < npairs; p += blockDim.x) {
+    for (int p = tid; p < npairs; p += blockDim.x) {
         const int64_t e = idx[p];
         if (e >= 0 && e < E) pl.order[atomicAdd(&s_cnt[(int)e], 1)] = p;
     }
@@ -368,7 +389,7 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
     float* H = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np));
     float* Yd = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np) + align256((size_t)np * P_dn * 4));
 
-    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)n_experts * 4, s, idx, (int)np, (int)n_experts, pl);
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)(n_experts + 8) * 4, s, idx, (int)np, (int)n_experts, pl);
     if (int rc = host::check_launch("qvb8_moe_experts plan")) return rc;
     const int64_t slots = moe_slots(n_experts, np);
 
