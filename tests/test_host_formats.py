@@ -164,3 +164,18 @@ def test_operators_fail_loudly_without_a_gpu():
     lin = QVBandLinearV8.from_encoded(enc)
     with pytest.raises(RuntimeError):
         lin(torch.zeros(1, 128))
+
+
+def test_format_registry():
+    from qvb8_amd.common import formats as F
+    assert F.known_formats() == ("qvb8", "qvb8r", "qvband")
+    spec = F.get_format("qvband")
+    assert spec.linear.__name__ == "QVBandLinearV8" and spec.experts.__name__ == "QVBandExpertsV8"
+    assert spec.filename("model.layers.0.mlp.up_proj.weight") == "model_layers_0_mlp_up_proj_weight.qvband"
+    assert F.get_format("qvb8r").linear.__name__ == "QVBandLinearV8R" and F.get_format("qvb8r").experts is None
+    with pytest.raises(NotImplementedError):
+        F.require(F.get_format("qvb8r"), "experts")
+    with pytest.raises(NotImplementedError):
+        F.require(spec, "cpu_linear")
+    with pytest.raises(ValueError):
+        F.get_format("fp8n")
