@@ -10,9 +10,9 @@ Restates, with the reference lines each part follows:
   ids / restore    id = symbol + drow[row]; value = fmaf(id, tau_s, min_s) (qvb8r_cuda.cu:113-115, 302); escapes overwrite
 Pinning: slot_tables and blocks_for against the reference's own outputs (tests/golden/ref_qvb8r_tables.npz); the walk by
 round trip, a closed-form single-lane rANS and, where oracle/_ref builds, by the reference's compiled encoder and row
-decoder; restore by the invariant "QVB8R restore == QVB8 restore of the same ids".  read_container is pinned by the
-layout description and by reading files the product writer makes (the reference's reader accepted such a file when the
-golden vectors were made); parity of the writer POLICY is unpinned by construction (the reference ships none).
+decoder; restore by the invariant "QVB8R restore == QVB8 restore of the same ids".  read_container and runtime_tables
+by what the reference's own reader returned for a file of this build and by a file the reference's writer made
+(tests/golden/ref_qvb8r_file.npz); parity of the writer POLICY is unpinned by construction (the reference ships none).
 """
 from __future__ import annotations
 

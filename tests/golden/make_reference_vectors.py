@@ -162,8 +162,41 @@ def qvb8r_vectors():
                           RF.VERSION], np.int64))
 
 
+def qvb8r_file_vectors():
+    """A .qvb8r file written by the REFERENCE's container.write from arrays this build's writer made, and what the
+    reference's container.read / runtime_tables return for the file THIS build's container writes."""
+    import tempfile
+    from qvb8_amd.formats.qvb8r import codec as MK
+    from qvb8_amd.formats.qvb8r import container as MC
+    rng = np.random.default_rng(9)
+    Q, P = 12, 256
+    ids = np.clip(np.round(rng.normal(40, 8, (Q, P))), 0, 127).astype(np.int64)
+    enc = MK.encode_ids(ids, n_classes=2, rows_per_tile=3)
+    min_s = rng.normal(-0.08, 0.01, Q).astype(np.float32)
+    tau_s = np.full(Q, 2e-3, np.float32)
+    esc_idx = np.array([7, P * 5 + 9], np.int64)
+    esc_val = np.array([0.5, -0.25], np.float32)
+    esc_delta = np.array([0.41, -0.2], np.float32)
+    cert = dict(tau=2e-3, restore="fp16")
+    with tempfile.TemporaryDirectory() as td:
+        ref_path = os.path.join(td, "ref.qvb8r")
+        RF.write(ref_path, enc, Q, P, min_s, tau_s, esc_idx, esc_val, esc_delta, cert)
+        ref_blob = open(ref_path, "rb").read()
+        mine = MC.to_bytes(enc, Q, P, min_s, tau_s, esc_idx, esc_val, esc_delta, cert)
+        d = RF.read(blob=mine)                                   # the reference's reader on this build's bytes
+        tab, tiles, words, off = RF.runtime_tables(d)
+    out = dict(ids=ids, min_s=min_s, tau_s=tau_s, esc_idx=esc_idx, esc_val=esc_val, esc_delta=esc_delta,
+               ref_blob=np.frombuffer(ref_blob, np.uint8), my_blob=np.frombuffer(mine, np.uint8),
+               rt_tab=tab, rt_tiles=tiles, rt_words=words, rt_off=off,
+               hdr=np.array([d["Q"], d["P"], d["T"], d["K"], d["N"], d["PB"]], np.int64))
+    for k in MC.ARRAYS:
+        out["read_" + k] = np.asarray(d[k])
+    save("ref_qvb8r_file.npz", **out)
+
+
 if __name__ == "__main__":
     bits_vectors()
     restore_vectors()
     blob_vectors()
     qvb8r_vectors()
+    qvb8r_file_vectors()

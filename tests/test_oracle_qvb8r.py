@@ -156,3 +156,24 @@ def test_writer_limits():
     assert np.array_equal(R.ids(dict(e, P=128, Q=3)), const)
     f = K.quantise_frequencies(np.array([10**6, 1, 0, 3]))
     assert f.sum() == 4096 and f.max() <= 1024 and f[1] >= 1 and f[3] >= 1
+
+
+def test_container_against_the_reference_reader_and_writer(golden):
+    """The reference's container.write output for this build's arrays is reproduced byte for byte, and what the
+    reference's container.read / runtime_tables returned for this build's file equals what the readers here return."""
+    g = golden("ref_qvb8r_file.npz")
+    ids, Q, P = g["ids"], int(g["hdr"][0]), int(g["hdr"][1])
+    enc = K.encode_ids(ids, n_classes=2, rows_per_tile=3)
+    mine = C.to_bytes(enc, Q, P, g["min_s"], g["tau_s"], g["esc_idx"], g["esc_val"], g["esc_delta"], dict(tau=2e-3, restore="fp16"))
+    assert mine == g["my_blob"].tobytes() == g["ref_blob"].tobytes()
+    for reader in (lambda b: C.read(blob=b), R.read_container):
+        d = reader(g["ref_blob"].tobytes())
+        for k in C.ARRAYS:
+            assert np.array_equal(np.asarray(d[k]), g["read_" + k]) and np.asarray(d[k]).dtype == g["read_" + k].dtype, k
+        assert [d["Q"], d["P"], d["T"], d["K"], d["N"], d["PB"]] == g["hdr"].tolist()
+    d = C.read(blob=mine)
+    for got, want in zip(C.runtime_tables(d), (g["rt_tab"], g["rt_tiles"], g["rt_words"], g["rt_off"])):
+        assert np.array_equal(got, want) and got.dtype == want.dtype
+    for got, want in zip(R.runtime_tables(R.read_container(mine)), (g["rt_tab"], g["rt_tiles"], g["rt_words"], g["rt_off"])):
+        assert np.array_equal(got, want)
+    assert np.array_equal(R.ids(R.read_container(mine)), ids)
