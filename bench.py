@@ -8,7 +8,7 @@ the clock starts (5+ GB of distinct buffers, so nothing is served from cache).  
 HIP graph and replayed; `value` is the algorithmic bytes of a step (packed ids + row metadata + escapes + activations
 in and out) divided by the measured time per step.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--no-cpu] [--no-fuse] [--copy-probe]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--no-cpu] [--no-fuse] [--no-sort] [--copy-probe]
                     [--workload decode9b|moe|qvb8r] [--tokens T]
 
 Prints ONE JSON line.  `roofline` covers the dominant kernel (the tile kernel, every launch of the step):
@@ -17,6 +17,7 @@ algorithmic bytes per launch / average launch time, timed with HIP events on the
 sample of the same workload (its first projections, about 12 s of CPU work), on the host cores of this machine.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -73,8 +74,8 @@ def build_layers(n_layers, dev, fuse):
             group = next((g for g in SAME_INPUT if name in g), (name,)) if fuse else (name,)
             lin = concat_linears([mods[n] for n in group])[0] if len(group) > 1 else mods[name]
             done.update(group)
-            perm, rowinfo = lin._mma_order()
-            units.append(dict(name="+".join(group), lin=lin, perm=perm, rowinfo=rowinfo, Q=lin.out_features,
+            perm, rowinfo, layout = lin._mma_order()
+            units.append(dict(name="+".join(group), lin=lin, perm=perm, rowinfo=rowinfo, layout=layout, Q=lin.out_features,
                               P=lin.in_features, n_esc=lin.esc_idx.numel(),
                               Y=torch.empty((1, lin.out_features), dtype=torch.float32, device=dev),
                               bytes=sum(algorithmic_bytes(e, 1) for e in encs if e["name"] in group)))
@@ -269,6 +270,9 @@ def main():
                          "qvb8r: entropy-coded 27B-class FFN shapes")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sort", action="store_true",
+                    help="keep the file's row order in memory (row addresses are then read from the row records instead of "
+                         "being computed from the width-sorted layout)")
     ap.add_argument("--no-fuse", action="store_true",
                     help="one launch per projection (7 per layer) instead of one per same-input group (q+k+v, gate+up: 4)")
     ap.add_argument("--copy-probe", action="store_true",
@@ -292,6 +296,9 @@ def main():
     if args.workload != "decode9b":
         print(json.dumps(bench_moe(args, dev) if args.workload == "moe" else bench_qvb8r(args, dev)))
         return 0
+    if args.no_sort:
+        from qvb8_amd.formats.qvb8.module import QVBandLinearV8
+        QVBandLinearV8.sort_rows = False
     layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse)
     g = torch.Generator(device=dev).manual_seed(7)
     x_by_p = {P: torch.randn(1, P, device=dev, generator=g).to(torch.bfloat16) for P in (4096, 12288)}
@@ -308,7 +315,9 @@ def main():
                               lin.min_s.data_ptr(), lin.tau_s.data_ptr(), lin.nbits.data_ptr(), lin.bit_off.data_ptr(),
                               u["Q"], u["P"], lin.esc_idx.data_ptr() if u["n_esc"] else None,
                               lin.esc_vals.data_ptr() if u["n_esc"] else None, u["n_esc"],
-                              u["perm"].data_ptr(), u["rowinfo"].data_ptr(), MMA_FLAGS, u["Y"].data_ptr(), None, 0, s)
+                              u["perm"].data_ptr(), u["rowinfo"].data_ptr(),
+                              ctypes.addressof(u["layout"]) if u["layout"] is not None else None,
+                              MMA_FLAGS, u["Y"].data_ptr(), None, 0, s)
             if rc != 0:
                 raise RuntimeError(lib.qvb8_last_error().decode())
 

@@ -106,6 +106,18 @@ int64_t qvb8_mma_rowinfo_bytes(int64_t Q);
 int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, const float* tau_s, const float* min_s,
                      const int32_t* perm, int64_t Q, int64_t P, int64_t ids_bytes, uint64_t* rowinfo, void* stream);
 
+/* Optional description of a pack whose rows are STORED in tile order from bit 0 of `ids`, back to back, one run per
+ * width (what a loader gets by copying the rows once, sorted by width): positions [first_pos[c], first_pos[c+1]) have
+ * width nbits[c] and row number perm[pos]; at most three runs.  A host struct, passed by pointer: with it the kernel
+ * computes where a row's ids are instead of reading that from the row records, which takes one dependent memory round
+ * trip off the start of every call. */
+#define QVB8_MMA_MAX_CLASSES 3
+typedef struct qvb8_mma_layout {
+    int32_t n_classes;
+    int32_t first_pos[QVB8_MMA_MAX_CLASSES + 1];
+    int32_t nbits[QVB8_MMA_MAX_CLASSES];
+} qvb8_mma_layout;
+
 /* Workspace qvb8_mma needs when it is called WITHOUT row records (it then builds them itself first). */
 int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
 
@@ -115,15 +127,16 @@ int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
  * in fp32 afterwards, so the result equals X times the UN-narrowed fp32 band value, escapes exact.
  * `perm` (i32[Q], position -> row, or NULL): order in which rows are grouped into tiles of 16; rows sorted by
  * width keep each tile on one decode pass (any order is correct).  `rowinfo`: from qvb8_mma_prepare for the same
- * perm, or NULL (then `workspace` must hold qvb8_mma_workspace_bytes).  Widths 4..8 on dword-aligned rows take the
- * fast path; other rows are read element by element.
+ * perm, or NULL (then `workspace` must hold qvb8_mma_workspace_bytes).  `layout`: NULL, or the description of rows stored
+ * in tile order (needs `rowinfo`).  Widths 4..8 on dword-aligned rows take the fast path; other rows are read element
+ * by element.
  * Replaces: ext.mma_multi  qvb8_mma_multi_forward qvb8_cuda.cu:2566-2671 (kernels :2321-2441, escape fix
  * :2503-2548), and, through the Python module, the M <= 8 GEMV of :1059-1166 when P % 128 == 0. */
 int qvb8_mma(const void* X, int x_dtype, int64_t M,
              const uint8_t* ids, int64_t ids_bytes, const float* min_s, const float* tau_s,
              const uint8_t* nbits, const int64_t* bit_off, int64_t Q, int64_t P,
              const int64_t* esc_idx, const float* esc_vals, int64_t n_esc,
-             const int32_t* perm, const uint64_t* rowinfo, int flags, float* Y,
+             const int32_t* perm, const uint64_t* rowinfo, const qvb8_mma_layout* layout, int flags, float* Y,
              void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- routed MoE expert stack (decode: a few tokens, top-k experts each) ---------------------------------------- */

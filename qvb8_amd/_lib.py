@@ -62,7 +62,7 @@ def load(build_if_missing: bool = True):
     lib.qvb8_mma_rowinfo_bytes.argtypes = [i64]
     lib.qvb8_mma_rowinfo_bytes.restype = i64
     lib.qvb8_mma_prepare.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, vp]
-    lib.qvb8_mma.argtypes = [vp, i32, i64, vp, i64, vp, vp, vp, vp, i64, i64, vp, vp, i64, vp, vp, i32, vp, vp, i64, vp]
+    lib.qvb8_mma.argtypes = [vp, i32, i64, vp, i64, vp, vp, vp, vp, i64, i64, vp, vp, i64, vp, vp, vp, i32, vp, vp, i64, vp]
     lib.qvb8_moe_workspace_bytes.argtypes = [i64] * 6
     lib.qvb8_moe_workspace_bytes.restype = i64
     lib.qvb8_moe_experts.argtypes = ([vp, i32, i64, vp, vp, i64, i64] + [vp, i64, vp, vp, vp, vp, i64, i64] * 2
@@ -76,6 +76,15 @@ def load(build_if_missing: bool = True):
         getattr(lib, name)                           # every declared symbol must be exported
     _LIB = lib
     return lib
+
+
+MMA_MAX_CLASSES = 3
+
+
+class MmaLayout(ctypes.Structure):
+    """qvb8_mma_layout of include/qvb8_amd.h."""
+    _fields_ = [("n_classes", ctypes.c_int32), ("first_pos", ctypes.c_int32 * (MMA_MAX_CLASSES + 1)),
+                ("nbits", ctypes.c_int32 * MMA_MAX_CLASSES)]
 
 
 class RCore(ctypes.Structure):

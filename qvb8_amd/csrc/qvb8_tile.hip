@@ -98,6 +98,10 @@ struct TileArgs {
     int n_steps;                  // P / 128
     int W, G, panels;             // waves per tile, tile groups per workgroup, column panels
     int TW;                       // tiles per workgroup (multiple of G)
+    // Rows STORED in tile order from bit 0 of `ids`, one run per width (at most three): positions [0, first1) have width
+    // nb[0], [first1, first2) nb[1], [first2, Q) nb[2].  n_classes == 0: addresses come from `loc`.
+    int n_classes, first1, first2;
+    int nb[3];
 };
 
 __global__ void __launch_bounds__(256) rowinfo_kernel(const uint8_t* __restrict__ nbits, const int64_t* __restrict__ bit_off,
@@ -173,9 +177,19 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
 // g.  Its activations for that range stay in registers for the whole panel.  Per tile it requests its T slices in
 // one burst (2T loads), turns them into MFMA operands as they arrive, and puts its partial sums into its own LDS
 // slots.  After one barrier the whole workgroup combines the column ranges of each row in a fixed order.
+// The kernel's arguments are 56 bytes of scalars (measured: every further 64 bytes of kernel arguments cost about a
+// microsecond per launch): fin follows loc, n_steps follows P, the small counts share one word.
 template <int NT, int T, bool BF, bool XC>
-__global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
+__global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ ids,
+                                                   const uint64_t* __restrict__ loc, float* __restrict__ Y, int64_t ids_bytes,
+                                                   int Q, int P, uint32_t counts, int TW, int first1, int first2, uint32_t widths) {
     static_assert(!(BF && XC), "narrowing on the way in exists for fp16 operands only");
+    TileArgs a;
+    a.X = X; a.ids = ids; a.loc = loc; a.fin = reinterpret_cast<const uint4*>(loc + rowinfo_loc_words(Q)); a.Y = Y;
+    a.ids_bytes = ids_bytes; a.Q = Q; a.P = P; a.n_steps = P / kStepCols; a.TW = TW;
+    a.M = (int)(counts & 63u); a.W = (int)((counts >> 8) & 15u); a.G = (int)((counts >> 12) & 15u); a.panels = (int)(counts >> 16);
+    a.first1 = first1; a.first2 = first2; a.n_classes = (int)(widths >> 24);
+    a.nb[0] = (int)(widths & 255u); a.nb[1] = (int)((widths >> 8) & 255u); a.nb[2] = (int)((widths >> 16) & 255u);
     using F = Fmt<BF>;
     using XI = XIn<BF, XC>;
     constexpr int TM = 16 * NT;
@@ -206,7 +220,23 @@ __global__ void __launch_bounds__(512) tile_kernel(TileArgs a) {
     uint64_t* my_loc = s_loc + (size_t)wave * wave_rows;
     for (int i = lane; i < n_tiles * kTileRows; i += kWave) {
         const int pos = local_to_pos((g + a.G * (i >> 4)) * kTileRows + (i & 15));
-        my_loc[i] = pos < a.Q ? a.loc[pos] : (3ull << 56);
+        uint64_t rec = 3ull << 56;
+        if (pos < a.Q) {
+            if (a.n_classes > 0) {
+                // no request: where the row is follows from the layout in the kernel arguments
+                const uint64_t P64 = (uint64_t)a.P;
+                const uint64_t base1 = (uint64_t)a.first1 * P64 * (uint64_t)a.nb[0];
+                const uint64_t base2 = base1 + (uint64_t)(a.first2 - a.first1) * P64 * (uint64_t)a.nb[1];
+                const int c = (pos >= a.first1 ? 1 : 0) + (pos >= a.first2 ? 1 : 0);
+                const uint64_t nbc = (uint64_t)(c == 0 ? a.nb[0] : c == 1 ? a.nb[1] : a.nb[2]);
+                const uint64_t bit0 = (c == 0 ? 0 : c == 1 ? base1 : base2)
+                                      + (uint64_t)(pos - (c == 0 ? 0 : c == 1 ? a.first1 : a.first2)) * P64 * nbc;
+                rec = bit0 | (nbc << 48) | ((uint64_t)((nbc >= 4 && nbc <= 8) ? 1 : 2) << 56);
+            } else {
+                rec = a.loc[pos];
+            }
+        }
+        my_loc[i] = rec;
     }
     // ---- what the end needs for row `tid`: requested now, parked in registers, put in LDS before the barrier ----
     uint4 e_fin = {0u, 0u, 0xffffffffu, 0u};
@@ -492,7 +522,11 @@ int launch_tile(TileArgs& a, hipStream_t s) {
             return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: cannot raise the kernel's LDS limit");
         attr[dev] = true;
     }
-    hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s, a);
+    if (pl.panels > 0xffff) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: rows too long");
+    const uint32_t counts = (uint32_t)a.M | ((uint32_t)a.W << 8) | ((uint32_t)a.G << 12) | ((uint32_t)a.panels << 16);
+    hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s,
+                       a.X, a.ids, a.loc, a.Y, a.ids_bytes, a.Q, a.P, counts, a.TW, a.first1, a.first2,
+                       (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16) | ((uint32_t)a.n_classes << 24));
     return host::check_launch("qvb8_mma");
 }
 }  // namespace
@@ -519,7 +553,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
                         const uint8_t* ids, int64_t ids_bytes, const float* min_s, const float* tau_s,
                         const uint8_t* nbits, const int64_t* bit_off, int64_t Q, int64_t P,
                         const int64_t* esc_idx, const float* esc_vals, int64_t n_esc,
-                        const int32_t* perm, const uint64_t* rowinfo, int flags, float* Y,
+                        const int32_t* perm, const uint64_t* rowinfo, const qvb8_mma_layout* layout, int flags, float* Y,
                         void* workspace, int64_t workspace_bytes, void* stream) {
     if (Q < 0 || P < 0 || Q > 0x7fffffff || P > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8_mma: Q or P out of range");
     if (M < 1 || M > 48) return host::fail(QVB8_ERR_ARG, "qvb8 mma-multi: M=%lld outside 1..48", (long long)M);
@@ -540,6 +574,24 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     }
     TileArgs a;
     a.X = (const uint16_t*)X; a.ids = ids; a.loc = rowinfo; a.fin = reinterpret_cast<const uint4*>(rowinfo + rowinfo_loc_words(Q));
+    a.n_classes = 0; a.first1 = a.first2 = (int)Q; a.nb[0] = a.nb[1] = a.nb[2] = 0;
+    if (layout) {
+        if (!rowinfo) return host::fail(QVB8_ERR_ARG, "qvb8_mma: a row layout goes with the row records of the same order");
+        const int n = layout->n_classes;
+        if (n < 1 || n > QVB8_MMA_MAX_CLASSES || layout->first_pos[0] != 0 || layout->first_pos[n] != Q)
+            return host::fail(QVB8_ERR_ARG, "qvb8_mma: bad row layout (1..3 classes that cover positions 0..Q)");
+        int64_t bits = 0;
+        for (int c = 0; c < n; ++c) {
+            const int64_t rows = (int64_t)layout->first_pos[c + 1] - layout->first_pos[c], nbc = layout->nbits[c];
+            if (rows < 0 || nbc < 1 || nbc > 14) return host::fail(QVB8_ERR_ARG, "qvb8_mma: bad row layout class %d", c);
+            bits += rows * P * nbc;
+            a.nb[c] = (int)nbc;
+        }
+        if ((bits >> 3) + 8 > ids_bytes) return host::fail(QVB8_ERR_ARG, "qvb8_mma: the row layout does not fit the ids buffer");
+        a.first1 = n > 1 ? layout->first_pos[1] : (int)Q;
+        a.first2 = n > 2 ? layout->first_pos[2] : (int)Q;
+        a.n_classes = n;
+    }
     a.Y = Y; a.ids_bytes = ids_bytes; a.M = (int)M; a.Q = (int)Q; a.P = (int)P; a.n_steps = (int)(P / kStepCols);
     // mode 0: fp16 X, fp16 operands; 1: bf16 X narrowed to saturated fp16 on the way in, fp16 operands; 2: bf16 operands
     const int mode = x_dtype == QVB8_F16 ? 0 : (flags & QVB8_MMA_SATURATE_X) ? 1 : 2;

@@ -12,6 +12,8 @@ saturating_half.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -168,11 +170,54 @@ def mma_prepare(row_nbits, row_bit_off, tau_s, min_s, P, ids_bytes, perm=None):
     return out
 
 
+def sort_rows_by_width(ids, row_nbits, row_bit_off, P, perm):
+    """Copies the rows of a pack into `perm` order (rows of one width back to back, from byte 0), once, at load: returns
+    (ids_sorted, row_bit_off_sorted, layout) -- the new ids buffer, the new per-row bit offsets (still indexed by row) and
+    the _lib.MmaLayout that lets mma_tiles compute row addresses instead of reading them.  None when the pack cannot be
+    laid out that way (P % 128 != 0, rows that do not start on 16-byte boundaries, more than 3 distinct widths)."""
+    _lib.require_cuda(ids, row_nbits, row_bit_off, perm)
+    Q, P = row_nbits.numel(), int(P)
+    if Q == 0 or P % 128 != 0 or bool((row_bit_off % 128 != 0).any()):
+        return None
+    nb_sorted = row_nbits[perm.long()].to(torch.int64)
+    widths, counts = torch.unique_consecutive(nb_sorted, return_counts=True)
+    widths, counts = widths.tolist(), counts.tolist()                      # one host read, at load
+    if len(widths) > _lib.MMA_MAX_CLASSES or sorted(set(widths)) != widths:
+        return None
+    row_bits = nb_sorted * P
+    new_off_sorted = torch.cumsum(row_bits, 0) - row_bits                  # rows back to back in the new order
+    total_bytes = int(row_bits.sum().item()) // 8
+    out = torch.zeros(total_bytes + 8, dtype=torch.uint8, device=ids.device)
+    src16 = ids[: (ids.numel() // 16) * 16].view(-1, 16)
+    dst16 = out[:total_bytes].view(-1, 16)
+    src_off = row_bit_off[perm.long()]
+    layout = _lib.MmaLayout()
+    layout.n_classes = len(widths)
+    pos = 0
+    for c, (w, n) in enumerate(zip(widths, counts)):
+        layout.first_pos[c], layout.nbits[c] = pos, int(w)
+        blocks = P * w // 128                                              # 16-byte blocks per row
+        ar = torch.arange(blocks, device=ids.device)
+        for r0 in range(pos, pos + n, 4096):                               # bounded index tensors
+            r1 = min(pos + n, r0 + 4096)
+            s_idx = (src_off[r0:r1, None] // 128 + ar[None, :]).reshape(-1)
+            d_idx = (new_off_sorted[r0:r1, None] // 128 + ar[None, :]).reshape(-1)
+            if int(s_idx.max().item()) >= src16.shape[0]:
+                return None
+            dst16[d_idx] = src16[s_idx]
+        pos += n
+    layout.first_pos[len(widths)] = Q
+    new_off = torch.empty_like(row_bit_off)
+    new_off[perm.long()] = new_off_sorted
+    return out, new_off, layout
+
+
 def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm=None, saturate=True,
-              rowinfo=None):
+              rowinfo=None, layout=None):
     """Matrix-core path for 1 <= M <= 48 and P % 128 == 0: X (fp16 or bf16) times the fp32 band value, fp32 (M, Q).
     `perm` (int32, position -> row) groups rows of equal width into tiles; `rowinfo` = mma_prepare(...) for the
-    same perm (built on the fly when absent).  `saturate` (bf16 X only): X is narrowed like saturating_half while it
+    same perm (built on the fly when absent); `layout` = the third result of sort_rows_by_width for a pack whose rows were
+    copied into that order (needs `rowinfo`).  `saturate` (bf16 X only): X is narrowed like saturating_half while it
     is loaded and the product runs on fp16 operands, as every fp16 path of the reference does; without it bf16 X is
     multiplied as it is on bf16 operands."""
     lib = _lib.load()
@@ -210,6 +255,7 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
                                  _lib.ptr(min_s), _lib.ptr(tau_s), _lib.ptr(row_nbits), _lib.ptr(row_bit_off),
                                  Q, int(P), _lib.ptr(ei), _lib.ptr(ev), n_esc, _lib.ptr(perm),
                                  None if rowinfo is None else rowinfo.contiguous().data_ptr(),
+                                 None if layout is None else ctypes.addressof(layout),
                                  MMA_SATURATE_X if saturate else 0, _lib.ptr(Y),
                                  None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel() * 8,
                                  _lib.stream_of(Xc)), lib)

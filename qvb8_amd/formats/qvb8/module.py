@@ -49,6 +49,10 @@ def apply_keeping_fp32_metadata(module: nn.Module, fn, recurse=True):
 
 
 class QVBandLinearV8(nn.Module):
+    # The first call of the matrix-core path copies the rows once into width-sorted order (same total size; `ids` and
+    # `bit_off` are replaced, every kernel keeps working through bit_off), so that calls compute row addresses instead of
+    # reading them.  Set False to keep the file's row order in memory.
+    sort_rows = True
     bf16_gemm = False             # opt-in: M > 96 bf16 callers decode to bf16 and run one bf16 GEMM (module.py:60-65)
     bf16_certified = False        # the pack certifies |orig - bf16(band)| <= tau (container restore code 3)
     fp16_table_missing = False    # fp16+bf16 pack loaded without escape_tables.json: fp16 forwards refuse
@@ -188,7 +192,7 @@ class QVBandLinearV8(nn.Module):
     # ---- launch metadata ---------------------------------------------------------------------------------------
 
     def _mma_order(self):
-        """(perm, rowinfo) for ext.mma_tiles, or None when the tile kernel cannot read this weight.  Rows are sorted by
+        """(perm, rowinfo, layout) for ext.mma_tiles, or None when the tile kernel cannot read this weight.  Rows are sorted by
         width so that a 16-row tile shares one width (one decode pass); the row records hold, in that order, where each
         row's ids start, its width, tau_s, min_s and its output row.  Built once per weight, like the reference's
         perm / tile_nb (module.py:230-277); never built inside a graph capture (the width check reads the device)."""
@@ -202,9 +206,15 @@ class QVBandLinearV8(nn.Module):
             nb = self.nbits.to(torch.int16)
             if 1 <= int(nb.min()) and int(nb.max()) <= 14:
                 perm = torch.argsort(nb, stable=True).to(torch.int32).contiguous()
+                layout = None
+                row_bytes = int((self.nbits.to(torch.int64) * self.in_features).sum().item()) // 8
+                if self.sort_rows and 2 * row_bytes >= self.ids.numel():      # not for a small view into a shared stack
+                    srt = ext.sort_rows_by_width(self.ids, self.nbits, self.bit_off, self.in_features, perm)
+                    if srt is not None:
+                        self.ids, self.bit_off, layout = srt
                 rowinfo = ext.mma_prepare(self.nbits, self.bit_off, self.tau_s, self.min_s, self.in_features,
                                           self.ids.numel(), perm)
-                order = (perm, rowinfo)
+                order = (perm, rowinfo, layout)
         self._mma_cache = order
         return order
 
@@ -247,10 +257,10 @@ class QVBandLinearV8(nn.Module):
             return torch.cat([self.forward(xk[i:i + step]) for i in range(0, M, step)]) \
                 .reshape(*orig[:-1], self.out_features).to(out_dtype)
         if order is not None:
-            perm, rowinfo = order
+            perm, rowinfo, layout = order
             xm = xk if xk.dtype in (torch.float16, torch.bfloat16) else ext.saturating_half(xk)
             y = ext.mma_tiles(xm, self.ids, self.min_s, self.nbits, self.bit_off, self.in_features, self.tau_s,
-                              ei, ev, perm=perm, saturate=not bf16_mode, rowinfo=rowinfo)
+                              ei, ev, perm=perm, saturate=not bf16_mode, rowinfo=rowinfo, layout=layout)
             return self._finish(y, orig, out_dtype)
         if M <= 8:
             y = ext.gemv_multi(xk, self.ids, self.min_s, self.nbits, self.bit_off, self.in_features, self.tau_s,

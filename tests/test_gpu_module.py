@@ -147,3 +147,30 @@ def test_same_input_fusion_is_bit_identical():
     for a, b in zip(got, want):
         assert torch.equal(a, b)
     assert blk.self_attn._qvb8_fused._x is None           # every member took its part: nothing is held
+
+
+@pytest.mark.parametrize("widths,sortable", [([7, 6, 9], True), ([5], True), ([7, 6, 9, 3, 8, 5], False)])
+def test_rows_copied_into_width_order(widths, sortable):
+    """The module copies its rows once into width-sorted order and then lets the kernel compute row addresses (at most
+    three widths; other packs keep the row records).  Either way results match the oracle and the dense restore is
+    unchanged by the copy."""
+    d = H.mixed_width_pack(70, 256, widths, seed=21)
+    d["tau_s"] = d["tau_s"] * (1.0 / 64)
+    a = H.to_device_args(d, DEV)
+    lin = QVBandLinearV8(min_s=a[1], nbits=a[2], bit_off=a[3], ids=a[0], Q=70, P=256, tau_s=a[5], esc_idx=a[6], esc_vals=a[7])
+    from qvb8_amd import ext_qvb8 as ext
+    before = ext.decode_f32(lin.ids, lin.min_s, lin.nbits, lin.bit_off, 256, lin.tau_s, lin.esc_idx, lin.esc_vals)
+    old_ptr = lin.ids.data_ptr()
+    Wr = O.reconstruct(d["min_s"], d["tau_s"], d["ids_dense"], d["esc_idx"], d["esc_vals"])
+    for M, dtype in ((1, torch.bfloat16), (20, torch.float16)):
+        x = torch.randn(M, 256, generator=torch.Generator().manual_seed(M)).to(dtype).to(DEV)
+        y = lin(x)
+        xs = O.sat_half(x.float().cpu().numpy())
+        _close(y, O.linear_f64(xs, Wr), Wr, xs, dtype)
+    perm, rowinfo, layout = lin._mma_order()
+    assert (layout is not None) == sortable and (lin.ids.data_ptr() != old_ptr) == sortable
+    if sortable:
+        assert layout.n_classes == len(set(widths)) and layout.first_pos[layout.n_classes] == 70
+        assert bool((lin.nbits[perm.long()][1:] >= lin.nbits[perm.long()][:-1]).all())
+    after = ext.decode_f32(lin.ids, lin.min_s, lin.nbits, lin.bit_off, 256, lin.tau_s, lin.esc_idx, lin.esc_vals)
+    assert torch.equal(before, after)
