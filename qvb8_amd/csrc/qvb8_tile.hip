@@ -324,8 +324,9 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
                     *dst = first_panel ? sx[nt][e] : *dst + sx[nt][e];
                 }
         }
-        // The first tile's ids are requested only now: the few activation requests above must not queue up behind
-        // the flood of id requests of the whole chip (measured: asking for the ids first costs about a microsecond).
+        // The first tile's ids are requested only now, after the activations have ARRIVED: requesting them earlier --
+        // before the activations, or right behind them -- was measured to cost about a microsecond per launch (the few
+        // activation requests then compete with the flood of id requests of the whole chip).
         // Later panels' first ids are in flight already (requested at the end of the panel before).
         if (n_mine > 0 && first_panel) info = issue_tile(0, step0, wlo, whi);
 
