@@ -9,7 +9,7 @@ HIP graph and replayed; `value` is the algorithmic bytes of a step (packed ids +
 in and out) divided by the measured time per step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--no-cpu] [--no-fuse] [--no-sort] [--copy-probe]
-                    [--workload decode9b|moe|qvb8r] [--tokens T]
+                    [--workload decode9b|smallm|moe|qvb8r] [--tokens T]
 
 Prints ONE JSON line.  `roofline` covers the dominant kernel (the tile kernel, every launch of the step):
 algorithmic bytes per launch / average launch time, timed with HIP events on the launch stream over the timed region.
@@ -259,15 +259,53 @@ def bench_qvb8r(args, dev):
             "cpu_baseline": None}
 
 
+def bench_smallm(args, dev):
+    """Config 3: the 9B projections with M = `--tokens` rows (draft-verify / prefill chunk), through QVBandLinearV8's own
+    dispatch: M <= 48 one fused decode + MFMA launch per projection group, 49..96 two passes, above that dense restore
+    to fp16 + library GEMM.  Reports GB/s on the packed bytes and TFLOP/s (2 M Q P per projection, decode ops not counted)."""
+    import torch
+    layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse)
+    M = args.tokens
+    g = torch.Generator(device=dev).manual_seed(7)
+    x_by_p = {P: torch.randn(M, P, device=dev, generator=g).to(torch.bfloat16) for P in (4096, 12288)}
+    flat = [enc for lay in layers for enc in lay]
+    step_bytes = sum(algorithmic_bytes(e, M) for e in flat)
+    flops = sum(2.0 * M * e["Q"] * e["P"] for e in flat)
+    for u in units:
+        u["lin"](x_by_p[u["P"]])                                    # builds the per-weight launch data outside the graph
+
+    def step():
+        for u in units:
+            u["out"] = u["lin"](x_by_p[u["P"]])
+    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
+    ms = max(ev_ms, wall_ms)
+    gbs = step_bytes / (ms * 1e-3) / 1e9
+    tflops = flops / (ms * 1e-3) / 1e12
+    path = "fused decode + MFMA (qvb8_mma)" if M <= 48 else "two fused passes" if M <= 96 else "fp16 restore + library GEMM"
+    bound = "hbm" if M <= 96 else "mfma"
+    return {"metric": "small-M fused decode + GEMM: GB/s on packed bytes and TFLOP/s, 9B projections, 1 MI355X",
+            "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16 activations, fp32 accumulate, bf16 out", "data": "synthetic", "tflops": round(tflops, 3),
+            "config": {"workload": "9B-shape projections, QVB8 tau=1e-3, M=%d, %d layers, path: %s" % (M, args.layers, path),
+                       "bytes_per_step": step_bytes, "flops_per_step": flops, "launch_units": len(units)},
+            "roofline": ({"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+                         if bound == "hbm" else
+                         {"bound": "mfma", "achieved": round(tflops, 3), "peak": 2500.0, "unit": "TFLOP/s",
+                          "frac": round(tflops / 2500.0, 5), "traffic": None}),
+            "cpu_baseline": None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=None, help="layers of distinct packs (default 32; moe 4; qvb8r 2)")
-    ap.add_argument("--workload", choices=("decode9b", "moe", "qvb8r"), default="decode9b",
+    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r"), default="decode9b",
                     help="decode9b (default, the headline metric): 9B-shape decode step; moe: 35B-A3B-shape expert stack; "
-                         "qvb8r: entropy-coded 27B-class FFN shapes")
+                         "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256)")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sort", action="store_true",
@@ -292,9 +330,10 @@ def main():
     torch.cuda.set_device(dev)
     lib = _lib.load()                                       # raises when the HIP library is missing: no fallback
     if args.layers is None:
-        args.layers = {"decode9b": 32, "moe": 4, "qvb8r": 2}[args.workload]
+        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 2}[args.workload]
     if args.workload != "decode9b":
-        print(json.dumps(bench_moe(args, dev) if args.workload == "moe" else bench_qvb8r(args, dev)))
+        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm}[args.workload]
+        print(json.dumps(fn(args, dev)))
         return 0
     if args.no_sort:
         from qvb8_amd.formats.qvb8.module import QVBandLinearV8
