@@ -206,7 +206,7 @@ def bench_moe(args, dev):
 
 
 def bench_qvb8r(args, dev):
-    """Config 5 (27B-class shapes): hidden 5120, FFN 17408, QVB8R at tau = 2e-3, `--tokens` rows (1..16).  A step = gate,
+    """Config 5 (27B-class shapes): hidden 5120, FFN 17408, QVB8R at tau = 2e-3, `--tokens` rows (1..48).  A step = gate,
     up (17408 x 5120) and down (5120 x 17408) of `--layers` layers through qvb8r_gemv; bytes = coded words + states +
     slot tables + row metadata."""
     import ctypes
@@ -243,17 +243,18 @@ def bench_qvb8r(args, dev):
     ms = max(ev_ms, wall_ms)
     gbs = step_bytes / (ms * 1e-3) / 1e9
     launch_us = ev_ms * 1e3 / len(units)
-    mb = 1 if M <= 1 else 2 if M <= 2 else 4 if M <= 4 else 8 if M <= 8 else 16
+    kernel = "qvb8::r_gemv_kernel<2>" if M == 1 else "qvb8::r_mma_kernel<%d, false> (+ r_pack_x_kernel)" % ((M + 15) // 16)
     return {"metric": "QVB8R fused entropy-decode + GEMV GB/s on coded bytes, 27B-class FFN shapes, 1 MI355X",
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "bf16 activations as fp32 x fp32 band value, fp32 accumulate", "data": "synthetic",
+            "dtype": "bf16 activations x fp32 band value (M > 1: exact fp16 operands on the matrix cores), fp32 accumulate",
+            "data": "synthetic",
             "config": {"workload": "QVB8R tau=2e-3, hidden 5120 / FFN 17408 (gate, up, down), M=%d, %d layers" % (M, args.layers),
                        "bytes_per_step": step_bytes, "bits_per_weight": round(8.0 * step_bytes / n_sym, 3),
                        "symbols_per_s": round(n_sym / (ms * 1e-3), 1)},
             "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                         "kernel": "qvb8::r_gemv_kernel<%d> (+ r_transpose_kernel)" % mb,
+                         "kernel": kernel,
                          "bytes_per_launch": step_bytes // len(units), "launch_us": round(launch_us, 3),
                          "note": "the walk is bound by dependent LDS lookups and a 64-bit multiply per symbol, not by HBM"},
             "cpu_baseline": None}

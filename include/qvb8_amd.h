@@ -192,13 +192,18 @@ typedef struct qvb8r_core {
 int qvb8r_decode(const qvb8r_core* core, int64_t max_tile_rows, int out_dtype, int64_t b0, int64_t nb, int64_t row_base,
                  void* out, int64_t out_rows, void* stream);
 
-/* Bytes of workspace qvb8r_gemv needs (the activations transposed to (P, 1|2|4|8|16) fp32). */
+/* Bytes of workspace qvb8r_gemv needs: 16 for M = 1 (X is read in place); for M = 2..48 the activations packed as
+ * fp16 hi + lo planes in matrix-core operand order plus one sum and one scale exponent per row. */
 int64_t qvb8r_gemv_workspace_bytes(int64_t M, int64_t P);
 
-/* Y[m, q] = sum_c X[m, c] * value(q, c) for M = 1..16, X (M, P) in x_dtype used in fp32 as it is (no narrowing), fp32
- * accumulate, Y f32 (M, Q) row-major, every row written.  Escapes are NOT corrected (qvb8r_fix_escapes).
- * Replaces: ext.gemv  qvb8r_gemv qvb8r_cuda.cu:88-131, ext.multi  qvb8r_multi :153-194 and, for 9..16 rows, ext.tc
- * qvb8r_tc :199-272 (which multiplies fp16-rounded weights; this one keeps the fp32 band value). */
+/* Y[m, q] = sum_c X[m, c] * value(q, c) for M = 1..48, fp32 accumulate, Y f32 (M, Q) row-major, every row written.
+ * M = 1: X in x_dtype is used in fp32 as it is.  M >= 2: one walk of the stream serves all rows on the matrix cores;
+ * each row of X is scaled by a power of two into fp16 range and used as fp16 hi + lo (fp32 X: 22 significant bits;
+ * fp16 / bf16 X: exact), the symbols are exact fp16 integers, so the product differs from fp32 arithmetic only by the
+ * split of fp32 activations.  A row of X with a non-finite element gives non-finite outputs for that row.
+ * Escapes are NOT corrected (qvb8r_fix_escapes).
+ * Replaces: ext.gemv  qvb8r_gemv qvb8r_cuda.cu:88-131, ext.multi  qvb8r_multi :153-194 and ext.tc  qvb8r_tc :199-272
+ * (which multiplies fp16-rounded weights; this one keeps the fp32 band value). */
 int qvb8r_gemv(const void* X, int x_dtype, int64_t M, const qvb8r_core* core, int64_t max_tile_rows, float* Y,
                void* workspace, int64_t workspace_bytes, void* stream);
 

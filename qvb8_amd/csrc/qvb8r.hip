@@ -9,7 +9,11 @@
 // class) maps one block to one workgroup.  id = symbol + drow[row]; value = fmaf(id, tau_s[row], min_s[row]).
 //
 //   qvb8r_decode   dense rows (fp32 / fp16 / bf16 values, or the ids as int16), bit-exact with the QVB8 restore
-//   qvb8r_gemv     M = 1..16 rows of X (fp32 arithmetic): Y = tau_s * (sum x * symbol + drow * sum x) + min_s * sum x
+//   qvb8r_gemv     Y = tau_s * (sum x * symbol + drow * sum x) + min_s * sum x.  M = 1: fp32 multiply-adds per lane.
+//                  M = 2..48: the symbols of a workgroup's eight rows go through LDS as exact fp16 integers and meet X on
+//                  the matrix cores (v_mfma_f32_16x16x32_f16, fp32 accumulate), so the cost of a launch is the walk and
+//                  hardly depends on M.  X is scaled per row by a power of two into fp16 range and split hi + lo (lo only
+//                  for fp32 X: fp16 / bf16 values are exact in hi), the scale is undone exactly at the end.
 //   qvb8r_fix_escapes   Y[m, q] += sum over q's escapes of x[m, c] * delta, in stored order, one thread per output
 //
 // The walk is bound by the dependent LDS lookups and the 64-bit multiply per symbol, not by HBM (the stream is about
@@ -161,33 +165,9 @@ __global__ void __launch_bounds__(kRThreads) r_decode_kernel(RCore c, int b0, in
     }
 }
 
-// ---- activations, transposed: Xt[c][mb] fp32, mb < MB (rows past M are zero) ----------------------------------------
-__global__ void __launch_bounds__(256) r_transpose_kernel(const void* __restrict__ X, int x_dtype, int M, int P, int MB, float* __restrict__ Xt) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= (int64_t)P * MB) return;
-    const int c = (int)(i / MB), mb = (int)(i - (int64_t)c * MB);
-    Xt[i] = mb < M ? load_as_f32(X, (int64_t)mb * P + c, x_dtype) : 0.f;
-}
-
-// ---- fused decode + product, M = 1..16 -------------------------------------------------------------------------------
-template <int MB>
-__device__ __forceinline__ void load_xt(const float* __restrict__ p, float (&v)[MB]) {
-    if constexpr (MB >= 4) {
-#pragma unroll
-        for (int i = 0; i < MB; i += 4) {
-            const float4 q = *reinterpret_cast<const float4*>(p + i);
-            v[i] = q.x; v[i + 1] = q.y; v[i + 2] = q.z; v[i + 3] = q.w;
-        }
-    } else if constexpr (MB == 2) {
-        const float2 q = *reinterpret_cast<const float2*>(p);
-        v[0] = q.x; v[1] = q.y;
-    } else {
-        v[0] = p[0];
-    }
-}
-
-template <int MB>
-__global__ void __launch_bounds__(kRThreads) r_gemv_kernel(RCore c, const float* __restrict__ Xt, int M, float* __restrict__ Y, int T) {
+// ---- fused decode + product, one row of X ------------------------------------------------------------------------------
+template <int DT>
+__global__ void __launch_bounds__(kRThreads) r_gemv_kernel(RCore c, const void* __restrict__ X, float* __restrict__ Y, int T) {
     __shared__ uint32_t st[4096];
     __shared__ uint32_t ring[kRTiles][kRing];
     const int lane = threadIdx.x & 63, l32 = lane & 31, half = lane >> 5, h8 = threadIdx.x >> 5;
@@ -198,47 +178,196 @@ __global__ void __launch_bounds__(kRThreads) r_gemv_kernel(RCore c, const float*
     t.room = c.n_words - 1 - (z.wp - c.words);
     __syncthreads();
     const int S = c.P >> 5;
-    // sums of x over this lane's columns (the same for every row): taken while the first row is walked
-    float sx[MB];
-#pragma unroll
-    for (int i = 0; i < MB; ++i) sx[i] = 0.f;
+    float sx = 0.f;                  // sum of x over this lane's columns (the same for every row): taken while the first row is walked
     for (int r = 0; r < T; ++r) {
         if (!(t.has && r < t.nr)) continue;                                // per half-wave
         const int orow = c.perm[t.r0 + r];
         const bool row_ok = orow >= 0 && orow < c.Q;
-        float acc[MB], x1[MB], x2[MB];
-#pragma unroll
-        for (int i = 0; i < MB; ++i) acc[i] = 0.f;
-        load_xt<MB>(Xt + (int64_t)l32 * MB, x1);
-        load_xt<MB>(Xt + (int64_t)(32 + l32) * MB, x2);
+        float acc = 0.f;
+        float x1 = load_as_f32<DT>(X, l32), x2 = load_as_f32<DT>(X, 32 + l32);
         for (int s0 = 0; s0 < S; s0 += 2) {
-            float n1[MB], n2[MB];
             const int sn = s0 + 2 < S ? s0 + 2 : s0;                       // the last pair reloads itself (unused)
-            load_xt<MB>(Xt + (int64_t)(sn * 32 + l32) * MB, n1);
-            load_xt<MB>(Xt + (int64_t)((sn + 1) * 32 + l32) * MB, n2);
+            const float n1 = load_as_f32<DT>(X, sn * 32 + l32), n2 = load_as_f32<DT>(X, (sn + 1) * 32 + l32);
             uint32_t s1, s2;
             walk_pair(z, st, rg, l32, half, t.room, s1, s2);
-            const float f1 = (float)s1, f2 = (float)s2;
-#pragma unroll
-            for (int i = 0; i < MB; ++i) {
-                acc[i] = __builtin_fmaf(x1[i], f1, acc[i]);
-                acc[i] = __builtin_fmaf(x2[i], f2, acc[i]);
-                if (r == 0) sx[i] += x1[i] + x2[i];
-                x1[i] = n1[i]; x2[i] = n2[i];
-            }
+            acc = __builtin_fmaf(x1, (float)s1, acc);
+            acc = __builtin_fmaf(x2, (float)s2, acc);
+            if (r == 0) sx += x1 + x2;
+            x1 = n1; x2 = n2;
         }
-        if (r == 0) {
-#pragma unroll
-            for (int i = 0; i < MB; ++i) sx[i] = half_sum(sx[i]);
-        }
+        if (r == 0) sx = half_sum(sx);
         const double m = row_ok ? (double)c.min_s[orow] : 0.0, ts = row_ok ? (double)c.tau_s[orow] : 0.0;
         const double dr = row_ok ? (double)c.drow[orow] : 0.0;
+        const float a = half_sum(acc);
+        if (l32 == 0 && row_ok) Y[orow] = (float)(ts * ((double)a + dr * (double)sx) + m * (double)sx);
+    }
+}
+
+// ---- fused decode + product on the matrix cores, M = 2..48 ---------------------------------------------------------------
+// A batch is 256 columns = four step pairs of every half-wave.  In LDS a pair's two symbols share a dword, so LDS
+// position kk of a batch holds column  64 * (kk / 64) + 32 * (kk & 1) + (kk % 64) / 2  of the batch; X is packed in the
+// same order, already in the A-operand layout: chunk (32 positions) x token tile x lane -> 8 halfs.
+constexpr int kRBatchCols = 256;
+constexpr int kRSymStride = kRBatchCols / 2 + 4;                           // dwords per row of a batch in LDS (padded)
+
+struct RPacked {
+    const uint4* hi; const uint4* lo;        // [chunks][NT][64]
+    const float* sx;                         // [16 NT] sum of the scaled row as the matrix cores see it
+    const int* kexp;                         // [16 NT] the row was scaled by 2^kexp
+};
+
+__device__ __forceinline__ int r_batch_col(int kk) { return 64 * (kk >> 6) + 32 * (kk & 1) + ((kk & 63) >> 1); }
+
+// one workgroup per (padded) row of X
+template <bool LO>
+__global__ void __launch_bounds__(256) r_pack_x_kernel(const void* __restrict__ X, int x_dtype, int M, int P, int NT,
+                                                       uint4* __restrict__ hi, uint4* __restrict__ lo, float* __restrict__ sx, int* __restrict__ kexp) {
+    __shared__ float s_max[256];
+    __shared__ double s_sum[256];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const bool valid = m < M;
+    float mx = 0.f;
+    if (valid) for (int col = tid; col < P; col += 256) {
+        const float v = __builtin_fabsf(load_as_f32(X, (int64_t)m * P + col, x_dtype));
+        if (v < __builtin_inff()) mx = __builtin_fmaxf(mx, v);
+    }
+    s_max[tid] = mx;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) { if (tid < w) s_max[tid] = __builtin_fmaxf(s_max[tid], s_max[tid + w]); __syncthreads(); }
+    mx = s_max[0];
+    int k = 0;
+    if (mx > 0.f) { int ex; (void)__builtin_frexpf(mx, &ex); k = 14 - ex; k = k < -100 ? -100 : (k > 100 ? 100 : k); }   // scaled max in [8192, 16384)
+    const float scale = __builtin_ldexpf(1.f, k);
+    const int Pp = (P + kRBatchCols - 1) / kRBatchCols * kRBatchCols;
+    const int nt = m >> 4, r16 = m & 15;
+    double sum = 0.0;
+    for (int g = tid; g < Pp / 8; g += 256) {                              // eight LDS positions = one lane's share of a chunk
+        const int chunk = g >> 2, kg = g & 3;
+        uint32_t h[4], l[4];
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
-            const float a = half_sum(acc[i]);
-            if (l32 == 0 && i < M && row_ok)
-                Y[(int64_t)i * c.Q + orow] = (float)(ts * ((double)a + dr * (double)sx[i]) + m * (double)sx[i]);
+        for (int j = 0; j < 8; ++j) {
+            const int kk = (chunk & 7) * 32 + kg * 8 + j;
+            const int col = (chunk >> 3) * kRBatchCols + r_batch_col(kk);
+            const float v = valid && col < P ? load_as_f32(X, (int64_t)m * P + col, x_dtype) * scale : 0.f;
+            const _Float16 vh = (_Float16)v;
+            const _Float16 vl = LO ? (_Float16)(v - (float)vh) : (_Float16)0.f;
+            sum += (double)(float)vh + (double)(float)vl;
+            const uint32_t bh = __builtin_bit_cast(uint16_t, vh), bl = __builtin_bit_cast(uint16_t, vl);
+            if (j & 1) { h[j >> 1] |= bh << 16; l[j >> 1] |= bl << 16; } else { h[j >> 1] = bh; l[j >> 1] = bl; }
         }
+        const int64_t at = ((int64_t)chunk * NT + nt) * 64 + kg * 16 + r16;
+        hi[at] = make_uint4(h[0], h[1], h[2], h[3]);
+        if (LO) lo[at] = make_uint4(l[0], l[1], l[2], l[3]);
+    }
+    s_sum[tid] = sum;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) { if (tid < w) s_sum[tid] += s_sum[tid + w]; __syncthreads(); }
+    if (tid == 0) { sx[m] = (float)s_sum[0]; kexp[m] = k; }
+}
+
+// fp16 bits (low half of the result) of an integer below 2048: exact
+__device__ __forceinline__ uint32_t u16_to_half_bits(uint32_t v) {
+    uint32_t r;
+    asm("v_cvt_f16_u16_e32 %0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+
+typedef _Float16 r_v8h_t __attribute__((ext_vector_type(8)));
+typedef float r_v4f_t __attribute__((ext_vector_type(4)));
+
+template <int NT, bool LO>
+__global__ void __launch_bounds__(kRThreads) r_mma_kernel(RCore c, RPacked xp, int M, float* __restrict__ Y, int T) {
+    __shared__ uint32_t st[4096];
+    __shared__ uint32_t ring[kRTiles][kRing];
+    __shared__ __align__(16) uint32_t sym[2][kRTiles][kRSymStride];
+    __shared__ float red[kRThreads / 64][NT][256];
+    __shared__ int s_row[kRTiles];
+    __shared__ float s_ts[kRTiles], s_min[kRTiles], s_dr[kRTiles];
+    const int lane = threadIdx.x & 63, l32 = lane & 31, half = lane >> 5, h8 = threadIdx.x >> 5, wave = threadIdx.x >> 6;
+    TileCtx t = block_setup(c, blockIdx.x, st, h8);
+    uint32_t* rg = ring[h8];
+    Walker z;
+    walk_init(z, rg, c, t.tile, l32);
+    t.room = c.n_words - 1 - (z.wp - c.words);
+    __syncthreads();
+    const int S = c.P >> 5;
+    const int n_batches = (c.P + kRBatchCols - 1) / kRBatchCols;
+    const int n16 = lane & 15, kg = lane >> 4;
+    int flip = 0;
+    for (int r = 0; r < T; ++r) {
+        const bool active = t.has && r < t.nr;                             // per half-wave
+        r_v4f_t acc[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[nt] = r_v4f_t{0.f, 0.f, 0.f, 0.f};
+        for (int b = 0; b < n_batches; ++b) {
+            // this wave's two chunks of the batch: the X operands are requested before the walk
+            uint4 xh[2][NT], xl[2][NT];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    const int64_t at = ((int64_t)(b * 8 + wave * 2 + j) * NT + nt) * 64 + lane;
+                    xh[j][nt] = xp.hi[at];
+                    if (LO) xl[j][nt] = xp.lo[at];
+                }
+            uint32_t* sb = sym[flip][h8] + l32;
+            const int pairs = (S - b * 8) >> 1;                            // step pairs left in the row: a short last batch ends in zeros
+            if (active) {
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    uint32_t out = 0;
+                    if (p < pairs) {                                       // uniform
+                        uint32_t s1, s2;
+                        walk_pair(z, st, rg, l32, half, t.room, s1, s2);
+                        out = __builtin_amdgcn_perm(u16_to_half_bits(s2), u16_to_half_bits(s1), 0x05040100u);
+                    }
+                    sb[p * 32] = out;
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < 4; ++p) sb[p * 32] = 0u;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint4 w = make_uint4(0, 0, 0, 0);
+                if (n16 < kRTiles) w = *reinterpret_cast<const uint4*>(&sym[flip][n16][(wave * 2 + j) * 16 + kg * 4]);
+                const r_v8h_t bop = __builtin_bit_cast(r_v8h_t, w);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(r_v8h_t, xh[j][nt]), bop, acc[nt], 0, 0, 0);
+                    if (LO) acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(r_v8h_t, xl[j][nt]), bop, acc[nt], 0, 0, 0);
+                }
+            }
+            flip ^= 1;
+        }
+        // the row is done: lane holds tokens 4 kg + i of tile row n16; add the four waves' column shares
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave][nt][lane * 4 + i] = acc[nt][i];
+        if (l32 == 0) {
+            const int orow = active ? c.perm[t.r0 + r] : -1;
+            const bool row_ok = orow >= 0 && orow < c.Q;
+            s_row[h8] = row_ok ? orow : -1;
+            s_ts[h8] = row_ok ? c.tau_s[orow] : 0.f;
+            s_min[h8] = row_ok ? c.min_s[orow] : 0.f;
+            s_dr[h8] = row_ok ? (float)c.drow[orow] : 0.f;
+        }
+        __syncthreads();
+        for (int o = threadIdx.x; o < 16 * NT * kRTiles; o += kRThreads) {
+            const int n = o & (kRTiles - 1), m = o >> 3, nt = m >> 4, m16 = m & 15;
+            const int orow = s_row[n];
+            if (orow < 0 || m >= M) continue;
+            const int at = (((m16 >> 2) * 16 + n) << 2) + (m16 & 3);
+            double a = 0.0;
+#pragma unroll
+            for (int w = 0; w < kRThreads / 64; ++w) a += (double)red[w][nt][at];
+            const double sx = (double)xp.sx[m];
+            const double v = (double)s_ts[n] * (a + (double)s_dr[n] * sx) + (double)s_min[n] * sx;
+            Y[(int64_t)m * c.Q + orow] = (float)__builtin_ldexp(v, -xp.kexp[m]);
+        }
+        // red and s_row are written again only after the next row's batch barriers, which every thread reaches after this loop
     }
 }
 
@@ -278,7 +407,8 @@ int check_core(const char* who, const qvb8r_core* k, RCore& c) {
     c.n_tiles = (int)k->n_tiles; c.n_blocks = (int)k->n_blocks; c.K = (int)k->n_classes; c.Q = (int)k->Q; c.P = (int)k->P;
     return 0;
 }
-int mb_for(int64_t M) { return M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16; }
+int64_t packed_cols(int64_t P) { return (P + kRBatchCols - 1) / kRBatchCols * kRBatchCols; }
+int64_t packed_plane_bytes(int64_t M, int64_t P) { return packed_cols(P) / 32 * ((M + 15) / 16) * 64 * 16; }
 }  // namespace
 
 extern "C" int qvb8r_decode(const qvb8r_core* core, int64_t max_tile_rows, int out_dtype, int64_t b0, int64_t nb, int64_t row_base,
@@ -303,37 +433,47 @@ extern "C" int qvb8r_decode(const qvb8r_core* core, int64_t max_tile_rows, int o
 }
 
 extern "C" int64_t qvb8r_gemv_workspace_bytes(int64_t M, int64_t P) {
-    if (M < 1 || M > 16 || P <= 0) return 0;
-    return (int64_t)mb_for(M) * P * 4;
+    if (M < 1 || M > 48 || P <= 0) return 0;
+    if (M == 1) return 16;                                                 // X is read in place
+    return 2 * packed_plane_bytes(M, P) + 2 * 48 * 4;                      // hi, lo, row sums, row exponents
 }
 
 extern "C" int qvb8r_gemv(const void* X, int x_dtype, int64_t M, const qvb8r_core* core, int64_t max_tile_rows, float* Y,
                           void* workspace, int64_t workspace_bytes, void* stream) {
     RCore c;
     if (int rc = check_core("qvb8r_gemv", core, c)) return rc;
-    if (M < 1 || M > 16) return host::fail(QVB8_ERR_ARG, "qvb8r_gemv: M=%lld outside 1..16", (long long)M);
+    if (M < 1 || M > 48) return host::fail(QVB8_ERR_ARG, "qvb8r_gemv: M=%lld outside 1..48", (long long)M);
     if (x_dtype < QVB8_F32 || x_dtype > QVB8_BF16) return host::fail(QVB8_ERR_ARG, "qvb8r_gemv: bad activation dtype");
     if (max_tile_rows < 1 || max_tile_rows > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8r_gemv: bad rows-per-tile bound");
     if (c.Q == 0 || c.n_blocks == 0) return QVB8_OK;
     if (!X || !Y) return host::fail(QVB8_ERR_ARG, "qvb8r_gemv: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((unsigned)c.n_blocks), block(kRThreads);
+    const int T = (int)max_tile_rows;
+    if (M == 1) {
+        if (x_dtype == QVB8_F32) hipLaunchKernelGGL(r_gemv_kernel<0>, grid, block, 0, s, c, X, Y, T);
+        else if (x_dtype == QVB8_F16) hipLaunchKernelGGL(r_gemv_kernel<1>, grid, block, 0, s, c, X, Y, T);
+        else hipLaunchKernelGGL(r_gemv_kernel<2>, grid, block, 0, s, c, X, Y, T);
+        return host::check_launch("qvb8r_gemv");
+    }
     const int64_t need = qvb8r_gemv_workspace_bytes(M, c.P);
     if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u))
         return host::fail(QVB8_ERR_WORKSPACE, "qvb8r_gemv: needs %lld bytes of 16-byte aligned workspace", (long long)need);
-    hipStream_t s = (hipStream_t)stream;
-    const int MB = mb_for(M);
-    float* Xt = (float*)workspace;
-    const int64_t n = (int64_t)c.P * MB;
-    hipLaunchKernelGGL(r_transpose_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, X, x_dtype, (int)M, c.P, MB, Xt);
-    if (int rc = host::check_launch("qvb8r_gemv transpose")) return rc;
-    dim3 grid((unsigned)c.n_blocks), block(kRThreads);
-    const int T = (int)max_tile_rows;
-    switch (MB) {
-        case 1: hipLaunchKernelGGL(r_gemv_kernel<1>, grid, block, 0, s, c, Xt, (int)M, Y, T); break;
-        case 2: hipLaunchKernelGGL(r_gemv_kernel<2>, grid, block, 0, s, c, Xt, (int)M, Y, T); break;
-        case 4: hipLaunchKernelGGL(r_gemv_kernel<4>, grid, block, 0, s, c, Xt, (int)M, Y, T); break;
-        case 8: hipLaunchKernelGGL(r_gemv_kernel<8>, grid, block, 0, s, c, Xt, (int)M, Y, T); break;
-        default: hipLaunchKernelGGL(r_gemv_kernel<16>, grid, block, 0, s, c, Xt, (int)M, Y, T); break;
-    }
+    const int NT = (int)((M + 15) / 16);
+    const int64_t plane = packed_plane_bytes(M, c.P);
+    uint8_t* ws = (uint8_t*)workspace;
+    RPacked xp;
+    uint4* hi = (uint4*)ws; uint4* lo = (uint4*)(ws + plane);
+    float* sx = (float*)(ws + 2 * plane); int* kexp = (int*)(ws + 2 * plane + 48 * 4);
+    xp.hi = hi; xp.lo = lo; xp.sx = sx; xp.kexp = kexp;
+    const bool split = x_dtype == QVB8_F32;                                // fp16 / bf16 values, scaled by a power of two, are exact in hi
+    if (split) hipLaunchKernelGGL(r_pack_x_kernel<true>, dim3(16 * NT), dim3(256), 0, s, X, x_dtype, (int)M, c.P, NT, hi, lo, sx, kexp);
+    else hipLaunchKernelGGL(r_pack_x_kernel<false>, dim3(16 * NT), dim3(256), 0, s, X, x_dtype, (int)M, c.P, NT, hi, lo, sx, kexp);
+    if (int rc = host::check_launch("qvb8r_gemv pack")) return rc;
+#define QVB8R_MMA(NT_) do { if (split) hipLaunchKernelGGL((r_mma_kernel<NT_, true>), grid, block, 0, s, c, xp, (int)M, Y, T); \
+                            else hipLaunchKernelGGL((r_mma_kernel<NT_, false>), grid, block, 0, s, c, xp, (int)M, Y, T); } while (0)
+    if (NT == 1) QVB8R_MMA(1); else if (NT == 2) QVB8R_MMA(2); else QVB8R_MMA(3);
+#undef QVB8R_MMA
     return host::check_launch("qvb8r_gemv");
 }
 

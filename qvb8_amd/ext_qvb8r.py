@@ -14,7 +14,7 @@ import torch
 
 from . import _lib
 
-MAX_M = 16
+MAX_M = 48
 _OUT = {0: torch.float16, 1: torch.bfloat16, 2: torch.float32}        # the reference's out_dtype codes of decode()
 _ABI_DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.int16: 3}
 
@@ -72,12 +72,12 @@ def gemv(X, words, off, states, tiles, blocks, tab, perm, mn, ts, drow, T=None):
 
 
 def multi(X, words, off, states, tiles, blocks, tab, perm, mn, ts, drow, T=None):
-    """M = 2..8 (here up to 16): X (M, P) fp32 or bf16 -> Y (M, Q) fp32 (qvb8r_cuda.cu:359-383)."""
+    """M = 2..8 (here up to 48): X (M, P) fp32, fp16 or bf16 -> Y (M, Q) fp32 (qvb8r_cuda.cu:359-383)."""
     return _product(X, (words, off, states, tiles, blocks, tab, perm, mn, ts, drow), T)
 
 
 def tc(X, words, off, states, tiles, blocks, tab, perm, mn, ts, drow, T):
-    """M = 9..16 (qvb8r_cuda.cu:385-396).  The same kernel as multi: the fp32 band value is multiplied, not its fp16
+    """M = 9..16 (here up to 48; qvb8r_cuda.cu:385-396).  The same kernel as multi: the fp32 band value is multiplied, not its fp16
     rounding, so the escape correction that goes with it is the fp32 one (esc_delta)."""
     return _product(X, (words, off, states, tiles, blocks, tab, perm, mn, ts, drow), T)
 

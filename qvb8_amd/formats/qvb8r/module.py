@@ -3,8 +3,9 @@
 Same constructor `(d, bias=None, device="cuda", path=None)` over the dict container.read returns, same buffer names and
 `from_packfile` / `dense` / `forward` as the reference's module (src/qv_band/formats/qvb8r/module.py:57-325).  Dispatch:
 
-    M <= 16        one fused walk + product (ext.multi), fp32 band value, escapes corrected after it (esc_delta)
-    17 .. 48 rows  equal passes of <= 16 rows (module.py:297-305)
+    M <= 48        one fused walk + product (ext.gemv / ext.multi; from two rows on the matrix cores), fp32 band value,
+                   escapes corrected after it (esc_delta); the reference splits 17..48 rows into passes of <= 16
+                   (module.py:297-305), here one walk serves them all
     more           dense restore in chunks of whole blocks (<= CHUNK_BYTES of fp16 / bf16 weight each) + library GEMMs
 """
 from __future__ import annotations
