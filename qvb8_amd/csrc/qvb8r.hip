@@ -210,26 +210,33 @@ __global__ void __launch_bounds__(kRThreads) r_gemv_kernel(RCore c, const void* 
 constexpr int kRBatchCols = 256;
 constexpr int kRSymStride = kRBatchCols / 2 + 4;                           // dwords per row of a batch in LDS (padded)
 
+constexpr int kRSlabCols = 1024;                                          // columns one workgroup of the packing kernel writes
+
 struct RPacked {
     const uint4* hi; const uint4* lo;        // [chunks][NT][64]
-    const float* sx;                         // [16 NT] sum of the scaled row as the matrix cores see it
+    const double* sums;                      // [16 NT][slabs] sum of the scaled row, per slab, as the matrix cores see it
     const int* kexp;                         // [16 NT] the row was scaled by 2^kexp
+    int slabs;
 };
 
 __device__ __forceinline__ int r_batch_col(int kk) { return 64 * (kk >> 6) + 32 * (kk & 1) + ((kk & 63) >> 1); }
 
-// one workgroup per (padded) row of X
-template <bool LO>
-__global__ void __launch_bounds__(256) r_pack_x_kernel(const void* __restrict__ X, int x_dtype, int M, int P, int NT,
-                                                       uint4* __restrict__ hi, uint4* __restrict__ lo, float* __restrict__ sx, int* __restrict__ kexp) {
+// Workgroup (m, slab): the largest finite |x| of row m (every slab of the row finds it again: the row is a few KB of
+// L2 hits), then this slab's columns scaled, split and laid out, and the slab's sum.
+template <int DT, bool LO>
+__global__ void __launch_bounds__(256) r_pack_x_kernel(const void* __restrict__ X, int M, int P, int NT,
+                                                       uint4* __restrict__ hi, uint4* __restrict__ lo, double* __restrict__ sums, int* __restrict__ kexp) {
     __shared__ float s_max[256];
     __shared__ double s_sum[256];
-    const int m = blockIdx.x, tid = threadIdx.x;
+    const int m = blockIdx.x, slab = blockIdx.y, tid = threadIdx.x;
     const bool valid = m < M;
     float mx = 0.f;
-    if (valid) for (int col = tid; col < P; col += 256) {
-        const float v = __builtin_fabsf(load_as_f32(X, (int64_t)m * P + col, x_dtype));
-        if (v < __builtin_inff()) mx = __builtin_fmaxf(mx, v);
+    if (valid) for (int c0 = tid * 8; c0 < P; c0 += 256 * 8) {            // P is a multiple of 128: whole groups of eight
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = __builtin_fabsf(load_as_f32<DT>(X, (int64_t)m * P + c0 + j));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mx = v[j] < __builtin_inff() ? __builtin_fmaxf(mx, v[j]) : mx;
     }
     s_max[tid] = mx;
     __syncthreads();
@@ -241,14 +248,15 @@ __global__ void __launch_bounds__(256) r_pack_x_kernel(const void* __restrict__ 
     const int Pp = (P + kRBatchCols - 1) / kRBatchCols * kRBatchCols;
     const int nt = m >> 4, r16 = m & 15;
     double sum = 0.0;
-    for (int g = tid; g < Pp / 8; g += 256) {                              // eight LDS positions = one lane's share of a chunk
+    const int g = slab * (kRSlabCols / 8) + tid;                            // eight LDS positions = one lane's share of a chunk
+    if (tid < kRSlabCols / 8 && g < Pp / 8) {
         const int chunk = g >> 2, kg = g & 3;
         uint32_t h[4], l[4];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int kk = (chunk & 7) * 32 + kg * 8 + j;
             const int col = (chunk >> 3) * kRBatchCols + r_batch_col(kk);
-            const float v = valid && col < P ? load_as_f32(X, (int64_t)m * P + col, x_dtype) * scale : 0.f;
+            const float v = valid && col < P ? load_as_f32<DT>(X, (int64_t)m * P + col) * scale : 0.f;
             const _Float16 vh = (_Float16)v;
             const _Float16 vl = LO ? (_Float16)(v - (float)vh) : (_Float16)0.f;
             sum += (double)(float)vh + (double)(float)vl;
@@ -262,7 +270,7 @@ __global__ void __launch_bounds__(256) r_pack_x_kernel(const void* __restrict__ 
     s_sum[tid] = sum;
     __syncthreads();
     for (int w = 128; w > 0; w >>= 1) { if (tid < w) s_sum[tid] += s_sum[tid + w]; __syncthreads(); }
-    if (tid == 0) { sx[m] = (float)s_sum[0]; kexp[m] = k; }
+    if (tid == 0) { sums[(int64_t)m * gridDim.y + slab] = s_sum[0]; if (slab == 0) kexp[m] = k; }
 }
 
 // fp16 bits (low half of the result) of an integer below 2048: exact
@@ -283,7 +291,13 @@ __global__ void __launch_bounds__(kRThreads) r_mma_kernel(RCore c, RPacked xp, i
     __shared__ float red[kRThreads / 64][NT][256];
     __shared__ int s_row[kRTiles];
     __shared__ float s_ts[kRTiles], s_min[kRTiles], s_dr[kRTiles];
+    __shared__ double s_sx[16 * NT];
     const int lane = threadIdx.x & 63, l32 = lane & 31, half = lane >> 5, h8 = threadIdx.x >> 5, wave = threadIdx.x >> 6;
+    if (threadIdx.x < 16 * NT) {
+        double a = 0.0;
+        for (int i = 0; i < xp.slabs; ++i) a += xp.sums[threadIdx.x * xp.slabs + i];
+        s_sx[threadIdx.x] = a;
+    }
     TileCtx t = block_setup(c, blockIdx.x, st, h8);
     uint32_t* rg = ring[h8];
     Walker z;
@@ -363,7 +377,7 @@ __global__ void __launch_bounds__(kRThreads) r_mma_kernel(RCore c, RPacked xp, i
             double a = 0.0;
 #pragma unroll
             for (int w = 0; w < kRThreads / 64; ++w) a += (double)red[w][nt][at];
-            const double sx = (double)xp.sx[m];
+            const double sx = s_sx[m];
             const double v = (double)s_ts[n] * (a + (double)s_dr[n] * sx) + (double)s_min[n] * sx;
             Y[(int64_t)m * c.Q + orow] = (float)__builtin_ldexp(v, -xp.kexp[m]);
         }
@@ -408,6 +422,7 @@ int check_core(const char* who, const qvb8r_core* k, RCore& c) {
     return 0;
 }
 int64_t packed_cols(int64_t P) { return (P + kRBatchCols - 1) / kRBatchCols * kRBatchCols; }
+int64_t packed_slabs(int64_t P) { return (packed_cols(P) + kRSlabCols - 1) / kRSlabCols; }
 int64_t packed_plane_bytes(int64_t M, int64_t P) { return packed_cols(P) / 32 * ((M + 15) / 16) * 64 * 16; }
 }  // namespace
 
@@ -435,7 +450,7 @@ extern "C" int qvb8r_decode(const qvb8r_core* core, int64_t max_tile_rows, int o
 extern "C" int64_t qvb8r_gemv_workspace_bytes(int64_t M, int64_t P) {
     if (M < 1 || M > 48 || P <= 0) return 0;
     if (M == 1) return 16;                                                 // X is read in place
-    return 2 * packed_plane_bytes(M, P) + 2 * 48 * 4;                      // hi, lo, row sums, row exponents
+    return 2 * packed_plane_bytes(M, P) + 48 * 8 * packed_slabs(P) + 48 * 4;   // hi, lo, slab sums, row exponents
 }
 
 extern "C" int qvb8r_gemv(const void* X, int x_dtype, int64_t M, const qvb8r_core* core, int64_t max_tile_rows, float* Y,
@@ -463,12 +478,15 @@ extern "C" int qvb8r_gemv(const void* X, int x_dtype, int64_t M, const qvb8r_cor
     const int64_t plane = packed_plane_bytes(M, c.P);
     uint8_t* ws = (uint8_t*)workspace;
     RPacked xp;
+    const int slabs = (int)packed_slabs(c.P);
     uint4* hi = (uint4*)ws; uint4* lo = (uint4*)(ws + plane);
-    float* sx = (float*)(ws + 2 * plane); int* kexp = (int*)(ws + 2 * plane + 48 * 4);
-    xp.hi = hi; xp.lo = lo; xp.sx = sx; xp.kexp = kexp;
+    double* sums = (double*)(ws + 2 * plane); int* kexp = (int*)(ws + 2 * plane + 48 * 8 * (int64_t)slabs);
+    xp.hi = hi; xp.lo = lo; xp.sums = sums; xp.kexp = kexp; xp.slabs = slabs;
     const bool split = x_dtype == QVB8_F32;                                // fp16 / bf16 values, scaled by a power of two, are exact in hi
-    if (split) hipLaunchKernelGGL(r_pack_x_kernel<true>, dim3(16 * NT), dim3(256), 0, s, X, x_dtype, (int)M, c.P, NT, hi, lo, sx, kexp);
-    else hipLaunchKernelGGL(r_pack_x_kernel<false>, dim3(16 * NT), dim3(256), 0, s, X, x_dtype, (int)M, c.P, NT, hi, lo, sx, kexp);
+    const dim3 pgrid(16 * NT, slabs);
+    if (split) hipLaunchKernelGGL((r_pack_x_kernel<0, true>), pgrid, dim3(256), 0, s, X, (int)M, c.P, NT, hi, lo, sums, kexp);
+    else if (x_dtype == QVB8_F16) hipLaunchKernelGGL((r_pack_x_kernel<1, false>), pgrid, dim3(256), 0, s, X, (int)M, c.P, NT, hi, lo, sums, kexp);
+    else hipLaunchKernelGGL((r_pack_x_kernel<2, false>), pgrid, dim3(256), 0, s, X, (int)M, c.P, NT, hi, lo, sums, kexp);
     if (int rc = host::check_launch("qvb8r_gemv pack")) return rc;
 #define QVB8R_MMA(NT_) do { if (split) hipLaunchKernelGGL((r_mma_kernel<NT_, true>), grid, block, 0, s, c, xp, (int)M, Y, T); \
                             else hipLaunchKernelGGL((r_mma_kernel<NT_, false>), grid, block, 0, s, c, xp, (int)M, Y, T); } while (0)
