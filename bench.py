@@ -262,8 +262,8 @@ def bench_qvb8r(args, dev):
 
 def bench_smallm(args, dev):
     """Config 3: the 9B projections with M = `--tokens` rows (draft-verify / prefill chunk), through QVBandLinearV8's own
-    dispatch: M <= 48 one fused decode + MFMA launch per projection group, 49..96 two passes, above that dense restore
-    to fp16 + library GEMM.  Reports GB/s on the packed bytes and TFLOP/s (2 M Q P per projection, decode ops not counted)."""
+    dispatch: M <= 48 the tile kernel (X in registers), 49..256 the workgroup-tiled decode + GEMM kernel (X staged in LDS,
+    ids decoded in registers), above that dense restore to fp16 + library GEMM.  Reports GB/s on the packed bytes and TFLOP/s (2 M Q P per projection, decode ops not counted)."""
     import torch
     layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse)
     M = args.tokens
@@ -282,8 +282,9 @@ def bench_smallm(args, dev):
     ms = max(ev_ms, wall_ms)
     gbs = step_bytes / (ms * 1e-3) / 1e9
     tflops = flops / (ms * 1e-3) / 1e12
-    path = "fused decode + MFMA (qvb8_mma)" if M <= 48 else "two fused passes" if M <= 96 else "fp16 restore + library GEMM"
-    bound = "hbm" if M <= 96 else "mfma"
+    path = ("fused decode + MFMA, X in registers (qvb8_mma, tile kernel)" if M <= 48 else
+            "fused decode + MFMA GEMM, X staged in LDS (qvb8_mma, workgroup-tiled kernel)" if M <= 256 else "fp16 restore + library GEMM")
+    bound = "hbm" if M <= 64 else "mfma"
     return {"metric": "small-M fused decode + GEMM: GB/s on packed bytes and TFLOP/s, 9B projections, 1 MI355X",
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

@@ -88,7 +88,7 @@ int qvb8_gemv(const void* X, int x_dtype, int64_t M,
               const int64_t* esc_idx, const float* esc_vals, int64_t n_esc,
               float* Y, void* workspace, int64_t workspace_bytes, void* stream);
 
-/* ---- fused decode + small-M GEMM on the matrix cores, M = 1..48 ------------------------------------------- */
+/* ---- fused decode + small-M GEMM on the matrix cores, M = 1..48 (and 49..256, see qvb8_mma) ---------------- */
 
 enum qvb8_mma_flags {
     QVB8_MMA_SATURATE_X = 1   /* bf16 X is narrowed as saturating_half does (clamp to +-65504, round to fp16, NaN kept) while
@@ -118,7 +118,8 @@ typedef struct qvb8_mma_layout {
     int32_t nbits[QVB8_MMA_MAX_CLASSES];
 } qvb8_mma_layout;
 
-/* Workspace qvb8_mma needs when it is called WITHOUT row records (it then builds them itself first). */
+/* Workspace qvb8_mma needs: for M <= 48 only when it is called WITHOUT row records (it then builds them itself first);
+ * for 49 <= M <= 256 always (narrowed activations, their sums per column range, partial results of the column ranges). */
 int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
 
 /* Y[m, q] = sum_c X[m, c] * value(q, c), fp32 accumulate on v_mfma 16x16x32, Y f32 (M, Q) row-major.
@@ -130,6 +131,10 @@ int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
  * perm, or NULL (then `workspace` must hold qvb8_mma_workspace_bytes).  `layout`: NULL, or the description of rows stored
  * in tile order (needs `rowinfo`).  Widths 4..8 on dword-aligned rows take the fast path; other rows are read element
  * by element.
+ * 49 <= M <= 256 runs a workgroup-tiled decode + GEMM (X staged in LDS, v_mfma 32x32x16, column ranges added in a fixed
+ * order): it needs `layout` with widths 4..8 (4..7 for bf16 operands), P % 256 == 0 and `workspace`; otherwise
+ * QVB8_ERR_UNSUPPORTED / QVB8_ERR_WORKSPACE.  The reference restores the weight and calls a library GEMM there
+ * (formats/qvb8/module.py:402-457).
  * Replaces: ext.mma_multi  qvb8_mma_multi_forward qvb8_cuda.cu:2566-2671 (kernels :2321-2441, escape fix
  * :2503-2548), and, through the Python module, the M <= 8 GEMV of :1059-1166 when P % 128 == 0. */
 int qvb8_mma(const void* X, int x_dtype, int64_t M,

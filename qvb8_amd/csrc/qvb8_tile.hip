@@ -27,6 +27,7 @@ typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
 typedef float v4f_t __attribute__((ext_vector_type(4)));
 typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
+typedef float v16f_t __attribute__((ext_vector_type(16)));
 
 constexpr int kTileRows = 16;
 constexpr int kStepCols = 128;          // columns one wave step covers (4 lane groups x 32 ids)
@@ -39,6 +40,9 @@ template <> struct Fmt<false> {          // fp16: 0x6400 | id == 1024 + id for i
     static __device__ __forceinline__ v4f_t mfma(const v4u_t& a, const v4u_t& b, const v4f_t& c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h_t, a), __builtin_bit_cast(v8h_t, b), c, 0, 0, 0);
     }
+    static __device__ __forceinline__ v16f_t mfma32(const v4u_t& a, const v4u_t& b, const v16f_t& c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, a), __builtin_bit_cast(v8h_t, b), c, 0, 0, 0);
+    }
     static __device__ __forceinline__ float to_f32(uint32_t h) { return f16_bits_to_f32(h); }
 };
 template <> struct Fmt<true> {           // bf16: 0x4300 | id == 128 + id for id < 128
@@ -47,6 +51,9 @@ template <> struct Fmt<true> {           // bf16: 0x4300 | id == 128 + id for id
     static constexpr int max_nb = 7;
     static __device__ __forceinline__ v4f_t mfma(const v4u_t& a, const v4u_t& b, const v4f_t& c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, a), __builtin_bit_cast(v8bf_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ v16f_t mfma32(const v4u_t& a, const v4u_t& b, const v16f_t& c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf_t, a), __builtin_bit_cast(v8bf_t, b), c, 0, 0, 0);
     }
     static __device__ __forceinline__ float to_f32(uint32_t h) { return bf16_bits_to_f32(h); }
 };
@@ -471,9 +478,212 @@ __global__ void __launch_bounds__(256) tile_fix_escapes_kernel(const uint16_t* _
     Y[(size_t)t * Q + q] += acc;
 }
 
+// ---- fused decode + GEMM, M = 49..256 ---------------------------------------------------------------------------------
+// For this many rows of X the activations no longer fit a wave's registers, and every byte of X must serve many weight
+// rows: a workgroup (4 waves) takes 256 weight rows of ONE width x TMK = 32 * MT rows of X x one range of columns.  X goes
+// through LDS in stages of 128 columns (double-buffered); the weights never touch LDS: lane (n = l % 32, kh = l / 32) of a
+// wave owns the 32 consecutive ids of row n at columns 64 * step + 32 * kh, fetched as two 16-byte loads and decoded
+// into the B operands of four v_mfma_f32_32x32x16 (the K order inside a step is a permutation that X follows).  The id
+// registers form a ring of four steps: a step's registers are asked for the step four ahead as soon as it has been
+// decoded, so about 256 columns of every row of the workgroup are in flight at any time.  A wave keeps 2 row tiles x MT
+// token tiles of 32 x 32 sums (every X operand read from LDS feeds two MFMAs).  The main loop has no branch: a column
+// range is a whole number of 256-column groups, and requests past its end read its last step again.
+// A pass over X beforehand (gemm_prep_kernel) narrows bf16 activations once (XC) and adds up each row of X per column
+// range: the sums remove the bias of `bias + id` and carry min_s.  Column ranges (blockIdx.z) write partial results that
+// a last kernel adds in order.  Needs rows stored in width order (the layout of qvb8_mma), widths 4..8 (bf16 operands:
+// 4..7) and P % 256 == 0.
+constexpr int kGemmRows = 256, kGemmWaveRows = 64, kGemmStageCols = 128;
+constexpr int kGemmXStride = kGemmStageCols * 2 + 16;              // bytes per row of X of one stage in LDS (padded: conflict-free 16-byte reads)
+
+struct GemmArgs {
+    const uint16_t* X;             // (M, P) in the operand format
+    const uint8_t* ids; const uint4* fin;
+    const float* sx;               // [splits][M] sums of X over each column range
+    float* out;                    // Y (one column range) or the partial results [splits][M][Q]
+    int M, Q, P;
+    int stages_per_split;          // even
+    int first1, first2;            // positions where the second and the third width start (Q when there is none)
+    int blocks1, blocks2;          // row blocks before the second / the third width (blocks of 256 positions from a width's first)
+    uint32_t widths;               // nb0 | nb1 << 8 | nb2 << 16
+};
+
+// grid (M, splits): sx[z][m] = sum of row m of X over column range z, as the operands see it; XC: X16[m] = the row narrowed
+template <bool BF, bool XC>
+__global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t* __restrict__ X, int M, int P, int cols_per_split,
+                                                        uint16_t* __restrict__ X16, float* __restrict__ sx) {
+    __shared__ float red[4];
+    const int m = blockIdx.x, z = blockIdx.y, tid = threadIdx.x;
+    const int c_begin = z * cols_per_split, c_end = min(P, c_begin + cols_per_split);
+    float part = 0.f;
+    for (int c = c_begin + 8 * tid; c < c_end; c += 8 * 256) {
+        const uint4 v = *reinterpret_cast<const uint4*>(X + (size_t)m * P + c);
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            w[k] = XIn<BF, XC>::pair(w[k]);
+            part += Fmt<BF>::to_f32(w[k] & 0xFFFFu) + Fmt<BF>::to_f32(w[k] >> 16);
+        }
+        if constexpr (XC) *reinterpret_cast<uint4*>(X16 + (size_t)m * P + c) = uint4{w[0], w[1], w[2], w[3]};
+    }
+    part = wave_sum(part);
+    if ((tid & 63) == 0) red[tid >> 6] = part;
+    __syncthreads();
+    if (tid == 0) sx[(size_t)z * M + m] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// The workgroup's rows are positions [pos0, pos0 + 256) of a run of width NB that ends at pos_end and starts at byte
+// run_byte0 (position run_first) of the ids buffer.
+template <int MT, bool BF, int NB>
+__device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_end, int run_first, uint64_t run_byte0, unsigned char* smem) {
+    using F = Fmt<BF>;
+    constexpr int TMK = 32 * MT;                   // rows of X per workgroup
+    constexpr int XL = TMK * 16 / 256;             // 16-byte pieces of a stage per thread
+    unsigned char* xs = smem;                                              // [2][TMK][kGemmXStride]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, kh = lane >> 5;
+    const int tok0 = (int)blockIdx.y * TMK;
+    const int s_begin = (int)blockIdx.z * a.stages_per_split;
+    const int s_end = min(a.P / kGemmStageCols, s_begin + a.stages_per_split);
+    const int u_begin = 2 * s_begin, u_end = 2 * s_end;                    // 64-column steps; u_end - u_begin is a multiple of 4
+    if (u_begin >= u_end) return;
+
+    // ---- this lane's two rows; a position past the run reads the run's last row (finite operands, result not stored) ----
+    const uint8_t* row_ptr[2]; int row_pos[2]; bool row_ok[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const int pos = pos0 + wave * kGemmWaveRows + rt * 32 + n;
+        row_ok[rt] = pos < pos_end;
+        row_pos[rt] = row_ok[rt] ? pos : pos_end - 1;
+        row_ptr[rt] = a.ids + run_byte0 + (uint64_t)(row_pos[rt] - run_first) * ((uint64_t)a.P * NB / 8) + (uint32_t)kh * (4u * NB);
+    }
+    uint4 raw[4][2][2];                            // [step % 4][row tile][first / last four dwords]
+    const uint8_t* const rp0 = row_ptr[0];
+    const uint8_t* const rp1 = row_ptr[1];
+    auto request_ids = [u_end, rp0, rp1](int u, uint4 (&w)[2][2]) {
+        const uint32_t off = (uint32_t)min(u, u_end - 1) * (8u * NB);      // a step is 64 columns = 8 NB bytes of a row
+        w[0][0] = *reinterpret_cast<const uint4*>(rp0 + off);
+        w[0][1] = *reinterpret_cast<const uint4*>(rp0 + off + 4u * (NB - 4u));
+        w[1][0] = *reinterpret_cast<const uint4*>(rp1 + off);
+        w[1][1] = *reinterpret_cast<const uint4*>(rp1 + off + 4u * (NB - 4u));
+    };
+    // ---- X: thread tid stages piece tid % 16 (8 columns) of rows tid / 16 + 16 * i; rows past M read row M - 1 (not stored at the end) ----
+    const int xch = tid & 15, xrow = tid >> 4;
+    const uint16_t* const x_base = a.X + 8 * xch;
+    const int M = a.M, P = a.P;
+    v4u_t xg[XL];
+    auto request_x = [=](int st, v4u_t (&g)[XL]) {
+        const uint32_t c = (uint32_t)min(st, s_end - 1) * kGemmStageCols;
+#pragma unroll
+        for (int i = 0; i < XL; ++i) g[i] = *reinterpret_cast<const v4u_t*>(x_base + (size_t)min(tok0 + xrow + 16 * i, M - 1) * P + c);
+    };
+    auto store_x = [=](int buf, const v4u_t (&g)[XL]) {
+#pragma unroll
+        for (int i = 0; i < XL; ++i)
+            *reinterpret_cast<v4u_t*>(xs + ((size_t)buf * TMK + xrow + 16 * i) * kGemmXStride + 16 * xch) = g[i];
+    };
+
+    v16f_t acc[2][MT];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[rt][mt][i] = 0.f;
+
+    request_x(s_begin, xg);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) request_ids(u_begin + k, raw[k]);
+    store_x(0, xg);
+    __syncthreads();
+    for (int u0 = u_begin; u0 < u_end; u0 += 4) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int h = k & 1, buf = k >> 1;
+            if (h == 0) request_x((u0 >> 1) + buf + 1, xg);
+            v4u_t b[2][4];
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) decode_slice<NB, BF>(raw[k][rt][0], raw[k][rt][1], b[rt]);
+            request_ids(u0 + k + 4, raw[k]);
+            __builtin_amdgcn_sched_barrier(0);                             // the requests stay ahead of the products
+            const unsigned char* xb = xs + (size_t)buf * TMK * kGemmXStride + (size_t)n * kGemmXStride + 2 * (64 * h + 32 * kh);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const uint4 v = *reinterpret_cast<const uint4*>(xb + (size_t)(32 * mt) * kGemmXStride + 16 * j);
+                    const v4u_t av = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int rt = 0; rt < 2; ++rt) acc[rt][mt] = F::mfma32(av, b[rt][j], acc[rt][mt]);
+                }
+            if (h == 1) {
+                store_x(buf ^ 1, xg);
+                __syncthreads();
+            }
+        }
+    }
+    // ---- the end: lane holds, for row n of each row tile, tokens 32 mt + 8 (i / 4) + 4 kh + i % 4 ----
+    float* sxs = reinterpret_cast<float*>(smem);                           // the X stages are no longer read (barrier above)
+    if (tid < TMK) sxs[tid] = tok0 + tid < a.M ? a.sx[(size_t)blockIdx.z * a.M + tok0 + tid] : 0.f;
+    __syncthreads();
+    float* out = a.out + (size_t)blockIdx.z * (size_t)a.M * (size_t)a.Q;
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        if (!row_ok[rt]) continue;
+        const uint4 f = a.fin[row_pos[rt]];
+        if (f.z >= (uint32_t)a.Q) continue;
+        const double ts = (double)__uint_as_float(f.x), mn = (double)__uint_as_float(f.y);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int tl = 32 * mt + 8 * (i >> 2) + 4 * kh + (i & 3);
+                const int t = tok0 + tl;
+                if (t < a.M) {
+                    const float sx = sxs[tl];
+                    const float d = __builtin_fmaf(-F::bias, sx, acc[rt][mt][i]);
+                    out[(size_t)t * a.Q + f.z] = (float)(ts * (double)d + mn * (double)sx);
+                }
+            }
+    }
+}
+
+template <int MT, bool BF>
+__global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    // which run of equal widths this workgroup's 256 positions belong to
+    const int bx = (int)blockIdx.x;
+    const int c = (bx >= a.blocks1 ? 1 : 0) + (bx >= a.blocks2 ? 1 : 0);
+    const uint32_t nb0 = a.widths & 255u, nb1 = (a.widths >> 8) & 255u, nb2 = (a.widths >> 16) & 255u;
+    const uint64_t row0 = (uint64_t)a.P * nb0 / 8, row1 = (uint64_t)a.P * nb1 / 8;
+    const int run_first = c == 0 ? 0 : c == 1 ? a.first1 : a.first2;
+    const int run_end = c == 0 ? a.first1 : c == 1 ? a.first2 : a.Q;
+    const uint64_t byte0 = c == 0 ? 0 : c == 1 ? (uint64_t)a.first1 * row0 : (uint64_t)a.first1 * row0 + (uint64_t)(a.first2 - a.first1) * row1;
+    const int pos0 = run_first + (bx - (c == 0 ? 0 : c == 1 ? a.blocks1 : a.blocks2)) * kGemmRows;
+    if (pos0 >= run_end) return;
+    switch (c == 0 ? nb0 : c == 1 ? nb1 : nb2) {
+        case 4: gemm_run<MT, BF, 4>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 5: gemm_run<MT, BF, 5>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 6: gemm_run<MT, BF, 6>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 7: gemm_run<MT, BF, 7>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 8: if constexpr (!BF) gemm_run<MT, BF, 8>(a, pos0, run_end, run_first, byte0, smem); break;
+        default: break;
+    }
+}
+
+// Y = sum of the column ranges' partial results, in ascending order
+__global__ void __launch_bounds__(256) gemm_reduce_kernel(const float* __restrict__ part, float* __restrict__ Y, int64_t n, int splits) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = part[i];
+    for (int s = 1; s < splits; ++s) v += part[(int64_t)s * n + i];
+    Y[i] = v;
+}
+
 }  // namespace qvb8
 
 using namespace qvb8;
+
+extern "C" int64_t qvb8_mma_rowinfo_bytes(int64_t Q);
 
 namespace {
 struct TilePlan { int W, G, panels, TW, threads; size_t lds; unsigned blocks; };
@@ -530,6 +740,52 @@ int launch_tile(TileArgs& a, hipStream_t s) {
                        (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16) | ((uint32_t)a.n_classes << 24));
     return host::check_launch("qvb8_mma");
 }
+struct GemmPlan {
+    int MT, tok_blocks, row_blocks, splits, stages_per_split;
+    size_t lds;
+    int64_t x16_at, sx_at, part_at, bytes;      // workspace layout, bytes from its start (after the row records' place)
+};
+int64_t align256i(int64_t n) { return (n + 255) & ~(int64_t)255; }
+
+// Column ranges of whole 256-column groups, enough of them for about one workgroup per CU (row blocks counted as
+// ceil(Q / 256): up to two more exist when the rows have several widths).
+GemmPlan plan_gemm(int64_t M, int64_t Q, int64_t P) {
+    GemmPlan g;
+    g.MT = M <= 64 ? 2 : 4;
+    const int TMK = 32 * g.MT;
+    g.tok_blocks = (int)((M + TMK - 1) / TMK);
+    g.row_blocks = (int)((Q + kGemmRows - 1) / kGemmRows);
+    const int64_t groups = P / (2 * kGemmStageCols);
+    const int64_t base = (int64_t)g.tok_blocks * g.row_blocks;
+    const int64_t target = (int64_t)host::env_int("QVB8_GEMM_WGS_PER_CU", 1) * host::device_cus();
+    int64_t splits = (target + base - 1) / base;
+    if (splits > groups) splits = groups;
+    if (splits > 16) splits = 16;
+    if (splits < 1) splits = 1;
+    const int64_t groups_per_split = (groups + splits - 1) / splits;
+    g.stages_per_split = (int)(2 * groups_per_split);
+    g.splits = (int)((groups + groups_per_split - 1) / groups_per_split);
+    g.lds = (size_t)2 * TMK * kGemmXStride;
+    g.x16_at = align256i(qvb8_mma_rowinfo_bytes(Q));
+    g.sx_at = g.x16_at + align256i(M * P * 2);
+    g.part_at = g.sx_at + align256i((int64_t)g.splits * M * 4);
+    g.bytes = g.part_at + (g.splits > 1 ? (int64_t)g.splits * M * Q * 4 : 0);
+    return g;
+}
+
+template <int MT, bool BF>
+int launch_gemm(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_t s) {
+    static bool attr[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: no current device");
+    if (!attr[dev]) {
+        if (hipFuncSetAttribute((const void*)gemm_kernel<MT, BF>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds) != hipSuccess)
+            return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: cannot raise the kernel's LDS limit");
+        attr[dev] = true;
+    }
+    hipLaunchKernelGGL((gemm_kernel<MT, BF>), dim3((unsigned)row_blocks, (unsigned)g.tok_blocks, (unsigned)g.splits), dim3(256), g.lds, s, a);
+    return host::check_launch("qvb8_mma");
+}
 }  // namespace
 
 extern "C" int64_t qvb8_mma_rowinfo_bytes(int64_t Q) { return Q > 0 ? (int64_t)(rowinfo_loc_words(Q) * 8 + (size_t)Q * 16) : 0; }
@@ -546,7 +802,7 @@ extern "C" int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, co
 }
 
 extern "C" int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P) {
-    (void)M; (void)P;
+    if (M > 48 && M <= 256 && Q > 0 && P > 0 && (P % (2 * kGemmStageCols)) == 0) return plan_gemm(M, Q, P).bytes;
     return qvb8_mma_rowinfo_bytes(Q);
 }
 
@@ -557,7 +813,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
                         const int32_t* perm, const uint64_t* rowinfo, const qvb8_mma_layout* layout, int flags, float* Y,
                         void* workspace, int64_t workspace_bytes, void* stream) {
     if (Q < 0 || P < 0 || Q > 0x7fffffff || P > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8_mma: Q or P out of range");
-    if (M < 1 || M > 48) return host::fail(QVB8_ERR_ARG, "qvb8 mma-multi: M=%lld outside 1..48", (long long)M);
+    if (M < 1 || M > 256) return host::fail(QVB8_ERR_ARG, "qvb8 mma-multi: M=%lld outside 1..256", (long long)M);
     if (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16) return host::fail(QVB8_ERR_ARG, "qvb8_mma: X must be fp16 or bf16 (narrow fp32 activations with qvb8_sat_half first)");
     if ((P % kStepCols) != 0 || (reinterpret_cast<uintptr_t>(ids) & 3u) != 0)
         return host::fail(QVB8_ERR_ARG, "qvb8 mma-multi: needs P%%128==0 and 4-byte-aligned ids");
@@ -597,12 +853,51 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     // mode 0: fp16 X, fp16 operands; 1: bf16 X narrowed to saturated fp16 on the way in, fp16 operands; 2: bf16 operands
     const int mode = x_dtype == QVB8_F16 ? 0 : (flags & QVB8_MMA_SATURATE_X) ? 1 : 2;
     int rc;
+    if (M > 48) {
+        // many rows of X: the workgroup-tiled kernel.  It addresses rows arithmetically and decodes whole slices only.
+        if (!layout) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: M > 48 needs rows stored in width order (a row layout)");
+        if ((P % (2 * kGemmStageCols)) != 0) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: M > 48 needs P %% 256 == 0");
+        for (int c = 0; c < a.n_classes; ++c)
+            if (a.nb[c] < 4 || a.nb[c] > (mode == 2 ? 7 : 8))
+                return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: M > 48 needs widths 4..8 (4..7 on bf16 operands), found %d", a.nb[c]);
+        const GemmPlan g = plan_gemm(M, Q, P);
+        if (!workspace || workspace_bytes < g.bytes || (reinterpret_cast<uintptr_t>(workspace) & 15u))
+            return host::fail(QVB8_ERR_WORKSPACE, "qvb8_mma: M=%lld needs %lld bytes of 16-byte aligned workspace", (long long)M, (long long)g.bytes);
+        unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
+        uint16_t* x16 = reinterpret_cast<uint16_t*>(ws + g.x16_at);
+        float* sx = reinterpret_cast<float*>(ws + g.sx_at);
+        float* out = g.splits > 1 ? reinterpret_cast<float*>(ws + g.part_at) : Y;
+        const int cols_per_split = g.stages_per_split * kGemmStageCols;
+        const dim3 pgrid((unsigned)M, (unsigned)g.splits);
+        if (mode == 0) hipLaunchKernelGGL((gemm_prep_kernel<false, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx);
+        else if (mode == 1) hipLaunchKernelGGL((gemm_prep_kernel<false, true>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx);
+        else hipLaunchKernelGGL((gemm_prep_kernel<true, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx);
+        if (int rc2 = host::check_launch("qvb8_mma activations")) return rc2;
+        GemmArgs ga;
+        ga.X = mode == 1 ? x16 : a.X; ga.ids = ids; ga.fin = a.fin; ga.sx = sx; ga.out = out;
+        ga.M = (int)M; ga.Q = (int)Q; ga.P = (int)P; ga.stages_per_split = g.stages_per_split;
+        ga.first1 = a.first1; ga.first2 = a.first2;
+        const int rows0 = a.first1, rows1 = a.first2 - a.first1, rows2 = (int)Q - a.first2;
+        ga.blocks1 = (rows0 + kGemmRows - 1) / kGemmRows;
+        ga.blocks2 = ga.blocks1 + (rows1 + kGemmRows - 1) / kGemmRows;
+        const int row_blocks = ga.blocks2 + (rows2 + kGemmRows - 1) / kGemmRows;
+        ga.widths = (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16);
+        if (mode == 2) rc = g.MT == 2 ? launch_gemm<2, true>(ga, g, row_blocks, s) : launch_gemm<4, true>(ga, g, row_blocks, s);
+        else rc = g.MT == 2 ? launch_gemm<2, false>(ga, g, row_blocks, s) : launch_gemm<4, false>(ga, g, row_blocks, s);
+        if (rc) return rc;
+        if (g.splits > 1) {
+            const int64_t n = M * Q;
+            hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, out, Y, n, g.splits);
+            if (int rc2 = host::check_launch("qvb8_mma reduce")) return rc2;
+        }
+    } else {
 #define QVB8_TILE_LAUNCH(NT_, T_) (mode == 0 ? launch_tile<NT_, T_, false, false>(a, s) : mode == 1 ? launch_tile<NT_, T_, false, true>(a, s) : launch_tile<NT_, T_, true, false>(a, s))
     if (M <= 16) rc = QVB8_TILE_LAUNCH(1, 4);
     else if (M <= 32) rc = QVB8_TILE_LAUNCH(2, 2);
     else rc = QVB8_TILE_LAUNCH(3, 2);
 #undef QVB8_TILE_LAUNCH
-    if (rc) return rc;
+        if (rc) return rc;
+    }
     if (n_esc > 0) {
         dim3 grid((unsigned)((n_esc + 255) / 256), (unsigned)M);
 #define QVB8_FIX_ARGS grid, dim3(256), 0, s, (const uint16_t*)X, (int)M, ids, ids_bytes, min_s, tau_s, nbits, bit_off, esc_idx, esc_vals, n_esc, Y, (int)Q, (int)P

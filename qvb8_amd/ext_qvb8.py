@@ -146,6 +146,7 @@ def gemv(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
 
 
 MMA_MAX_M = 48
+MMA_GEMM_MAX_M = 256          # with a row layout (rows stored in width order, widths 4..8): the workgroup-tiled kernel
 MMA_SATURATE_X = 1
 
 
@@ -214,7 +215,8 @@ def sort_rows_by_width(ids, row_nbits, row_bit_off, P, perm):
 
 def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm=None, saturate=True,
               rowinfo=None, layout=None):
-    """Matrix-core path for 1 <= M <= 48 and P % 128 == 0: X (fp16 or bf16) times the fp32 band value, fp32 (M, Q).
+    """Matrix-core path for P % 128 == 0: X (fp16 or bf16) times the fp32 band value, fp32 (M, Q).  1 <= M <= 48 always;
+    49 <= M <= 256 (the workgroup-tiled decode + GEMM kernel) when `layout` is given and its widths are 4..8.
     `perm` (int32, position -> row) groups rows of equal width into tiles; `rowinfo` = mma_prepare(...) for the
     same perm (built on the fly when absent); `layout` = the third result of sort_rows_by_width for a pack whose rows were
     copied into that order (needs `rowinfo`).  `saturate` (bf16 X only): X is narrowed like saturating_half while it
@@ -227,8 +229,8 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
     if X.dim() != 2 or X.shape[1] != int(P):
         raise RuntimeError(f"X must be (M, {int(P)})")
     M = X.shape[0]
-    if not 1 <= M <= MMA_MAX_M:
-        raise RuntimeError(f"qvb8 mma-multi: M={M} outside 1..{MMA_MAX_M}")
+    if not 1 <= M <= (MMA_GEMM_MAX_M if layout is not None else MMA_MAX_M):
+        raise RuntimeError(f"qvb8 mma-multi: M={M} outside 1..{MMA_GEMM_MAX_M if layout is not None else MMA_MAX_M}")
     if int(P) % 128 != 0 or ids.data_ptr() % 4 != 0:
         raise RuntimeError("qvb8 mma-multi: needs P%128==0 and 4-byte-aligned ids")
     if X.dtype not in (torch.float16, torch.bfloat16):
@@ -249,8 +251,8 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
         Y = torch.empty((M, Q), dtype=torch.float32, device=Xc.device)
         ei = esc_idx.contiguous() if n_esc else None
         ev = esc_vals.contiguous() if n_esc else None
-        ws = None if rowinfo is not None else torch.empty(lib.qvb8_mma_workspace_bytes(M, Q, int(P)) // 8,
-                                                          dtype=torch.int64, device=Xc.device)
+        ws = None if (rowinfo is not None and M <= MMA_MAX_M) else \
+            torch.empty((lib.qvb8_mma_workspace_bytes(M, Q, int(P)) + 7) // 8, dtype=torch.int64, device=Xc.device)
         _lib._check(lib.qvb8_mma(_lib.ptr(Xc), _lib.dtype_code(Xc.dtype), M, _lib.ptr(ids), ids.numel(),
                                  _lib.ptr(min_s), _lib.ptr(tau_s), _lib.ptr(row_nbits), _lib.ptr(row_bit_off),
                                  Q, int(P), _lib.ptr(ei), _lib.ptr(ev), n_esc, _lib.ptr(perm),

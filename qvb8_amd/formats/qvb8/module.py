@@ -12,7 +12,10 @@ Dispatch on the row count M of the flattened input (the reference's: module.py:3
                             reference multiplies) -- in registers for bf16, so decode (M = 1) is ONE launch;
                             a bf16-certified pack with bf16 x multiplies bf16 operands (the reference's bf16 mode).
                             The band value is the un-narrowed fp32 one, as in the reference's GEMV.
-    49 .. 96 rows           equal passes of <= 48 rows (module.py:393-400)
+    49 .. 256 rows          the workgroup-tiled decode + GEMM kernel (same entry point) when the rows were copied into
+                            width order and all widths are 4..8 (4..7 in bf16 mode): X staged in LDS, ids decoded in
+                            registers, no dense weight written
+    49 .. 96 rows otherwise equal passes of <= 48 rows (module.py:393-400)
     M <= 8 otherwise        GEMV (ext.gemv_multi)
     else                    dense restore (fp16, or bf16 when bf16_gemm and certified) + one library GEMM
 """
@@ -218,6 +221,14 @@ class QVBandLinearV8(nn.Module):
         self._mma_cache = order
         return order
 
+    def _gemm_ok(self, layout, bf16_mode: bool) -> bool:
+        """Whether the workgroup-tiled kernel (49..256 rows) can read this weight: rows stored in width order, every
+        width one the sliced decode handles, whole 256-column groups."""
+        if layout is None or self.in_features % 256 != 0:
+            return False
+        top = 7 if bf16_mode else 8
+        return all(4 <= int(layout.nbits[c]) <= top for c in range(int(layout.n_classes)))
+
     # ---- forward -----------------------------------------------------------------------------------------------
 
     def _finish(self, y, orig, out_dtype):
@@ -250,12 +261,15 @@ class QVBandLinearV8(nn.Module):
             raise fp16_missing_error(getattr(self, "_where", "QVBandLinearV8"))
         ei, ev = (self.esc_idx_bf16, self.esc_vals_bf16) if bf16_mode else (self.esc_idx, self.esc_vals)
 
-        order = self._mma_order() if M <= _MMA_SPLIT_MAX else None
-        if order is not None and M > _MMA_MAX_M:
-            n = -(-M // _MMA_MAX_M)
-            step = -(-M // n)
-            return torch.cat([self.forward(xk[i:i + step]) for i in range(0, M, step)]) \
-                .reshape(*orig[:-1], self.out_features).to(out_dtype)
+        order = self._mma_order() if M <= max(_MMA_SPLIT_MAX, ext.MMA_GEMM_MAX_M) else None
+        if order is not None and M > _MMA_MAX_M and not self._gemm_ok(order[2], bf16_mode):
+            if M > _MMA_SPLIT_MAX:
+                order = None                                        # dense restore + library GEMM below
+            else:
+                n = -(-M // _MMA_MAX_M)
+                step = -(-M // n)
+                return torch.cat([self.forward(xk[i:i + step]) for i in range(0, M, step)]) \
+                    .reshape(*orig[:-1], self.out_features).to(out_dtype)
         if order is not None:
             perm, rowinfo, layout = order
             xm = xk if xk.dtype in (torch.float16, torch.bfloat16) else ext.saturating_half(xk)

@@ -78,9 +78,12 @@ def test_bf16_certified_pack_modes():
     x = torch.randn(16, 1024, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).to(DEV)
     ref, Wr, xs = _ref(enc, x, saturate=False, bf16_table=True)
     _close(lin(x), ref, Wr, xs, torch.bfloat16)             # bf16 operands, bf16 escape table
-    xl = torch.randn(128, 1024, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(DEV)
+    xm = torch.randn(128, 1024, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(DEV)
+    ref, Wr, xs = _ref(enc, xm, saturate=False, bf16_table=True)
+    _close(lin(xm), ref, Wr, xs, torch.bfloat16)            # 49..256 rows: still the fused path on bf16 operands
+    xl = torch.randn(300, 1024, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16).to(DEV)
     ref, Wr, xs = _ref(enc, xl, saturate=False, bf16_table=True, narrow="bf16")
-    _close(lin(xl), ref, Wr, xs, torch.bfloat16)            # M > 96: bf16 restore + one bf16 GEMM
+    _close(lin(xl), ref, Wr, xs, torch.bfloat16)            # more rows: bf16 restore + one bf16 GEMM
     rep = footprint_report(lin)
     assert rep["linears"] == 1 and rep["params"] == 128 * 1024 and rep["bytes_per_param"] < 1.2
 

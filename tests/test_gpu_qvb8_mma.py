@@ -127,3 +127,78 @@ def test_mma_bf16_activations_narrowed_on_load(M):
     xn[0, 11] = float("nan")
     yn = ext.mma_tiles(xn, *H.pack_args(enc), perm=perm, saturate=True)
     assert torch.isnan(yn[0]).all() and (M == 1 or not torch.isnan(yn[1:]).any())
+
+
+# ---- 49..256 rows of X: the workgroup-tiled decode + GEMM kernel behind the same entry point ------------------------------
+
+def _sorted_pack(d):
+    """Device arguments of a hand-made pack with its rows copied into width order + row records + layout."""
+    a = H.to_device_args(d, DEV)
+    ids, min_s, nbits, bit_off, P, tau_s, ei, ev = a
+    perm = _perm_by_width(nbits)
+    srt = ext.sort_rows_by_width(ids, nbits, bit_off, P, perm)
+    assert srt is not None
+    ids, bit_off, layout = srt
+    rowinfo = ext.mma_prepare(nbits, bit_off, tau_s, min_s, P, ids.numel(), perm)
+    return (ids, min_s, nbits, bit_off, P, tau_s, ei, ev), perm, rowinfo, layout
+
+
+@pytest.mark.parametrize("M", [49, 64, 65, 100, 128, 129, 256])
+@pytest.mark.parametrize("mode", ["fp16", "bf16_saturated", "bf16_operands"])
+def test_gemm_many_rows(M, mode):
+    """Three widths in one weight (each run of equal widths fills only part of its 256-row block), an odd number of
+    256-column groups (uneven column ranges), token counts on both sides of the 64- and 128-row blocks."""
+    Q, P = 300, 768
+    widths = [7, 6, 5] if mode == "bf16_operands" else [8, 7, 4]
+    d = H.mixed_width_pack(Q, P, widths, seed=M)
+    d["tau_s"] = d["tau_s"] * (1.0 / 64)
+    args, perm, rowinfo, layout = _sorted_pack(d)
+    dtype = torch.float16 if mode == "fp16" else torch.bfloat16
+    x = _x(M, P, dtype, M)
+    if mode == "bf16_saturated":
+        x[0, 3] = 1.0e5                                                      # narrowed to 65504 on the way into LDS
+    y = ext.mma_tiles(x, *args, perm=perm, saturate=mode != "bf16_operands", rowinfo=rowinfo, layout=layout)
+    _check(d, None, x, y, saturate_ref=mode == "bf16_saturated")
+    # against the 16-row tile kernel on the same rows: only the order of the fp32 additions differs
+    for m0 in (0, M - 7):
+        small = ext.mma_tiles(x[m0:m0 + 7].contiguous(), *args, perm=perm, saturate=mode != "bf16_operands", rowinfo=rowinfo, layout=layout)
+        ref = np.abs(small.cpu().numpy()).max() + 1e-30
+        assert float((y[m0:m0 + 7] - small).abs().max()) <= 1e-4 * ref
+    assert torch.equal(y, ext.mma_tiles(x, *args, perm=perm, saturate=mode != "bf16_operands", rowinfo=rowinfo, layout=layout))
+
+
+def test_gemm_needs_layout_and_sliceable_widths():
+    d = H.mixed_width_pack(64, 256, [9, 6], seed=1)
+    args, perm, rowinfo, layout = _sorted_pack(d)
+    x = _x(64, 256, torch.float16, 1)
+    d2 = H.mixed_width_pack(64, 384, [6], seed=2)
+    args2, perm2, rowinfo2, layout2 = _sorted_pack(d2)
+    with pytest.raises(RuntimeError):
+        ext.mma_tiles(_x(64, 384, torch.float16, 2), *args2, perm=perm2, rowinfo=rowinfo2, layout=layout2)   # P % 256 != 0
+    with pytest.raises(RuntimeError):
+        ext.mma_tiles(x, *args, perm=perm, rowinfo=rowinfo, layout=layout)   # width 9 is not sliced
+    with pytest.raises(RuntimeError):
+        ext.mma_tiles(x, *args, perm=perm, rowinfo=rowinfo, layout=None)     # M > 48 without a layout
+    y = ext.mma_tiles(x[:48].contiguous(), *args, perm=perm, rowinfo=rowinfo, layout=layout)   # the tile kernel reads any width
+    _check(d, None, x[:48], y, saturate_ref=False)
+
+
+@pytest.mark.parametrize("Q,P,M", [(4096, 4096, 256), (1024, 12288, 64), (6144, 4096, 96)])
+def test_gemm_real_shapes_with_escapes(Q, P, M):
+    """Encoder-made packs at projection shapes (column ranges split over workgroups, two token blocks), escapes included,
+    through the operator: bf16 in, bf16 out."""
+    from qvb8_amd.formats.qvb8.module import QVBandLinearV8
+    W = H.synth_weight(Q, P, seed=Q + M).to(DEV)
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16", force_escapes=[5, P * (Q // 2) + 77, P * (Q - 1) + P - 1])
+    lin = QVBandLinearV8.from_encoded(enc)
+    x = _x(M, P, torch.bfloat16, Q)
+    y = lin(x)
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (M, Q)
+    assert lin._gemm_ok(lin._mma_order()[2], False)
+    v8 = H.oracle_view(enc)
+    Wr = O.reconstruct(v8["min_s"], v8["tau_s"], H.oracle_ids(v8), v8["esc_idx"], v8["esc_vals"])
+    xs = O.sat_half(x.float().cpu().numpy())
+    ref = O.linear_f64(xs, Wr)
+    tol = H.gemv_tolerance(ref, Wr, xs) + 2.0 ** -8 * np.abs(ref)
+    diff = np.abs(y.float().cpu().numpy().astype(np.float64) - ref)
+    assert np.all(diff <= tol), (float(diff.max()), float((diff / tol).max()))
