@@ -133,7 +133,8 @@ int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
  * by element.
  * 49 <= M <= 256 runs a workgroup-tiled decode + GEMM (X staged in LDS, v_mfma 32x32x16, column ranges added in a fixed
  * order): it needs `layout` with widths 4..8 (4..7 for bf16 operands), P % 256 == 0 and `workspace`; otherwise
- * QVB8_ERR_UNSUPPORTED / QVB8_ERR_WORKSPACE.  The reference restores the weight and calls a library GEMM there
+ * QVB8_ERR_UNSUPPORTED / QVB8_ERR_WORKSPACE.  33 <= M <= 48 takes the same kernel when those conditions hold and the
+ * workspace is there (it is the faster one from 33 rows on), else the 16-row tile kernel.  The reference restores the weight and calls a library GEMM there
  * (formats/qvb8/module.py:402-457).
  * Replaces: ext.mma_multi  qvb8_mma_multi_forward qvb8_cuda.cu:2566-2671 (kernels :2321-2441, escape fix
  * :2503-2548), and, through the Python module, the M <= 8 GEMV of :1059-1166 when P % 128 == 0. */

@@ -773,6 +773,10 @@ GemmPlan plan_gemm(int64_t M, int64_t Q, int64_t P) {
     return g;
 }
 
+// Fewest rows of X that go to the workgroup-tiled kernel when it can read the weight (49..: always; below that the tile
+// kernel is the alternative).
+int gemm_from() { const int v = host::env_int("QVB8_MMA_GEMM_FROM", 33); return v < 17 ? 17 : (v > 49 ? 49 : v); }
+
 template <int MT, bool BF>
 int launch_gemm(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_t s) {
     static bool attr[64] = {false};
@@ -802,7 +806,7 @@ extern "C" int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, co
 }
 
 extern "C" int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P) {
-    if (M > 48 && M <= 256 && Q > 0 && P > 0 && (P % (2 * kGemmStageCols)) == 0) return plan_gemm(M, Q, P).bytes;
+    if (M >= gemm_from() && M <= 256 && Q > 0 && P > 0 && (P % (2 * kGemmStageCols)) == 0) return plan_gemm(M, Q, P).bytes;
     return qvb8_mma_rowinfo_bytes(Q);
 }
 
@@ -853,8 +857,16 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     // mode 0: fp16 X, fp16 operands; 1: bf16 X narrowed to saturated fp16 on the way in, fp16 operands; 2: bf16 operands
     const int mode = x_dtype == QVB8_F16 ? 0 : (flags & QVB8_MMA_SATURATE_X) ? 1 : 2;
     int rc;
-    if (M > 48) {
-        // many rows of X: the workgroup-tiled kernel.  It addresses rows arithmetically and decodes whole slices only.
+    // Many rows of X: the workgroup-tiled kernel.  It addresses rows arithmetically and decodes whole slices only; from 33
+    // rows on it is also the faster one (the tile kernel then keeps too few bytes in flight), so it is taken whenever it
+    // can read the weight and the caller brought its workspace.
+    bool tiled = M > 48;
+    if (!tiled && M >= gemm_from() && layout && (P % (2 * kGemmStageCols)) == 0 && workspace
+        && workspace_bytes >= plan_gemm(M, Q, P).bytes && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
+        tiled = true;
+        for (int c = 0; c < a.n_classes; ++c) tiled = tiled && a.nb[c] >= 4 && a.nb[c] <= (mode == 2 ? 7 : 8);
+    }
+    if (tiled) {
         if (!layout) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: M > 48 needs rows stored in width order (a row layout)");
         if ((P % (2 * kGemmStageCols)) != 0) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: M > 48 needs P %% 256 == 0");
         for (int c = 0; c < a.n_classes; ++c)

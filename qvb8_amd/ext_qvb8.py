@@ -251,8 +251,9 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
         Y = torch.empty((M, Q), dtype=torch.float32, device=Xc.device)
         ei = esc_idx.contiguous() if n_esc else None
         ev = esc_vals.contiguous() if n_esc else None
-        ws = None if (rowinfo is not None and M <= MMA_MAX_M) else \
-            torch.empty((lib.qvb8_mma_workspace_bytes(M, Q, int(P)) + 7) // 8, dtype=torch.int64, device=Xc.device)
+        need = lib.qvb8_mma_workspace_bytes(M, Q, int(P))          # row records when none are passed; more for the tiled kernel
+        ws = None if (rowinfo is not None and need <= lib.qvb8_mma_rowinfo_bytes(Q)) else \
+            torch.empty((need + 7) // 8, dtype=torch.int64, device=Xc.device)
         _lib._check(lib.qvb8_mma(_lib.ptr(Xc), _lib.dtype_code(Xc.dtype), M, _lib.ptr(ids), ids.numel(),
                                  _lib.ptr(min_s), _lib.ptr(tau_s), _lib.ptr(row_nbits), _lib.ptr(row_bit_off),
                                  Q, int(P), _lib.ptr(ei), _lib.ptr(ev), n_esc, _lib.ptr(perm),

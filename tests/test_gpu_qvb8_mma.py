@@ -143,7 +143,7 @@ def _sorted_pack(d):
     return (ids, min_s, nbits, bit_off, P, tau_s, ei, ev), perm, rowinfo, layout
 
 
-@pytest.mark.parametrize("M", [49, 64, 65, 100, 128, 129, 256])
+@pytest.mark.parametrize("M", [33, 49, 64, 65, 100, 128, 129, 256])
 @pytest.mark.parametrize("mode", ["fp16", "bf16_saturated", "bf16_operands"])
 def test_gemm_many_rows(M, mode):
     """Three widths in one weight (each run of equal widths fills only part of its 256-row block), an odd number of
