@@ -329,7 +329,8 @@ size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 int launch_moe_gemv(int stage, MoeGemvArgs a, int64_t slots, hipStream_t s) {
     // enough workgroups to fill the chip four times over the selected experts, at least one unit per wave
     const int waves = kMoeThreads / 64;
-    const int64_t target_blocks = ((int64_t)host::env_int("QVB8_MOE_WGS_PER_CU", 4) * host::device_cus() + slots - 1) / slots;
+    // measured on the 35B-A3B shapes: four workgroups per CU are best for a handful of selected experts, eight for dozens
+    const int64_t target_blocks = ((int64_t)host::env_int("QVB8_MOE_WGS_PER_CU", slots > 16 ? 8 : 4) * host::device_cus() + slots - 1) / slots;
     int64_t upb = (a.units + target_blocks - 1) / target_blocks;
     upb = (upb + waves - 1) / waves * waves;
     a.units_per_block = (int)upb;
