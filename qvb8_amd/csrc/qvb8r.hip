@@ -65,9 +65,10 @@ __device__ __forceinline__ void walk_init(Walker& z, uint32_t* rg, const RCore& 
 }
 
 // one symbol: x' = f * (x >> 12) + d on the 64-bit state
+// `st` holds the slot table re-packed for the walk (block_setup): frequency << 21 | (slot - cumulative) << 11 | symbol.
 __device__ __forceinline__ uint32_t walk_dec(Walker& z, const uint32_t* st) {
     const uint32_t E = st[z.xl & 4095u];
-    const uint32_t f = (E >> 22) + 1u, d = (E >> 11) & 2047u;
+    const uint32_t f = E >> 21, d = (E >> 11) & 1023u;
     const uint64_t q = (((uint64_t)z.xh << 32) | z.xl) >> 12;
     const uint64_t x = (uint64_t)f * q + d;
     z.xl = (uint32_t)x; z.xh = (uint32_t)(x >> 32);
@@ -112,7 +113,12 @@ struct TileCtx { bool has; int tile, r0, nr; int64_t room; };
 __device__ __forceinline__ TileCtx block_setup(const RCore& c, int block, uint32_t* st, int h8) {
     int cls = c.blocks[3 * block], tb = c.blocks[3 * block + 1], ntb = c.blocks[3 * block + 2];
     cls = cls < 0 ? 0 : (cls >= c.K ? c.K - 1 : cls);
-    for (int i = threadIdx.x; i < 4096; i += blockDim.x) st[i] = c.tab[(int64_t)cls * 4096 + i];
+    // the file's entry is (frequency - 1) << 22 | (slot - cumulative) << 11 | symbol with frequency <= 1024; the walk wants
+    // the frequency itself, one instruction per symbol less
+    for (int i = threadIdx.x; i < 4096; i += blockDim.x) {
+        const uint32_t E = c.tab[(int64_t)cls * 4096 + i];
+        st[i] = (((E >> 22) + 1u) << 21) | (E & 0x1FFFFFu);
+    }
     TileCtx t;
     t.tile = tb + h8;
     t.has = h8 < ntb && t.tile >= 0 && t.tile < c.n_tiles;
