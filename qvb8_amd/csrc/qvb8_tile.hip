@@ -480,7 +480,7 @@ __global__ void __launch_bounds__(256) tile_fix_escapes_kernel(const uint16_t* _
 
 // ---- fused decode + GEMM, M = 49..256 ---------------------------------------------------------------------------------
 // For this many rows of X the activations no longer fit a wave's registers, and every byte of X must serve many weight
-// rows: a workgroup (4 waves) takes 256 weight rows of ONE width x TMK = 32 * MT rows of X x one range of columns.  X goes
+// rows: a workgroup (4 waves) takes 256 weight rows of ONE width x TMK = 32 * MT = 64 rows of X x one range of columns.  X goes
 // through LDS in stages of 128 columns (double-buffered); the weights never touch LDS: lane (n = l % 32, kh = l / 32) of a
 // wave owns the 32 consecutive ids of row n at columns 64 * step + 32 * kh, fetched as two 16-byte loads and decoded
 // into the B operands of four v_mfma_f32_32x32x16 (the K order inside a step is a permutation that X follows).  The id
@@ -751,7 +751,7 @@ int64_t align256i(int64_t n) { return (n + 255) & ~(int64_t)255; }
 // ceil(Q / 256): up to two more exist when the rows have several widths).
 GemmPlan plan_gemm(int64_t M, int64_t Q, int64_t P) {
     GemmPlan g;
-    g.MT = M <= 64 ? 2 : 4;
+    g.MT = 2;                                          // 64 rows of X per workgroup: measured faster than 128 (one wave per SIMD) at every M
     const int TMK = 32 * g.MT;
     g.tok_blocks = (int)((M + TMK - 1) / TMK);
     g.row_blocks = (int)((Q + kGemmRows - 1) / kGemmRows);
@@ -894,8 +894,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         ga.blocks2 = ga.blocks1 + (rows1 + kGemmRows - 1) / kGemmRows;
         const int row_blocks = ga.blocks2 + (rows2 + kGemmRows - 1) / kGemmRows;
         ga.widths = (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16);
-        if (mode == 2) rc = g.MT == 2 ? launch_gemm<2, true>(ga, g, row_blocks, s) : launch_gemm<4, true>(ga, g, row_blocks, s);
-        else rc = g.MT == 2 ? launch_gemm<2, false>(ga, g, row_blocks, s) : launch_gemm<4, false>(ga, g, row_blocks, s);
+        rc = mode == 2 ? launch_gemm<2, true>(ga, g, row_blocks, s) : launch_gemm<2, false>(ga, g, row_blocks, s);
         if (rc) return rc;
         if (g.splits > 1) {
             const int64_t n = M * Q;
