@@ -747,7 +747,7 @@ struct GemmPlan {
 };
 int64_t align256i(int64_t n) { return (n + 255) & ~(int64_t)255; }
 
-// Column ranges of whole 256-column groups, enough of them for about one workgroup per CU (row blocks counted as
+// Column ranges of whole 256-column groups, enough of them for about three workgroups per four CUs (row blocks counted as
 // ceil(Q / 256): up to two more exist when the rows have several widths).
 GemmPlan plan_gemm(int64_t M, int64_t Q, int64_t P) {
     GemmPlan g;
@@ -757,7 +757,8 @@ GemmPlan plan_gemm(int64_t M, int64_t Q, int64_t P) {
     g.row_blocks = (int)((Q + kGemmRows - 1) / kGemmRows);
     const int64_t groups = P / (2 * kGemmStageCols);
     const int64_t base = (int64_t)g.tok_blocks * g.row_blocks;
-    const int64_t target = (int64_t)host::env_int("QVB8_GEMM_WGS_PER_CU", 1) * host::device_cus();
+    // measured: three workgroups per four CUs is the best trade between idle CUs and partial-result traffic
+    const int64_t target = host::env_int("QVB8_GEMM_TARGET_WGS", 0) > 0 ? host::env_int("QVB8_GEMM_TARGET_WGS", 0) : 3 * (int64_t)host::device_cus() / 4;
     int64_t splits = (target + base - 1) / base;
     if (splits > groups) splits = groups;
     if (splits > 16) splits = 16;
