@@ -138,13 +138,25 @@ def time_graph(step, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall * 1e3 / steps
 
 
+def synthetic_routing(logits, k):
+    """softmax -> top-k -> renormalise, the reference's router (run/run_inference.py:92-100): synthetic input of the MoE
+    workload, built on the host before anything is timed."""
+    import numpy as np
+    z = np.asarray(logits, np.float64)
+    z = z - z.max(-1, keepdims=True)
+    p = np.exp(z)
+    p /= p.sum(-1, keepdims=True)
+    idx = np.argsort(-p, axis=-1, kind="stable")[:, :k]
+    w = np.take_along_axis(p, idx, -1)
+    return idx.astype(np.int64), (w / w.sum(-1, keepdims=True)).astype(np.float32)
+
+
 def bench_moe(args, dev):
     """Config 4: Qwen-35B-A3B-shape MoE layer (hidden 2048, 128 experts of gate/up 2048->768 and down 768->2048, top-8
     routing from softmax of N(0,1) logits), QVB8 at tau = 2e-3, `--tokens` tokens.  A step = the expert stacks of
     `--layers` distinct layers through qvb8_moe_experts; bytes = packed ids + row metadata of the UNIQUE selected experts."""
     import numpy as np
     import torch
-    from oracle import qvb8_oracle as O                      # router_topk only: builds the synthetic routing, not timed
     from qvb8_amd import _lib
     from qvb8_amd.formats.qvb8 import pack as PK
     from qvb8_amd.formats.qvb8.backends_experts import QVBandExpertsV8
@@ -169,7 +181,7 @@ def bench_moe(args, dev):
     ws = torch.empty(lib.qvb8_moe_workspace_bytes(T, k, E, 2 * inter, inter, hidden), dtype=torch.uint8, device=dev)
     routes, step_bytes = [], 0
     for g_, d_ in stacks:
-        idx, w = O.router_topk(rng.normal(size=(T, E)), k)
+        idx, w = synthetic_routing(rng.normal(size=(T, E)), k)
         routes.append((torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)))
         per_expert = (g_["ids"].numel() + d_["ids"].numel()) // E + 17 * (g_["Q"] + d_["Q"])
         step_bytes += len(np.unique(idx)) * per_expert + 2 * T * hidden * 2
@@ -348,9 +360,9 @@ def main():
     assert step_bytes == sum(u["bytes"] for u in units)
     n_launch = len(units)
 
-    def step():
+    def run_units(which):
         s = torch.cuda.current_stream().cuda_stream
-        for u in units:
+        for u in which:
             x, lin = x_by_p[u["P"]], u["lin"]
             rc = lib.qvb8_mma(x.data_ptr(), _lib.dtype_code(x.dtype), 1, lin.ids.data_ptr(), lin.ids.numel(),
                               lin.min_s.data_ptr(), lin.tau_s.data_ptr(), lin.nbits.data_ptr(), lin.bit_off.data_ptr(),
@@ -361,6 +373,9 @@ def main():
                               MMA_FLAGS, u["Y"].data_ptr(), None, 0, s)
             if rc != 0:
                 raise RuntimeError(lib.qvb8_last_error().decode())
+
+    def step():
+        run_units(units)
 
     if args.copy_probe:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
@@ -396,6 +411,15 @@ def main():
                      "kernel": "qvb8::tile_kernel<1,4,false,true>", "bytes_per_launch": step_bytes // n_launch,
                      "launch_us": round(launch_us, 3)},
     }
+    # GB/s per projection group: the launches of one kind over all layers, replayed on their own (not part of `value`)
+    per = {}
+    for name in sorted({u["name"] for u in units}, key=len):
+        mine = [u for u in units if u["name"] == name]
+        ev_g, wall_g = time_graph(lambda: run_units(mine), max(5, args.steps // 2), 2)
+        us = max(ev_g, wall_g) * 1e3 / len(mine)
+        b = sum(u["bytes"] for u in mine) / len(mine)
+        per[name] = {"us_per_launch": round(us, 2), "GB/s": round(b / (us * 1e-6) / 1e9, 1), "bytes_per_launch": int(b)}
+    out["per_projection"] = per
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(layers, x_by_p)
     else:
