@@ -29,6 +29,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 LAYER_9B = (("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
             ("gate", 12288, 4096), ("up", 12288, 4096), ("down", 4096, 12288))
+# 27B-class dense shapes (hidden 5120, FFN 17408; q/o 5120, k/v 1024 as in the 9B set): `--model 27b`, not the headline
+LAYER_27B = (("q", 5120, 5120), ("k", 1024, 5120), ("v", 1024, 5120), ("o", 5120, 5120),
+             ("gate", 17408, 5120), ("up", 17408, 5120), ("down", 5120, 17408))
 TAU = 1e-3
 # HBM bytes per launch of the tile kernel from hardware counters (FETCH_SIZE scaled by 2.0 against a plain 1 GiB pass,
 # plus WRITE_SIZE), as recorded in profiles/tile_kernel_9b_decode_step_hbm_traffic.md, by launch class
@@ -47,7 +50,7 @@ def algorithmic_bytes(enc, M):
 SAME_INPUT = (("q", "k", "v"), ("gate", "up"))          # projections fed the same activation: one launch each when fused
 
 
-def build_layers(n_layers, dev, fuse):
+def build_layers(n_layers, dev, fuse, shapes=None):
     """Per layer: the encoded projections (kept for byte counts and the CPU leg) and the launch units made of them: one
     QVBandLinearV8 per projection, or one per same-input group when `fuse` (rows concatenated, results split as views)."""
     import torch
@@ -55,9 +58,10 @@ def build_layers(n_layers, dev, fuse):
     from qvb8_amd.formats.qvb8.fuse import concat_linears
     from qvb8_amd.formats.qvb8.module import QVBandLinearV8
     layers, units = [], []
+    shapes = shapes or LAYER_9B
     for li in range(n_layers):
         encs, mods = [], {}
-        for pi, (name, Q, P) in enumerate(LAYER_9B):
+        for pi, (name, Q, P) in enumerate(shapes):
             g = torch.Generator(device=dev).manual_seed(1000 * li + pi)
             W = (0.02 * torch.randn(Q, P, device=dev, generator=g)).to(torch.bfloat16)
             enc = PK.encode_tensor(W, TAU, restore="fp16")
@@ -68,7 +72,7 @@ def build_layers(n_layers, dev, fuse):
             mods[name] = QVBandLinearV8.from_encoded(enc)
         layers.append(encs)
         done = set()
-        for name, _, _ in LAYER_9B:
+        for name, _, _ in shapes:
             if name in done:
                 continue
             group = next((g for g in SAME_INPUT if name in g), (name,)) if fuse else (name,)
@@ -321,6 +325,8 @@ def main():
                     help="decode9b (default, the headline metric): 9B-shape decode step; moe: 35B-A3B-shape expert stack; "
                          "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256)")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
+    ap.add_argument("--model", choices=("9b", "27b"), default="9b",
+                    help="decode9b workload only: layer shapes (9b = the headline configuration; 27b = hidden 5120, FFN 17408)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sort", action="store_true",
                     help="keep the file's row order in memory (row addresses are then read from the row records instead of "
@@ -352,9 +358,10 @@ def main():
     if args.no_sort:
         from qvb8_amd.formats.qvb8.module import QVBandLinearV8
         QVBandLinearV8.sort_rows = False
-    layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse)
+    shapes = LAYER_27B if args.model == "27b" else LAYER_9B
+    layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse, shapes=shapes)
     g = torch.Generator(device=dev).manual_seed(7)
-    x_by_p = {P: torch.randn(1, P, device=dev, generator=g).to(torch.bfloat16) for P in (4096, 12288)}
+    x_by_p = {P: torch.randn(1, P, device=dev, generator=g).to(torch.bfloat16) for P in sorted({p for _, _, p in shapes})}
     flat = [enc for lay in layers for enc in lay]
     step_bytes = sum(algorithmic_bytes(e, 1) for e in flat)
     assert step_bytes == sum(u["bytes"] for u in units)
@@ -398,14 +405,16 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 activations x fp32 band value, fp32 accumulate", "data": "synthetic",
         "tokens_per_s": round(1e3 / ms_per_step, 2), "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
-        "config": {"workload": "Qwen-9B-shape decoder layer set (q/k/v/o 4096x4096 with k/v 1024, gate/up 12288, down "
-                               "12288->4096), QVB8 tau=1e-3, bf16 activations, M=1, %d layers" % args.layers,
+        "config": {"workload": ("Qwen-9B-shape decoder layer set (q/k/v/o 4096x4096 with k/v 1024, gate/up 12288, down "
+                                "12288->4096), QVB8 tau=1e-3, bf16 activations, M=1, %d layers" % args.layers) if args.model == "9b" else
+                               ("27B-class decoder layer set (q/o 5120x5120, k/v 1024x5120, gate/up 17408, down 17408->5120), "
+                                "QVB8 tau=1e-3, bf16 activations, M=1, %d layers" % args.layers),
                    "launches_per_step": n_launch, "launch_units": "+".join(sorted({u["name"] for u in units}, key=len)),
                    "bytes_per_step": step_bytes, "escapes": esc,
                    "bits_per_weight": round(8.0 * sum(u["lin"].ids.numel() for u in units) / sum(e["Q"] * e["P"] for e in flat), 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": (None if MMA_FLAGS != 1 else
+                     "traffic": (None if MMA_FLAGS != 1 or args.model != "9b" else
                                  round(sum(MEASURED_TRAFFIC[256 if e["Q"] >= 4096 else 64] for e in flat) / n_launch) if args.no_fuse
                                  else round(sum(MEASURED_TRAFFIC["q+k+v" if u["name"] == "q+k+v" else "fused-other"] for u in units) / n_launch)),
                      "kernel": "qvb8::tile_kernel<1,4,false,true>", "bytes_per_launch": step_bytes // n_launch,
