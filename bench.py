@@ -400,7 +400,7 @@ def main():
     esc = sum(e["esc_idx"].numel() for e in flat)
 
     out = {
-        "metric": "dequant-GEMV HBM GB/s (% of peak) + decode tokens/s, 9B-shape pack, 1 MI355X",
+        "metric": "dequant-GEMV HBM GB/s (% of peak) + decode tokens/s, %s-shape pack, 1 MI355X" % ("9B" if args.model == "9b" else "27B"),
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 activations x fp32 band value, fp32 accumulate", "data": "synthetic",
@@ -417,7 +417,8 @@ def main():
                      "traffic": (None if MMA_FLAGS != 1 or args.model != "9b" else
                                  round(sum(MEASURED_TRAFFIC[256 if e["Q"] >= 4096 else 64] for e in flat) / n_launch) if args.no_fuse
                                  else round(sum(MEASURED_TRAFFIC["q+k+v" if u["name"] == "q+k+v" else "fused-other"] for u in units) / n_launch)),
-                     "kernel": "qvb8::tile_kernel<1,4,false,true>", "bytes_per_launch": step_bytes // n_launch,
+                     "kernel": "qvb8::tile_kernel<1,4,false,true>" + (" / <1,5,false,true> for 5120-column rows" if args.model == "27b" else ""),
+                     "bytes_per_launch": step_bytes // n_launch,
                      "launch_us": round(launch_us, 3)},
     }
     # GB/s per projection group: the launches of one kind over all layers, replayed on their own (not part of `value`)
