@@ -118,12 +118,14 @@ typedef struct qvb8_mma_layout {
     int32_t nbits[QVB8_MMA_MAX_CLASSES];
 } qvb8_mma_layout;
 
-/* Workspace qvb8_mma needs: for M <= 48 only when it is called WITHOUT row records (it then builds them itself first);
- * for 49 <= M <= 256 always (narrowed activations, their sums per column range, partial results of the column ranges). */
+/* Workspace qvb8_mma needs: up to 32 rows of X only when it is called WITHOUT row records (it then builds them itself
+ * first); from 33 rows on, when P % 256 == 0, what the workgroup-tiled kernel needs (narrowed activations, their sums per
+ * column range, partial results of the column ranges). */
 int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
 
 /* Y[m, q] = sum_c X[m, c] * value(q, c), fp32 accumulate on v_mfma 16x16x32, Y f32 (M, Q) row-major.
- * X is (M, P) fp16 or bf16 (x_dtype QVB8_F16 / QVB8_BF16), 16-byte aligned, P % 128 == 0, 1 <= M <= 48.
+ * X is (M, P) fp16 or bf16 (x_dtype QVB8_F16 / QVB8_BF16), 16-byte aligned, P % 128 == 0, 1 <= M <= 48 (up to 256 under the
+ * conditions below).
  * The ids enter the matrix product exactly (as bias + id in X's own 16-bit format) and tau_s / min_s are applied
  * in fp32 afterwards, so the result equals X times the UN-narrowed fp32 band value, escapes exact.
  * `perm` (i32[Q], position -> row, or NULL): order in which rows are grouped into tiles of 16; rows sorted by
@@ -134,8 +136,8 @@ int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
  * 49 <= M <= 256 runs a workgroup-tiled decode + GEMM (X staged in LDS, v_mfma 32x32x16, column ranges added in a fixed
  * order): it needs `layout` with widths 4..8 (4..7 for bf16 operands), P % 256 == 0 and `workspace`; otherwise
  * QVB8_ERR_UNSUPPORTED / QVB8_ERR_WORKSPACE.  33 <= M <= 48 takes the same kernel when those conditions hold and the
- * workspace is there (it is the faster one from 33 rows on), else the 16-row tile kernel.  The reference restores the weight and calls a library GEMM there
- * (formats/qvb8/module.py:402-457).
+ * workspace is there (it is the faster one from 33 rows on), else the 16-row tile kernel.  Above 48 rows the reference
+ * restores the weight and calls a library GEMM (formats/qvb8/module.py:402-457).
  * Replaces: ext.mma_multi  qvb8_mma_multi_forward qvb8_cuda.cu:2566-2671 (kernels :2321-2441, escape fix
  * :2503-2548), and, through the Python module, the M <= 8 GEMV of :1059-1166 when P % 128 == 0. */
 int qvb8_mma(const void* X, int x_dtype, int64_t M,
