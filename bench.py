@@ -9,7 +9,7 @@ HIP graph and replayed; `value` is the algorithmic bytes of a step (packed ids +
 in and out) divided by the measured time per step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--no-cpu] [--no-fuse] [--no-sort] [--copy-probe]
-                    [--workload decode9b|smallm|moe|qvb8r] [--tokens T]
+                    [--workload decode9b|smallm|moe|qvb8r|lmhead] [--tokens T]
 
 Prints ONE JSON line.  `roofline` covers the dominant kernel (the tile kernel, every launch of the step):
 algorithmic bytes per launch / average launch time, timed with HIP events on the launch stream over the timed region.
@@ -45,6 +45,10 @@ def algorithmic_bytes(enc, M):
     per escape, the bf16 activations in and the bf16 results out."""
     ids = enc["ids"] if "ids" in enc else enc["ids_host"]
     return int(ids.numel() + 17 * enc["Q"] + 12 * enc["esc_idx"].numel() + 2 * M * enc["P"] + 2 * M * enc["Q"])
+
+
+def decode_metric_name(model):
+    return "dequant-GEMV HBM GB/s (% of peak) + decode tokens/s, " + {"9b": "9B", "27b": "27B"}[model] + "-shape pack, 1 MI355X"
 
 
 SAME_INPUT = (("q", "k", "v"), ("gate", "up"))          # projections fed the same activation: one launch each when fused
@@ -276,6 +280,56 @@ def bench_qvb8r(args, dev):
             "cpu_baseline": None}
 
 
+def bench_lmhead(args, dev):
+    """The largest single GEMV of the 27B-class model: the output head, 248320 x 5120 at tau = 1e-3, M = `--tokens` (1 by
+    default): one launch of qvb8_mma per step over 1.1 GB of packed ids (far beyond the 256 MB last-level cache, so
+    every replay streams from HBM).  Shows what the kernel streams when the fixed cost of a launch no longer matters."""
+    import torch
+    from qvb8_amd.formats.qvb8 import pack as PK
+    from qvb8_amd.formats.qvb8.module import QVBandLinearV8
+    lib = __import__("qvb8_amd._lib", fromlist=["load"]).load()
+    from qvb8_amd import _lib
+    Q, P, M = 248320, 5120, args.tokens
+    parts = []
+    for i in range(0, Q, 31040):                                      # encode in eight slices of rows, then concatenate
+        g = torch.Generator(device=dev).manual_seed(9000 + i)
+        W = (0.02 * torch.randn(31040, P, device=dev, generator=g)).to(torch.bfloat16)
+        enc = PK.encode_tensor(W, TAU, restore="fp16")
+        assert enc["max_err"] < TAU
+        parts.append(QVBandLinearV8.from_encoded(enc))
+        del W, enc
+    from qvb8_amd.formats.qvb8.fuse import concat_linears
+    lin = concat_linears(parts)[0]
+    del parts
+    perm, rowinfo, layout = lin._mma_order()
+    x = torch.randn(M, P, device=dev, generator=torch.Generator(device=dev).manual_seed(3)).to(torch.bfloat16)
+    Y = torch.empty((M, Q), dtype=torch.float32, device=dev)
+    n_esc = lin.esc_idx.numel()
+    nbytes = int(lin.ids.numel() + 17 * Q + 12 * n_esc + 2 * M * P + 2 * M * Q)
+
+    def step():
+        rc = lib.qvb8_mma(x.data_ptr(), _lib.dtype_code(x.dtype), M, lin.ids.data_ptr(), lin.ids.numel(),
+                          lin.min_s.data_ptr(), lin.tau_s.data_ptr(), lin.nbits.data_ptr(), lin.bit_off.data_ptr(), Q, P,
+                          lin.esc_idx.data_ptr() if n_esc else None, lin.esc_vals.data_ptr() if n_esc else None, n_esc,
+                          perm.data_ptr(), rowinfo.data_ptr(), ctypes.addressof(layout) if layout is not None else None,
+                          MMA_FLAGS, Y.data_ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError(lib.qvb8_last_error().decode())
+    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
+    ms = max(ev_ms, wall_ms)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"metric": "dequant-GEMV HBM GB/s (% of peak), output head 248320 x 5120, 1 MI355X",
+            "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16 activations x fp32 band value, fp32 accumulate", "data": "synthetic",
+            "config": {"workload": "output head 248320 x 5120, QVB8 tau=1e-3, bf16 activations, M=%d, one launch per step" % M,
+                       "bytes_per_step": nbytes, "bits_per_weight": round(8.0 * lin.ids.numel() / (Q * P), 3)},
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                         "kernel": "qvb8::tile_kernel<1,5,false,true>", "bytes_per_launch": nbytes, "launch_us": round(ev_ms * 1e3, 2)},
+            "cpu_baseline": None}
+
+
 def bench_smallm(args, dev):
     """Config 3: the 9B projections with M = `--tokens` rows (draft-verify / prefill chunk), through QVBandLinearV8's own
     dispatch: M <= 48 the tile kernel (X in registers), 49..256 the workgroup-tiled decode + GEMM kernel (X staged in LDS,
@@ -321,7 +375,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=None, help="layers of distinct packs (default 32; moe 4; qvb8r 2)")
-    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r"), default="decode9b",
+    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead"), default="decode9b",
                     help="decode9b (default, the headline metric): 9B-shape decode step; moe: 35B-A3B-shape expert stack; "
                          "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256)")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
@@ -350,9 +404,9 @@ def main():
     torch.cuda.set_device(dev)
     lib = _lib.load()                                       # raises when the HIP library is missing: no fallback
     if args.layers is None:
-        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 2}[args.workload]
+        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 2, "lmhead": 1}[args.workload]
     if args.workload != "decode9b":
-        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm}[args.workload]
+        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead}[args.workload]
         print(json.dumps(fn(args, dev)))
         return 0
     if args.no_sort:
@@ -400,7 +454,7 @@ def main():
     esc = sum(e["esc_idx"].numel() for e in flat)
 
     out = {
-        "metric": "dequant-GEMV HBM GB/s (% of peak) + decode tokens/s, %s-shape pack, 1 MI355X" % ("9B" if args.model == "9b" else "27B"),
+        "metric": decode_metric_name(args.model),
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 activations x fp32 band value, fp32 accumulate", "data": "synthetic",
