@@ -9,7 +9,7 @@ HIP graph and replayed; `value` is the algorithmic bytes of a step (packed ids +
 in and out) divided by the measured time per step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--no-cpu] [--no-fuse] [--no-sort] [--copy-probe]
-                    [--workload decode9b|smallm|moe|qvb8r|lmhead] [--tokens T]
+                    [--workload decode9b|smallm|moe|qvb8r|lmhead|embed] [--tokens T]
 
 Prints ONE JSON line.  `roofline` covers the dominant kernel (the tile kernel, every launch of the step):
 algorithmic bytes per launch / average launch time, timed with HIP events on the launch stream over the timed region.
@@ -280,27 +280,76 @@ def bench_qvb8r(args, dev):
             "cpu_baseline": None}
 
 
-def bench_lmhead(args, dev):
-    """The largest single GEMV of the 27B-class model: the output head, 248320 x 5120 at tau = 1e-3, M = `--tokens` (1 by
-    default): one launch of qvb8_mma per step over 1.1 GB of packed ids (far beyond the 256 MB last-level cache, so
-    every replay streams from HBM).  Shows what the kernel streams when the fixed cost of a launch no longer matters."""
+def build_vocab_table(dev):
+    """248320 x 5120 at tau = 1e-3 (the 27B-class model's vocabulary table, output head and embedding alike), as one
+    QVBandLinearV8: encoded in eight slices of rows, then concatenated."""
     import torch
     from qvb8_amd.formats.qvb8 import pack as PK
+    from qvb8_amd.formats.qvb8.fuse import concat_linears
     from qvb8_amd.formats.qvb8.module import QVBandLinearV8
-    lib = __import__("qvb8_amd._lib", fromlist=["load"]).load()
-    from qvb8_amd import _lib
-    Q, P, M = 248320, 5120, args.tokens
+    Q, P = 248320, 5120
     parts = []
-    for i in range(0, Q, 31040):                                      # encode in eight slices of rows, then concatenate
+    for i in range(0, Q, 31040):
         g = torch.Generator(device=dev).manual_seed(9000 + i)
         W = (0.02 * torch.randn(31040, P, device=dev, generator=g)).to(torch.bfloat16)
         enc = PK.encode_tensor(W, TAU, restore="fp16")
         assert enc["max_err"] < TAU
         parts.append(QVBandLinearV8.from_encoded(enc))
         del W, enc
-    from qvb8_amd.formats.qvb8.fuse import concat_linears
-    lin = concat_linears(parts)[0]
-    del parts
+    return concat_linears(parts)[0]
+
+
+def bench_embed(args, dev):
+    """Embedding read of `--tokens` rows (default 4096, a prefill's worth) from the 248320 x 5120 table, bf16 out.  A
+    step = 16 launches of qvb8_lookup_rows, each with its own random rows and its own output (one graph replay costs
+    the host about 20 us, more than one launch takes).  Bytes: the looked-up rows' packed ids + 16 bytes of row
+    metadata + the row numbers in, the bf16 rows out."""
+    import torch
+    lib = __import__("qvb8_amd._lib", fromlist=["load"]).load()
+    from qvb8_amd import _lib
+    lin = build_vocab_table(dev)
+    Q, P = lin.out_features, lin.in_features
+    T = args.tokens if args.tokens > 1 else 4096
+    reps = 16
+    g = torch.Generator(device=dev).manual_seed(11)
+    toks = [torch.randint(0, Q, (T,), device=dev, generator=g) for _ in range(reps)]
+    outs = [torch.empty((T, P), dtype=torch.bfloat16, device=dev) for _ in range(reps)]
+    n_esc = lin.esc_idx.numel()
+    nbytes = sum(int((lin.nbits[t].to(torch.int64) * P // 8).sum()) for t in toks) // reps + T * (16 + 8) + 2 * T * P
+
+    def step():
+        for tok, out in zip(toks, outs):
+            rc = lib.qvb8_lookup_rows(tok.data_ptr(), T, lin.ids.data_ptr(), lin.ids.numel(), lin.min_s.data_ptr(),
+                                      lin.tau_s.data_ptr(), lin.nbits.data_ptr(), lin.bit_off.data_ptr(), Q, P,
+                                      lin.esc_idx.data_ptr() if n_esc else None, lin.esc_vals.data_ptr() if n_esc else None,
+                                      n_esc, _lib.BF16, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+            if rc != 0:
+                raise RuntimeError(lib.qvb8_last_error().decode())
+    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
+    ms = max(ev_ms, wall_ms)
+    us = ms * 1e3 / reps
+    gbs = nbytes / (us * 1e-6) / 1e9
+    return {"metric": "embedding read HBM GB/s, 248320 x 5120 table, 1 MI355X",
+            "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "fp32 band value, bf16 out", "data": "synthetic",
+            "config": {"workload": "embedding read of %d random rows, 248320 x 5120, QVB8 tau=1e-3, bf16 out, %d launches per step" % (T, reps),
+                       "bytes_per_launch": nbytes, "rows_per_s": round(T / (us * 1e-6)), "escapes": n_esc},
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "qvb8::decode_kernel<2, true>",
+                         "bytes_per_launch": nbytes, "launch_us": round(us, 3)},
+            "cpu_baseline": None}
+
+
+def bench_lmhead(args, dev):
+    """The largest single GEMV of the 27B-class model: the output head, 248320 x 5120 at tau = 1e-3, M = `--tokens` (1 by
+    default): one launch of qvb8_mma per step over 1.1 GB of packed ids (far beyond the 256 MB last-level cache, so
+    every replay streams from HBM).  Shows what the kernel streams when the fixed cost of a launch no longer matters."""
+    import torch
+    lib = __import__("qvb8_amd._lib", fromlist=["load"]).load()
+    from qvb8_amd import _lib
+    Q, P, M = 248320, 5120, args.tokens
+    lin = build_vocab_table(dev)
     perm, rowinfo, layout = lin._mma_order()
     x = torch.randn(M, P, device=dev, generator=torch.Generator(device=dev).manual_seed(3)).to(torch.bfloat16)
     Y = torch.empty((M, Q), dtype=torch.float32, device=dev)
@@ -375,7 +424,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=None, help="layers of distinct packs (default 32; moe 4; qvb8r 2)")
-    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead"), default="decode9b",
+    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead", "embed"), default="decode9b",
                     help="decode9b (default, the headline metric): 9B-shape decode step; moe: 35B-A3B-shape expert stack; "
                          "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256)")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
@@ -404,9 +453,9 @@ def main():
     torch.cuda.set_device(dev)
     lib = _lib.load()                                       # raises when the HIP library is missing: no fallback
     if args.layers is None:
-        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 2, "lmhead": 1}[args.workload]
+        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 2, "lmhead": 1, "embed": 1}[args.workload]
     if args.workload != "decode9b":
-        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead}[args.workload]
+        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead, "embed": bench_embed}[args.workload]
         print(json.dumps(fn(args, dev)))
         return 0
     if args.no_sort:

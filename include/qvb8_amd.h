@@ -53,6 +53,18 @@ int qvb8_decode(const uint8_t* ids, int64_t ids_bytes, const float* min_s, const
                 const uint8_t* nbits, const int64_t* bit_off, int64_t Q, int64_t P,
                 int out_dtype, void* out, void* stream);
 
+/* Row lookup (the embedding read): out[i*P + c] = (T)(min_s[r] + (float)id[r][c] * tau_s[r]) for r = rows[i], the
+ * product and the sum rounded separately in fp32 as the reference's lookup does (NOT the single rounding of
+ * qvb8_decode), then every escape of row r overwrites its column with (T)esc_vals[e].  rows: i64[n_rows] in device
+ * memory, any order, repeats allowed; a row number outside 0..Q-1 gives a row of NaN.  esc_idx ascending flat
+ * positions q*P+c of the whole table (may be null when n_esc = 0).  out: (n_rows, P) of out_dtype, 16-byte aligned.
+ * Replaces QVBandEmbeddingV8._decode_rows + the escape loop of forward  formats/qvb8/embedding.py:92-119, 121-152
+ * (there: torch byte gathers and a host loop over the looked-up rows). */
+int qvb8_lookup_rows(const int64_t* rows, int64_t n_rows, const uint8_t* ids, int64_t ids_bytes, const float* min_s,
+                     const float* tau_s, const uint8_t* nbits, const int64_t* bit_off, int64_t Q, int64_t P,
+                     const int64_t* esc_idx, const float* esc_vals, int64_t n_esc, int out_dtype, void* out,
+                     void* stream);
+
 /* out[esc_idx[e]] = (T)esc_vals[e] for every escape: the overwrite the reference does with
  * index_copy_(0, esc_idx, esc_vals.to(dt))  qvb8_cuda.cu:689-697, 1721-1725.  n_out = Q*P (bounds check). */
 int qvb8_scatter_escapes(void* out, int out_dtype, int64_t n_out, const int64_t* esc_idx,

@@ -16,6 +16,9 @@ Pinning status (what fixes each function besides this file's own text):
   fma32 / band_values / reconstruct   libm fmaf via ctypes (exhaustive over ids),
                                       float64 closed form, reference decode_tensor
                                       golden vectors
+  embedding_rows                      float64 closed form rounded twice, a known answer
+                                      on which the fused and the two-step value differ,
+                                      agreement with reconstruct within one ulp
   narrow_fp16 / narrow_bf16           numpy.float16, torch.bfloat16
   e4m3_lut / e4m3_decode              torch.float8_e4m3fn
   parse_qvb8_blob / parse_qvbd_blob   golden vectors produced by the reference's
@@ -174,6 +177,34 @@ def restore(min_s, tau_s, ids, esc_idx=None, esc_vals=None, dtype="fp32") -> np.
         return narrow_bf16(w)
     if dtype == "fp32":
         return w
+    raise ValueError(dtype)
+
+
+def embedding_rows(rows, min_s, tau_s, ids, P: int, esc_idx=None, esc_vals=None, dtype="fp32") -> np.ndarray:
+    """Rows `rows` of the table as the reference's embedding reads them (formats/qvb8/embedding.py:97-158): the band
+    value is `min_s[r] + float(id) * tau_s[r]` as an fp32 multiply then an fp32 add (two roundings; the linear layers'
+    restore fuses them), the escapes of the looked-up rows are written over it in fp32, and the result is narrowed once
+    to the output dtype.  `ids` is the dense (Q, P) id matrix.  Returns fp32 holding the narrowed values."""
+    rows = np.asarray(rows, np.int64).reshape(-1)
+    idf = np.asarray(ids)[rows].astype(np.float32)
+    ts = np.asarray(tau_s, np.float32)[rows].reshape(-1, 1)
+    m = np.asarray(min_s, np.float32)[rows].reshape(-1, 1)
+    prod = (idf * ts).astype(np.float32)
+    out = (m + prod).astype(np.float32)
+    if esc_idx is not None and len(esc_idx):
+        ei = np.asarray(esc_idx, np.int64)
+        er, ec = ei // P, ei - (ei // P) * P
+        ev = np.asarray(esc_vals, np.float32)
+        for i, r in enumerate(rows.tolist()):
+            hit = er == r
+            if hit.any():
+                out[i, ec[hit]] = ev[hit]
+    if dtype == "fp16":
+        return narrow_fp16(out)
+    if dtype == "bf16":
+        return narrow_bf16(out)
+    if dtype == "fp32":
+        return out
     raise ValueError(dtype)
 
 

@@ -16,7 +16,7 @@ F32, F16, BF16 = 0, 1, 2
 _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 # every symbol include/qvb8_amd.h declares
-SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_scatter_escapes", "qvb8_certify",
+SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_lookup_rows", "qvb8_scatter_escapes", "qvb8_certify",
            "qvb8_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma",
            "qvb8_moe_workspace_bytes", "qvb8_moe_experts",
            "qvb8r_decode", "qvb8r_gemv_workspace_bytes", "qvb8r_gemv", "qvb8r_fix_escapes")
@@ -51,6 +51,7 @@ def load(build_if_missing: bool = True):
     lib.qvb8_abi_version.restype = i32
     lib.qvb8_last_error.restype = ctypes.c_char_p
     lib.qvb8_decode.argtypes = [vp, i64, vp, vp, vp, vp, i64, i64, i32, vp, vp]
+    lib.qvb8_lookup_rows.argtypes = [vp, i64, vp, i64, vp, vp, vp, vp, i64, i64, vp, vp, i64, i32, vp, vp]
     lib.qvb8_scatter_escapes.argtypes = [vp, i32, i64, vp, vp, i64, vp]
     lib.qvb8_certify.argtypes = [vp, i32, vp, i32, i64, ctypes.c_float, vp, vp]
     lib.qvb8_sat_half.argtypes = [vp, i32, i64, vp, vp]

@@ -4,9 +4,9 @@
     spec = get_format(manifest["format"])
     lin  = spec.linear.from_packfile(path, device=dev)
 
-Entries: "qvb8" / "qvband" (the container's file extension) and "qvb8r".  There is no CPU reader and no embedding class in
-this build (`cpu_linear`, `embedding` are None): a caller that needs one gets a clear error from `require`, never another
-format's class.
+Entries: "qvb8" / "qvband" (the container's file extension) and "qvb8r".  There is no CPU reader in this build and no
+embedding class for "qvb8r" (`cpu_linear`, its `embedding` are None): a caller that needs one gets a clear error from
+`require`, never another format's class.
 """
 from __future__ import annotations
 
@@ -39,6 +39,7 @@ def _build_registry() -> None:
     import torch
     from qvb8_amd import ext_qvb8 as ext
     from qvb8_amd.formats.qvb8.backends_experts import QVBandExpertsV8
+    from qvb8_amd.formats.qvb8.embedding import QVBandEmbeddingV8
     from qvb8_amd.formats.qvb8.fuse import fuse_same_input
     from qvb8_amd.formats.qvb8.module import QVBandLinearV8
     from qvb8_amd.formats.qvb8r.module import QVBandLinearV8R
@@ -46,7 +47,7 @@ def _build_registry() -> None:
     def _decode_v8(lin):
         return ext.decode(lin.ids, lin.min_s, lin.nbits, lin.bit_off, lin.in_features, lin.tau_s, lin.esc_idx, lin.esc_vals)
 
-    _REGISTRY["qvb8"] = FormatSpec("qvb8", QVBandLinearV8, None, QVBandExpertsV8, decoder=_decode_v8, finalize=fuse_same_input)
+    _REGISTRY["qvb8"] = FormatSpec("qvb8", QVBandLinearV8, QVBandEmbeddingV8, QVBandExpertsV8, decoder=_decode_v8, finalize=fuse_same_input)
     _REGISTRY["qvband"] = dataclasses.replace(_REGISTRY["qvb8"], name="qvband")
     _REGISTRY["qvb8r"] = FormatSpec("qvb8r", QVBandLinearV8R, None, None, decoder=lambda lin: lin.dense(torch.float32))
 

@@ -57,64 +57,102 @@ template <> struct OutPack<2> {
     }
 };
 
-template <int NB, int J0, int J1>
+// FMA: the value of a linear layer's weight, fmaf(id, tau_s, min_s) (one rounding).  !FMA: the value the embedding
+// lookup of the reference computes, min_s + id * tau_s as two fp32 operations (two roundings).
+template <bool FMA>
+__device__ __forceinline__ float band_value(uint32_t id, float ts, float m) {
+#pragma clang fp contract(off)                  // the two-step form must stay a multiply and an add
+    if constexpr (FMA) return __builtin_fmaf((float)id, ts, m);
+    else { const float prod = (float)id * ts; return m + prod; }
+}
+
+template <int NB, bool FMA, int J0, int J1>
 __device__ __forceinline__ void restore_fields(const uint32_t (&w)[kMaxFastNb], float ts, float m, float (&v)[32]) {
     if constexpr (J0 < J1) {
-        v[J0] = __builtin_fmaf((float)field_of<NB, J0>(w), ts, m);
-        restore_fields<NB, J0 + 1, J1>(w, ts, m, v);
+        v[J0] = band_value<FMA>(field_of<NB, J0>(w), ts, m);
+        restore_fields<NB, FMA, J0 + 1, J1>(w, ts, m, v);
     }
 }
 
-template <int DT, int NB>
+template <int DT, int NB, bool FMA>
 __device__ __forceinline__ void restore_item_fast(const uint8_t* __restrict__ ids, int64_t row_byte, int slice,
                                                   float ts, float m, void* out, int64_t out_index) {
     uint32_t w[kMaxFastNb];
     load_slice<NB>(reinterpret_cast<const uint32_t*>(ids + row_byte) + (int64_t)slice * NB, w);
     float v[32];
-    restore_fields<NB, 0, 32>(w, ts, m, v);
+    restore_fields<NB, FMA, 0, 32>(w, ts, m, v);
     OutPack<DT>::store(out, out_index, v);
 }
 
 struct DecodeArgs {
     const uint8_t* ids; const float* min_s; const float* tau_s; const uint8_t* nbits; const int64_t* bit_off;
     void* out; int64_t ids_bytes; int64_t n_items; int Q; int P; int C;
+    // row lookup only: the rows wanted (output row i is row rows[i] of the pack) and the escapes of the whole pack
+    const int64_t* rows; const int64_t* esc_idx; const float* esc_vals; int64_t n_esc;
 };
 
-// One wave per item; 4 waves per workgroup.
-template <int DT>
+// One wave per item; 4 waves per workgroup.  LOOKUP: output row i is row rows[i] of the pack (any order, repeats allowed;
+// a row number outside 0..Q-1 gives a row of NaN), values are min_s + id * tau_s in two roundings, and the escapes of
+// the row overwrite the band values (a binary search of the ascending flat positions finds the item's range).
+template <int DT, bool LOOKUP>
 __global__ void __launch_bounds__(256) decode_kernel(DecodeArgs a) {
+    constexpr bool FMA = !LOOKUP;
     const int lane = threadIdx.x & 63;
     const int64_t item = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (item >= a.n_items) return;
-    const int q = (int)(item / a.C), c = (int)(item - (int64_t)q * a.C);
+    const int64_t orow = item / a.C;
+    const int c = (int)(item - orow * a.C);
+    int64_t q64 = orow;
+    if constexpr (LOOKUP) q64 = a.rows[orow];
+    const bool row_ok = q64 >= 0 && q64 < a.Q;
+    const int q = row_ok ? (int)q64 : 0;
     const int nb = __builtin_amdgcn_readfirstlane((int)a.nbits[q]);
     const int64_t bit0 = a.bit_off[q];
     const float ts = a.tau_s[q], m = a.min_s[q];
     const int col0 = c * kChunk;
     const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
     const int64_t row_bits = (int64_t)nb * a.P;
-    const bool in_bounds = nb >= 1 && nb <= 14 && bit0 >= 0 && ((bit0 + row_bits + 7) >> 3) + 8 <= a.ids_bytes;
+    const bool in_bounds = row_ok && nb >= 1 && nb <= 14 && bit0 >= 0 && ((bit0 + row_bits + 7) >> 3) + 8 <= a.ids_bytes;
+    // the lane's 32 values go out as 16-byte stores: the output row must start on 16 bytes as well
     const bool fast = in_bounds && (a.P % kFieldsPerLane) == 0 && (bit0 & 31) == 0 && nb >= 4 && nb <= kMaxFastNb;
+    const int col_end = min(a.P, col0 + kChunk);
     if (fast) {
         const int col = col0 + lane * kFieldsPerLane;
         if (col < a.P) {
-            const int64_t oi = (int64_t)q * a.P + col;
+            const int64_t oi = orow * a.P + col;
             const int slice = col / kFieldsPerLane;
             switch (nb) {
-                case 4: restore_item_fast<DT, 4>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
-                case 5: restore_item_fast<DT, 5>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
-                case 6: restore_item_fast<DT, 6>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
-                case 7: restore_item_fast<DT, 7>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
-                default: restore_item_fast<DT, 8>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
+                case 4: restore_item_fast<DT, 4, FMA>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
+                case 5: restore_item_fast<DT, 5, FMA>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
+                case 6: restore_item_fast<DT, 6, FMA>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
+                case 7: restore_item_fast<DT, 7, FMA>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
+                default: restore_item_fast<DT, 8, FMA>(a.ids, bit0 >> 3, slice, ts, m, a.out, oi); break;
             }
         }
-        return;
+    } else {
+        for (int col = col0 + lane; col < col_end; col += kWave) {
+            float v = __builtin_nanf("");
+            if (in_bounds) v = band_value<FMA>(load_field(a.ids, bit0 + (int64_t)col * nb, nb, clamp_byte), ts, m);
+            store_from_f32<DT>(a.out, orow * a.P + col, v);
+        }
     }
-    const int col_end = min(a.P, col0 + kChunk);
-    for (int col = col0 + lane; col < col_end; col += kWave) {
-        float v = __builtin_nanf("");
-        if (in_bounds) v = __builtin_fmaf((float)load_field(a.ids, bit0 + (int64_t)col * nb, nb, clamp_byte), ts, m);
-        store_from_f32<DT>(a.out, (int64_t)q * a.P + col, v);
+    if constexpr (LOOKUP) {
+        if (a.n_esc == 0 || !row_ok) return;
+        const int64_t lo_pos = q64 * a.P + col0, hi_pos = q64 * a.P + col_end;
+        int64_t lo = 0, hi = a.n_esc;                              // first escape at or after lo_pos
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (a.esc_idx[mid] < lo_pos) lo = mid + 1; else hi = mid;
+        }
+        if (lo >= a.n_esc || a.esc_idx[lo] >= hi_pos) return;
+        // the band values of this item are the wave's own earlier stores: wait until all of them have been
+        // acknowledged (vmcnt(0); the other counters stay unconstrained) before some are overwritten
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        for (int64_t e = lo + lane; e < a.n_esc; e += kWave) {
+            const int64_t at = a.esc_idx[e];
+            if (at >= hi_pos) break;
+            store_from_f32<DT>(a.out, orow * a.P + (at - q64 * a.P), a.esc_vals[e]);
+        }
     }
 }
 
@@ -511,15 +549,44 @@ extern "C" int qvb8_decode(const uint8_t* ids, int64_t ids_bytes, const float* m
     a.ids = ids; a.min_s = min_s; a.tau_s = tau_s; a.nbits = nbits; a.bit_off = bit_off; a.out = out;
     a.ids_bytes = ids_bytes; a.Q = (int)Q; a.P = (int)P; a.C = (int)((P + kChunk - 1) / kChunk);
     a.n_items = Q * a.C;
+    a.rows = nullptr; a.esc_idx = nullptr; a.esc_vals = nullptr; a.n_esc = 0;
     const int64_t blocks = (a.n_items + 3) / 4;
     if (blocks > 0x7fffffff) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_decode: tensor too large for one launch");
     hipStream_t s = (hipStream_t)stream;
     switch (out_dtype) {
-        case QVB8_F32: hipLaunchKernelGGL(decode_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, s, a); break;
-        case QVB8_F16: hipLaunchKernelGGL(decode_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, s, a); break;
-        default: hipLaunchKernelGGL(decode_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, s, a); break;
+        case QVB8_F32: hipLaunchKernelGGL((decode_kernel<0, false>), dim3((unsigned)blocks), dim3(256), 0, s, a); break;
+        case QVB8_F16: hipLaunchKernelGGL((decode_kernel<1, false>), dim3((unsigned)blocks), dim3(256), 0, s, a); break;
+        default: hipLaunchKernelGGL((decode_kernel<2, false>), dim3((unsigned)blocks), dim3(256), 0, s, a); break;
     }
     return host::check_launch("qvb8_decode");
+}
+
+extern "C" int qvb8_lookup_rows(const int64_t* rows, int64_t n_rows, const uint8_t* ids, int64_t ids_bytes, const float* min_s,
+                                const float* tau_s, const uint8_t* nbits, const int64_t* bit_off, int64_t Q, int64_t P,
+                                const int64_t* esc_idx, const float* esc_vals, int64_t n_esc, int out_dtype, void* out,
+                                void* stream) {
+    if (int rc = check_pack(ids, ids_bytes, min_s, tau_s, nbits, bit_off, Q, P, "qvb8_lookup_rows")) return rc;
+    if (out_dtype < 0 || out_dtype > 2) return host::fail(QVB8_ERR_ARG, "qvb8_lookup_rows: out_dtype %d", out_dtype);
+    if (n_rows < 0 || n_esc < 0) return host::fail(QVB8_ERR_ARG, "qvb8_lookup_rows: negative size");
+    if (n_rows == 0 || P == 0) return QVB8_OK;
+    if (Q == 0) return host::fail(QVB8_ERR_ARG, "qvb8_lookup_rows: rows wanted from an empty table");
+    if (!rows) return host::fail(QVB8_ERR_ARG, "qvb8_lookup_rows: null rows");
+    if (n_esc > 0 && (!esc_idx || !esc_vals)) return host::fail(QVB8_ERR_ARG, "qvb8_lookup_rows: null escape arrays");
+    if (!out || (reinterpret_cast<uintptr_t>(out) & 15u)) return host::fail(QVB8_ERR_ARG, "qvb8_lookup_rows: out must be 16-byte aligned");
+    DecodeArgs a;
+    a.ids = ids; a.min_s = min_s; a.tau_s = tau_s; a.nbits = nbits; a.bit_off = bit_off; a.out = out;
+    a.ids_bytes = ids_bytes; a.Q = (int)Q; a.P = (int)P; a.C = (int)((P + kChunk - 1) / kChunk);
+    a.n_items = n_rows * a.C;
+    a.rows = rows; a.esc_idx = esc_idx; a.esc_vals = esc_vals; a.n_esc = n_esc;
+    const int64_t blocks = (a.n_items + 3) / 4;
+    if (blocks > 0x7fffffff) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_lookup_rows: too many rows for one launch");
+    hipStream_t s = (hipStream_t)stream;
+    switch (out_dtype) {
+        case QVB8_F32: hipLaunchKernelGGL((decode_kernel<0, true>), dim3((unsigned)blocks), dim3(256), 0, s, a); break;
+        case QVB8_F16: hipLaunchKernelGGL((decode_kernel<1, true>), dim3((unsigned)blocks), dim3(256), 0, s, a); break;
+        default: hipLaunchKernelGGL((decode_kernel<2, true>), dim3((unsigned)blocks), dim3(256), 0, s, a); break;
+    }
+    return host::check_launch("qvb8_lookup_rows");
 }
 
 extern "C" int qvb8_scatter_escapes(void* out, int out_dtype, int64_t n_out, const int64_t* esc_idx,

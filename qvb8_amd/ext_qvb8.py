@@ -8,7 +8,7 @@ allocator, like the reference's torch::empty) and for the current stream only.
     decode(ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)       (Q, P) fp16
     decode_bf16(...)     (Q, P) bf16
 Additions without a counterpart there: decode_f32 (the fp32 band value), certify,
-saturating_half.
+saturating_half, lookup_rows (the embedding read, which the reference does in torch).
 """
 from __future__ import annotations
 
@@ -74,6 +74,30 @@ def decode_bf16(ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)
 def decode_f32(ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
     """Dense (Q, P) fp32 band values (what the GEMV multiplies), escapes exact."""
     return _decode_to(_lib.F32, torch.float32, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals)
+
+
+def lookup_rows(rows, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, out_dtype=torch.float32):
+    """(n, P) rows `rows` of the table in `out_dtype`: min_s + id * tau_s in two fp32 roundings, then the rows'
+    escapes written over it -- QVBandEmbeddingV8._decode_rows plus the escape loop of its forward
+    (formats/qvb8/embedding.py:92-152) as one launch.  A row number outside the table gives a row of NaN."""
+    lib = _lib.load()
+    Q = _check_pack(ids, min_s, row_nbits, row_bit_off, tau_s)
+    n_esc = _check_escapes(esc_idx, esc_vals)
+    _lib.require_cuda(rows)
+    if rows.dtype != torch.int64:
+        raise RuntimeError("rows must be int64")
+    rows = rows.reshape(-1).contiguous()
+    ids, min_s, tau_s = ids.contiguous(), min_s.contiguous(), tau_s.contiguous()
+    row_nbits, row_bit_off = row_nbits.contiguous(), row_bit_off.contiguous()
+    code = _lib.dtype_code(out_dtype)
+    with torch.cuda.device(ids.device):
+        out = torch.empty((rows.numel(), int(P)), dtype=out_dtype, device=ids.device)
+        ei = esc_idx.contiguous() if n_esc else None
+        ev = esc_vals.contiguous() if n_esc else None
+        _lib._check(lib.qvb8_lookup_rows(_lib.ptr(rows), rows.numel(), _lib.ptr(ids), ids.numel(), _lib.ptr(min_s),
+                                         _lib.ptr(tau_s), _lib.ptr(row_nbits), _lib.ptr(row_bit_off), Q, int(P),
+                                         _lib.ptr(ei), _lib.ptr(ev), n_esc, code, _lib.ptr(out), _lib.stream_of(ids)), lib)
+    return out
 
 
 def certify(restored: torch.Tensor, original: torch.Tensor, tau: float):

@@ -38,17 +38,19 @@ def apply_keeping_fp32_metadata(module: nn.Module, fn, recurse=True):
     """nn.Module._apply with the fp32 decode metadata protected from dtype casts: a `.to(bfloat16)` must not round
     min_s / tau_s / escape values (that would move weights by up to ~tau); only the device follows
     (reference: module.py:43-56)."""
-    keep = {n: module._buffers[n] for n in FP32_METADATA if module._buffers.get(n) is not None}
-    for n in keep:
-        module._buffers[n] = None
+    held = {}
+    for name in FP32_METADATA:
+        buf = module._buffers.get(name)
+        if buf is not None:
+            held[name] = buf
+            module._buffers[name] = None              # nn.Module._apply skips absent buffers
     try:
-        out = nn.Module._apply(module, fn, recurse)
+        result = nn.Module._apply(module, fn, recurse)
     finally:
-        ref = module._buffers.get("ids")
-        dev = ref.device if ref is not None else (next(iter(keep.values())).device if keep else None)
-        for n, b in keep.items():
-            module._buffers[n] = b.to(dev)
-    return out
+        anchor = module._buffers.get("ids")           # the metadata lives where the packed ids went
+        for name, buf in held.items():
+            module._buffers[name] = buf if anchor is None else buf.to(anchor.device)
+    return result
 
 
 class QVBandLinearV8(nn.Module):

@@ -190,3 +190,60 @@ def test_moe_reference_tiny_brute_force():
         g, u = y[:I], y[I:]
         want += w[t, j] * (Wdn[e].astype(np.float64) @ (g / (1 + np.exp(-g)) * u))
     assert np.allclose(out[t], want, rtol=1e-12)
+
+
+def test_embedding_rows_two_roundings_closed_form():
+    """The lookup value is fl(min + fl(id * tau)): checked against float64 arithmetic rounded explicitly at each step
+    (id * tau is exact in float64: 14 + 24 bits; min + product of two floats is exact in float64 unless the exponents
+    are more than 29 apart, which these magnitudes never are)."""
+    rng = np.random.default_rng(5)
+    Q, P = 40, 96
+    nb = rng.integers(1, 15, Q)
+    ids = np.stack([rng.integers(0, 1 << int(w), P) for w in nb])
+    min_s = rng.normal(0, 0.1, Q).astype(np.float32)
+    tau_s = (np.abs(rng.normal(2e-3, 1e-3, Q)) + 1e-6).astype(np.float32)
+    rows = np.array([3, 3, 39, 0, 17, 3], np.int64)
+    got = O.embedding_rows(rows, min_s, tau_s, ids, P)
+    prod = (ids[rows].astype(np.float64) * tau_s[rows].astype(np.float64)[:, None]).astype(np.float32)
+    want = (min_s[rows].astype(np.float64)[:, None] + prod.astype(np.float64)).astype(np.float32)
+    assert got.dtype == np.float32 and got.shape == (6, P)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # from the fused value by at most the two rounding errors (half a unit of the product, half a unit of the sum,
+    # plus the fused value's own half unit), and not always equal to it
+    fused = O.band_values(min_s, tau_s, ids)[rows].astype(np.float64)
+    bound = 0.5 * np.spacing(np.abs(prod)).astype(np.float64) + np.spacing(np.maximum(np.abs(got), np.abs(fused).astype(np.float32))).astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - fused) <= bound)
+    assert np.any(got.astype(np.float64) != fused)
+
+
+def test_embedding_rows_known_answer_differs_from_fused():
+    """id = 3, tau = 1 + 2^-23, min = -3: the product 3 + 3*2^-23 needs 26 bits and rounds to 3 + 2^-21 (tie to even),
+    so the two-step value is 2^-21 while the fused one keeps the exact 3*2^-23."""
+    tau = np.array([1.0 + 2.0 ** -23], np.float32)
+    mn = np.array([-3.0], np.float32)
+    ids = np.array([[3]])
+    two = O.embedding_rows([0], mn, tau, ids, 1)
+    one = O.band_values(mn, tau, ids)
+    assert two[0, 0] == np.float32(2.0 ** -21)
+    assert one[0, 0] == np.float32(3 * 2.0 ** -23)
+
+
+def test_embedding_rows_escapes_and_narrowing():
+    rng = np.random.default_rng(6)
+    Q, P = 8, 32
+    ids = rng.integers(0, 64, (Q, P))
+    min_s = rng.normal(0, 0.1, Q).astype(np.float32)
+    tau_s = np.full(Q, 2e-3, np.float32)
+    esc_idx = np.array([2 * P + 5, 2 * P + 31, 7 * P + 0], np.int64)
+    esc_vals = np.array([0.75, -1.5, 3.0e-5], np.float32)
+    rows = np.array([7, 2, 2, 1], np.int64)
+    out = O.embedding_rows(rows, min_s, tau_s, ids, P, esc_idx, esc_vals)
+    assert out[0, 0] == esc_vals[2] and out[1, 5] == esc_vals[0] and out[2, 31] == esc_vals[1]
+    plain = O.embedding_rows(rows, min_s, tau_s, ids, P)
+    mask = np.ones_like(out, bool)
+    mask[0, 0] = mask[1, 5] = mask[1, 31] = mask[2, 5] = mask[2, 31] = False
+    assert np.array_equal(out[mask], plain[mask])
+    h = O.embedding_rows(rows, min_s, tau_s, ids, P, esc_idx, esc_vals, dtype="fp16")
+    assert np.array_equal(h, out.astype(np.float16).astype(np.float32))
+    b = O.embedding_rows(rows, min_s, tau_s, ids, P, esc_idx, esc_vals, dtype="bf16")
+    assert np.array_equal(b, torch.from_numpy(out).to(torch.bfloat16).float().numpy())
