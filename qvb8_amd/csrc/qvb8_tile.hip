@@ -209,7 +209,8 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
     uint4* s_fin = reinterpret_cast<uint4*>(smem);                                       // [rows_cap]
     uint64_t* s_loc = reinterpret_cast<uint64_t*>(s_fin + rows_cap);                     // [n_waves][wave_rows]
     float* sxs = reinterpret_cast<float*>(s_loc + (size_t)n_waves * wave_rows);          // [ranges][TM]
-    float* part = sxs + (size_t)ranges * TM;                                             // [rows_cap][ranges][TM]
+    float* part = sxs + (size_t)ranges * TM;                                             // [rows_cap][ranges][M]
+    const int MS = a.M;                                       // a row's partial sums hold M tokens, not the TM the tile could take
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -255,11 +256,21 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
     // Requests the lane's slices of all T steps of the wave's tile number tk: 2T loads, none under a branch, all from
     // addresses inside the buffer (lanes whose row is not sliced, and steps past the end of the row, read the first
     // 32 bytes of `ids`).  Returns width | 1 << 8 for a sliced row, 0 otherwise.
+    // Requests go out in a lane order that the L1 can merge: lane l asks for chunk l % 4 of row l / 4, so four
+    // neighbouring lanes read 4 x 4*nb consecutive bytes of one row (in operand order -- lane = row + 16 * chunk --
+    // every lane is a row of its own: measured 61 L1 accesses per request instruction against 25 this way, and about
+    // 1.3 % of the decode step).  to_operand then moves a register from request order to operand order across the wave.
+    const int lr = lane >> 2, lk = lane & 3;
+    const int pull = 4 * (4 * r + kg);                         // byte address of the lane whose request holds this lane's operand
+    auto to_operand = [&](const uint4& v) -> uint4 {
+        return uint4{(uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y),
+                     (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w)};
+    };
     auto issue_tile = [&](int tk, int step0, uint4 (&wlo)[T], uint4 (&whi)[T]) -> uint32_t {
-        const uint64_t rec = my_loc[tk * kTileRows + r];
+        const uint64_t rec = my_loc[tk * kTileRows + lr];
         const uint32_t nb = (uint32_t)(rec >> 48) & 0xFFu, kind = (uint32_t)(rec >> 56) & 3u;
         const bool row_sliced = kind == 1u;
-        const uint64_t row_off = ((rec & kRowOffMask) >> 3) + (uint64_t)(step0 * 4 + kg) * (4u * nb);
+        const uint64_t row_off = ((rec & kRowOffMask) >> 3) + (uint64_t)(step0 * 4 + lk) * (4u * nb);
         const uint32_t step_bytes = 16u * nb;
         const uint32_t tail = row_sliced ? 4u * (nb - 4u) : 16u;
 #pragma unroll
@@ -269,7 +280,8 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
             wlo[it] = *reinterpret_cast<const uint4*>(a.ids + off);
             whi[it] = *reinterpret_cast<const uint4*>(a.ids + off + tail);
         }
-        return row_sliced ? (nb | (1u << 8)) : 0u;
+        const uint64_t rec2 = my_loc[tk * kTileRows + r];       // what the lane will decode: its operand row's width
+        return ((uint32_t)(rec2 >> 56) & 3u) == 1u ? (((uint32_t)(rec2 >> 48) & 0xFFu) | (1u << 8)) : 0u;
     };
 
     for (int panel = 0; panel < a.panels; ++panel) {
@@ -348,7 +360,7 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
 #pragma unroll
             for (int it = 0; it < T; ++it) {
                 v4u_t b[4];
-                const uint4 lo = wlo[it], hi = whi[it];
+                const uint4 lo = to_operand(wlo[it]), hi = to_operand(whi[it]);
                 if (uniform) {
                     switch (info0 & 0xFFu) {
                         case 7: decode_slice<7, BF>(lo, hi, b); break;
@@ -400,7 +412,7 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
                     float v = __builtin_fmaf(-F::bias, sx[nt][e], acc[nt][e]);
                     if constexpr (BF) v = __builtin_fmaf(kTopBitScale, acc_top[nt][e], v);
                     if (t < a.M) {
-                        float* dst = part + ((size_t)lrow * ranges + range) * TM + t;
+                        float* dst = part + ((size_t)lrow * ranges + range) * MS + t;
                         *dst = first_panel ? v : *dst + v;
                     }
                 }
@@ -429,7 +441,7 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
                     }
                     const float tot = wave_sum(sacc);
                     // the sliced pass stored this wave's value for the row already (zero contribution plus earlier panels)
-                    if (lane == 0) part[((size_t)lr2 * ranges + range) * TM + t] += tot;
+                    if (lane == 0) part[((size_t)lr2 * ranges + range) * MS + t] += tot;
                 }
             }
         }
@@ -446,7 +458,7 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
         if (f.z >= (uint32_t)a.Q) continue;
         double dsum = 0.0, xsum = 0.0;
         for (int w = 0; w < valid_ranges; ++w) {
-            dsum += (double)part[((size_t)rl * ranges + w) * TM + t];
+            dsum += (double)part[((size_t)rl * ranges + w) * MS + t];
             xsum += (double)sxs[w * TM + t];
         }
         a.Y[(size_t)t * a.Q + f.z] = (float)((double)__uint_as_float(f.x) * dsum + (double)__uint_as_float(f.y) * xsum);
@@ -690,7 +702,7 @@ struct TilePlan { int W, G, panels, TW, threads; size_t lds; unsigned blocks; };
 
 constexpr size_t kTileLdsLimit = 128 * 1024;
 
-bool plan_tile(int NT, int T, int64_t Q, int64_t P, TilePlan& pl) {
+bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl) {
     const int n_steps = (int)(P / kStepCols);
     const int ranges = (n_steps + T - 1) / T;                 // column ranges of T steps
     const int max_waves = 8;
@@ -710,20 +722,30 @@ bool plan_tile(int NT, int T, int64_t Q, int64_t P, TilePlan& pl) {
     const size_t TM = 16 * (size_t)NT, rg = (size_t)pl.W;
     for (;;) {
         const size_t rows = (size_t)tw * kTileRows;
-        pl.lds = rows * 16 + (size_t)pl.W * pl.G * (tw / pl.G) * kTileRows * 8 + rg * TM * 4 + rows * rg * TM * 4;
+        pl.lds = rows * 16 + (size_t)pl.W * pl.G * (tw / pl.G) * kTileRows * 8 + rg * TM * 4 + rows * rg * (size_t)M * 4;
         if (pl.lds <= kTileLdsLimit || tw <= pl.G) break;
         tw -= pl.G;
     }
     if (pl.lds > kTileLdsLimit) return false;
+    // more workgroups than the target (LDS or the thread count capped the tiles of one): a whole number of rounds over the
+    // CUs, the tiles spread evenly -- 1035 workgroups on 256 CUs would leave the fifth round to 11 of them
+    int64_t blocks = (tiles + tw - 1) / tw;
+    if (blocks > target) {
+        blocks = (blocks + target - 1) / target * target;
+        int64_t even = (tiles + blocks - 1) / blocks;
+        even = (even + pl.G - 1) / pl.G * pl.G;
+        if (even < tw) tw = even;
+        blocks = (tiles + tw - 1) / tw;
+    }
     pl.TW = (int)tw;
-    pl.blocks = (unsigned)((tiles + tw - 1) / tw);
+    pl.blocks = (unsigned)blocks;
     return true;
 }
 
 template <int NT, int T, bool BF, bool XC>
 int launch_tile(TileArgs& a, hipStream_t s) {
     TilePlan pl;
-    if (!plan_tile(NT, T, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
+    if (!plan_tile(NT, T, a.M, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
     a.W = pl.W; a.G = pl.G; a.panels = pl.panels; a.TW = pl.TW;
     static bool attr[64] = {false};                           // per device: the attribute belongs to the device's copy of the kernel
     int dev = 0;
