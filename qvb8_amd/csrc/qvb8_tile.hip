@@ -566,8 +566,16 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
         const int pos = pos0 + wave * kGemmWaveRows + rt * 32 + n;
         row_ok[rt] = pos < pos_end;
         row_pos[rt] = row_ok[rt] ? pos : pos_end - 1;
-        row_ptr[rt] = a.ids + run_byte0 + (uint64_t)(row_pos[rt] - run_first) * ((uint64_t)a.P * NB / 8) + (uint32_t)kh * (4u * NB);
+        // requests go out in the order lane = 2 * row + half, so that neighbouring lanes read neighbouring bytes
+        // (fewer L1 accesses per request); to_operand moves the registers into operand order (lane = row + 32 * half)
+        const int rpos = min(pos0 + wave * kGemmWaveRows + rt * 32 + (lane >> 1), pos_end - 1);
+        row_ptr[rt] = a.ids + run_byte0 + (uint64_t)(rpos - run_first) * ((uint64_t)a.P * NB / 8) + (uint32_t)(lane & 1) * (4u * NB);
     }
+    const int pull = 4 * (2 * n + kh);
+    auto to_operand = [pull](const uint4& v) -> uint4 {
+        return uint4{(uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y),
+                     (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w)};
+    };
     uint4 raw[4][2][2];                            // [step % 4][row tile][first / last four dwords]
     const uint8_t* const rp0 = row_ptr[0];
     const uint8_t* const rp1 = row_ptr[1];
@@ -614,7 +622,7 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
             if (h == 0) request_x((u0 >> 1) + buf + 1, xg);
             v4u_t b[2][4];
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) decode_slice<NB, BF>(raw[k][rt][0], raw[k][rt][1], b[rt]);
+            for (int rt = 0; rt < 2; ++rt) decode_slice<NB, BF>(to_operand(raw[k][rt][0]), to_operand(raw[k][rt][1]), b[rt]);
             request_ids(u0 + k + 4, raw[k]);
             __builtin_amdgcn_sched_barrier(0);                             // the requests stay ahead of the products
             const unsigned char* xb = xs + (size_t)buf * TMK * kGemmXStride + (size_t)n * kGemmXStride + 2 * (64 * h + 32 * kh);
@@ -773,7 +781,11 @@ int64_t align256i(int64_t n) { return (n + 255) & ~(int64_t)255; }
 // ceil(Q / 256): up to two more exist when the rows have several widths).
 GemmPlan plan_gemm(int64_t M, int64_t Q, int64_t P) {
     GemmPlan g;
-    g.MT = 2;                                          // 64 rows of X per workgroup: measured faster than 128 (one wave per SIMD) at every M
+    // 64 rows of X per workgroup (two waves per SIMD) up to 192 rows; beyond, 128 rows per workgroup read the ids half as
+    // often (measured at M = 256: 10 % faster although only one wave per SIMD fits)
+    const int mt_env = host::env_int("QVB8_GEMM_MT", 0);
+    g.MT = mt_env == 2 || mt_env == 4 ? mt_env : (M > 192 ? 4 : 2);
+    if (M <= 64) g.MT = 2;
     const int TMK = 32 * g.MT;
     g.tok_blocks = (int)((M + TMK - 1) / TMK);
     g.row_blocks = (int)((Q + kGemmRows - 1) / kGemmRows);
@@ -917,7 +929,8 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         ga.blocks2 = ga.blocks1 + (rows1 + kGemmRows - 1) / kGemmRows;
         const int row_blocks = ga.blocks2 + (rows2 + kGemmRows - 1) / kGemmRows;
         ga.widths = (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16);
-        rc = mode == 2 ? launch_gemm<2, true>(ga, g, row_blocks, s) : launch_gemm<2, false>(ga, g, row_blocks, s);
+        if (g.MT == 4) rc = mode == 2 ? launch_gemm<4, true>(ga, g, row_blocks, s) : launch_gemm<4, false>(ga, g, row_blocks, s);
+        else rc = mode == 2 ? launch_gemm<2, true>(ga, g, row_blocks, s) : launch_gemm<2, false>(ga, g, row_blocks, s);
         if (rc) return rc;
         if (g.splits > 1) {
             const int64_t n = M * Q;
