@@ -30,6 +30,7 @@ typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
 typedef float v16f_t __attribute__((ext_vector_type(16)));
 
 constexpr int kTileRows = 16;
+constexpr int kTileXPieces = 4;         // 16-byte pieces of X a thread may stage when X goes through LDS
 constexpr int kStepCols = 128;          // columns one wave step covers (4 lane groups x 32 ids)
 
 template <bool BF> struct Fmt;
@@ -186,7 +187,7 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
 // slots.  After one barrier the whole workgroup combines the column ranges of each row in a fixed order.
 // The kernel's arguments are 56 bytes of scalars (measured: every further 64 bytes of kernel arguments cost about a
 // microsecond per launch): fin follows loc, n_steps follows P, the small counts share one word.
-template <int NT, int T, bool BF, bool XC>
+template <int NT, int T, bool BF, bool XC, bool XL = false>
 __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ ids,
                                                    const uint64_t* __restrict__ loc, float* __restrict__ Y, int64_t ids_bytes,
                                                    int Q, int P, uint32_t counts, int TW, int first1, int first2, uint32_t widths) {
@@ -216,6 +217,18 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = wave / a.W, wc = wave - g * a.W;
     const int r = lane & 15, kg = lane >> 4;
+    // XL: the whole of X (at most kTileXPieces 16-byte pieces per thread) goes through LDS once: every thread requests its
+    // pieces before anything else, the first tile's ids follow at once, and the workgroup shares X after one barrier --
+    // so the trip of the activations and the first trip of the ids overlap, and later panels need no trip for theirs.
+    unsigned char* xs = reinterpret_cast<unsigned char*>(part + (size_t)rows_cap * ranges * MS);     // [M][P] in operand format
+    const int x_pieces = (a.M * a.P) >> 3;
+    v4u_t xg[kTileXPieces];
+    if constexpr (XL) {
+        const v4u_t* xsrc = reinterpret_cast<const v4u_t*>(a.X);
+#pragma unroll
+        for (int i = 0; i < kTileXPieces; ++i) xg[i] = xsrc[min(tid + i * (int)blockDim.x, x_pieces - 1)];
+        __builtin_amdgcn_sched_barrier(0);                     // these requests stay where they are: ahead of everything
+    }
     // The workgroup's local tile lt is global tile lt * gridDim.x + blockIdx.x: at any moment the workgroups of the
     // grid read neighbouring tiles, so the whole chip walks through memory together (spread over all channels).
     const int total_tiles = (a.Q + kTileRows - 1) / kTileRows;
@@ -248,7 +261,15 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
     }
     // ---- what the end needs for row `tid`: requested now, parked in registers, put in LDS before the barrier ----
     uint4 e_fin = {0u, 0u, 0xffffffffu, 0u};
-    if (tid < tiles_here * kTileRows && local_to_pos(tid) < a.Q) e_fin = a.fin[local_to_pos(tid)];
+    if constexpr (XL) {
+        // no request under a branch from here to the barrier: the counted waits for the activations must know exactly
+        // how many requests follow them
+        const bool has_row = tid < tiles_here * kTileRows && local_to_pos(tid) < a.Q;
+        const uint4 f = a.fin[has_row ? local_to_pos(tid) : 0];
+        if (has_row) e_fin = f;
+    } else {
+        if (tid < tiles_here * kTileRows && local_to_pos(tid) < a.Q) e_fin = a.fin[local_to_pos(tid)];
+    }
 
     const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
     uint4 wlo[T], whi[T];
@@ -266,8 +287,9 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
         return uint4{(uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y),
                      (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w)};
     };
-    auto issue_tile = [&](int tk, int step0, uint4 (&wlo)[T], uint4 (&whi)[T]) -> uint32_t {
-        const uint64_t rec = my_loc[tk * kTileRows + lr];
+    auto issue_tile = [&](int tk, int step0, uint4 (&wlo)[T], uint4 (&whi)[T], bool has_tile = true) -> uint32_t {
+        const uint64_t rec_read = my_loc[tk * kTileRows + lr];
+        const uint64_t rec = has_tile ? rec_read : 3ull << 56;  // a wave without tiles: no row, every request reads the buffer's start
         const uint32_t nb = (uint32_t)(rec >> 48) & 0xFFu, kind = (uint32_t)(rec >> 56) & 3u;
         const bool row_sliced = kind == 1u;
         const uint64_t row_off = ((rec & kRowOffMask) >> 3) + (uint64_t)(step0 * 4 + lk) * (4u * nb);
@@ -281,8 +303,28 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
             whi[it] = *reinterpret_cast<const uint4*>(a.ids + off + tail);
         }
         const uint64_t rec2 = my_loc[tk * kTileRows + r];       // what the lane will decode: its operand row's width
-        return ((uint32_t)(rec2 >> 56) & 3u) == 1u ? (((uint32_t)(rec2 >> 48) & 0xFFu) | (1u << 8)) : 0u;
+        return has_tile && ((uint32_t)(rec2 >> 56) & 3u) == 1u ? (((uint32_t)(rec2 >> 48) & 0xFFu) | (1u << 8)) : 0u;
     };
+
+    if constexpr (XL) {
+        info = issue_tile(0, wc * T, wlo, whi, n_tiles > 0);   // steps past the row's end read the buffer's start as well
+#pragma unroll
+        for (int i = 0; i < kTileXPieces; ++i) {
+            const int idx = tid + i * (int)blockDim.x;
+            v4u_t v = xg[i];
+            if constexpr (XC) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] = XI::pair(v[k]);
+            }
+            if (idx < x_pieces) reinterpret_cast<v4u_t*>(xs)[idx] = v;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // A bare barrier behind this wave's own LDS writes: __syncthreads() carries a release fence that would also wait
+        // for the ids just requested.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
 
     for (int panel = 0; panel < a.panels; ++panel) {
         const int step0 = (panel * a.W + wc) * T;             // first global step of this wave in this panel
@@ -303,16 +345,22 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
 #pragma unroll
                 for (int j = 0; j < 4; ++j) xa[nt][it][j] = v4u_t{0, 0, 0, 0};
                 if (active && t < a.M && (step0 + it) < a.n_steps) {
-                    const uint16_t* xp = a.X + (size_t)t * a.P + (size_t)(step0 + it) * kStepCols + kg * 32;
+                    const size_t at = (size_t)t * a.P + (size_t)(step0 + it) * kStepCols + kg * 32;
+                    if constexpr (XL) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const uint4 v = *reinterpret_cast<const uint4*>(xp + 8 * j);
-                        xa[nt][it][j] = v4u_t{v.x, v.y, v.z, v.w};
+                        for (int j = 0; j < 4; ++j) xa[nt][it][j] = *reinterpret_cast<const v4u_t*>(xs + 2 * at + 16 * j);
+                    } else {
+                        const uint16_t* xp = a.X + at;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const uint4 v = *reinterpret_cast<const uint4*>(xp + 8 * j);
+                            xa[nt][it][j] = v4u_t{v.x, v.y, v.z, v.w};
+                        }
                     }
                 }
             }
         }
-        if constexpr (XC) {                 // after ALL requests are out: narrowing inside the branches above would wait per branch
+        if constexpr (XC && !XL) {          // after ALL requests are out: narrowing inside the branches above would wait per branch
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -347,7 +395,7 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
         // before the activations, or right behind them -- was measured to cost about a microsecond per launch (the few
         // activation requests then compete with the flood of id requests of the whole chip).
         // Later panels' first ids are in flight already (requested at the end of the panel before).
-        if (n_mine > 0 && first_panel) info = issue_tile(0, step0, wlo, whi);
+        if constexpr (!XL) { if (n_mine > 0 && first_panel) info = issue_tile(0, step0, wlo, whi); }
 
         for (int tk = 0; tk < n_mine; ++tk) {
             v4f_t acc[NT], acc_top[NT];
@@ -709,6 +757,7 @@ namespace {
 struct TilePlan { int W, G, panels, TW, threads; size_t lds; unsigned blocks; };
 
 constexpr size_t kTileLdsLimit = 128 * 1024;
+constexpr size_t kTileXLdsLimit = 32 * 1024;     // X through LDS: up to this many bytes of activations on top
 
 bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl) {
     const int n_steps = (int)(P / kStepCols);
@@ -750,22 +799,27 @@ bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl) {
     return true;
 }
 
-template <int NT, int T, bool BF, bool XC>
+template <int NT, int T, bool BF, bool XC, bool XL = false>
 int launch_tile(TileArgs& a, hipStream_t s) {
     TilePlan pl;
     if (!plan_tile(NT, T, a.M, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
+    if constexpr (XL) {
+        const size_t x_bytes = (size_t)a.M * (size_t)a.P * 2;
+        if (x_bytes > kTileXLdsLimit || x_bytes / 16 > (size_t)kTileXPieces * pl.threads) return launch_tile<NT, T, BF, XC, false>(a, s);
+        pl.lds += x_bytes;
+    }
     a.W = pl.W; a.G = pl.G; a.panels = pl.panels; a.TW = pl.TW;
     static bool attr[64] = {false};                           // per device: the attribute belongs to the device's copy of the kernel
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: no current device");
     if (!attr[dev]) {
-        if (hipFuncSetAttribute((const void*)tile_kernel<NT, T, BF, XC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTileLdsLimit) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)tile_kernel<NT, T, BF, XC, XL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kTileLdsLimit + kTileXLdsLimit)) != hipSuccess)
             return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: cannot raise the kernel's LDS limit");
         attr[dev] = true;
     }
     if (pl.panels > 0xffff) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: rows too long");
     const uint32_t counts = (uint32_t)a.M | ((uint32_t)a.W << 8) | ((uint32_t)a.G << 12) | ((uint32_t)a.panels << 16);
-    hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s,
+    hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC, XL>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s,
                        a.X, a.ids, a.loc, a.Y, a.ids_bytes, a.Q, a.P, counts, a.TW, a.first1, a.first2,
                        (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16) | ((uint32_t)a.n_classes << 24));
     return host::check_launch("qvb8_mma");
@@ -942,7 +996,11 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     // rows of 33..40 steps (P = 5120): one panel of eight waves with five steps each instead of two panels of five waves
     // with four (measured on 27B-class shapes: 16 % faster; more steps per wave did not pay for longer rows)
     const int n_steps_all = (int)(P / kStepCols);
-    if (M <= 16 && n_steps_all > 32 && n_steps_all <= 40) rc = QVB8_TILE_LAUNCH(1, 5);
+#define QVB8_TILE_LAUNCH_XL(T_) (mode == 0 ? launch_tile<1, T_, false, false, true>(a, s) : mode == 1 ? launch_tile<1, T_, false, true, true>(a, s) : launch_tile<1, T_, true, false, true>(a, s))
+    const bool x_lds = M <= 16 && M * P * 2 <= (int64_t)kTileXLdsLimit && host::env_int("QVB8_TILE_X_LDS", 1) != 0;
+    if (x_lds) rc = n_steps_all > 32 && n_steps_all <= 40 ? QVB8_TILE_LAUNCH_XL(5) : QVB8_TILE_LAUNCH_XL(4);
+    else if (M <= 16 && n_steps_all > 32 && n_steps_all <= 40) rc = QVB8_TILE_LAUNCH(1, 5);
+#undef QVB8_TILE_LAUNCH_XL
     else if (M <= 16) rc = QVB8_TILE_LAUNCH(1, 4);
     else if (M <= 32) rc = QVB8_TILE_LAUNCH(2, 2);
     else rc = QVB8_TILE_LAUNCH(3, 2);
