@@ -35,7 +35,7 @@ LAYER_27B = (("q", 5120, 5120), ("k", 1024, 5120), ("v", 1024, 5120), ("o", 5120
 TAU = 1e-3
 # HBM bytes per launch of the tile kernel from hardware counters (FETCH_SIZE scaled by 2.0 against a plain 1 GiB pass,
 # plus WRITE_SIZE), as recorded in profiles/tile_kernel_9b_decode_step_hbm_traffic.md, by launch class
-MEASURED_TRAFFIC = {"q+k+v": (2 * 11013.2 + 33.2) * 1024, "fused-other": (2 * 24210.1 + 59.7) * 1024,      # default
+MEASURED_TRAFFIC = {"q+k+v": (2 * 10999.9 + 33.2) * 1024, "fused-other": (2 * 24196.5 + 59.7) * 1024,      # default
                     256: (2 * 16078.3 + 39.8) * 1024, 64: (2 * 2014.4 + 4.9) * 1024}                        # --no-fuse
 MMA_FLAGS = int(os.environ.get("QVB8_BENCH_MMA_FLAGS", "1"))     # 1 = QVB8_MMA_SATURATE_X: the operator's default for bf16 x
 
