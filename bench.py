@@ -520,7 +520,7 @@ def main():
                      "traffic": (None if MMA_FLAGS != 1 or args.model != "9b" else
                                  round(sum(MEASURED_TRAFFIC[256 if e["Q"] >= 4096 else 64] for e in flat) / n_launch) if args.no_fuse
                                  else round(sum(MEASURED_TRAFFIC["q+k+v" if u["name"] == "q+k+v" else "fused-other"] for u in units) / n_launch)),
-                     "kernel": "qvb8::tile_kernel<1,4,false,true,true>" + (" / <1,5,false,true,true> for 5120-column rows" if args.model == "27b" else ""),
+                     "kernel": "qvb8::tile_kernel<1,4,false,true,XP> (XP = 1 or 4 pieces of X per thread through LDS)" + (" / <1,5,false,true,XP> for 5120-column rows" if args.model == "27b" else ""),
                      "bytes_per_launch": step_bytes // n_launch,
                      "launch_us": round(launch_us, 3)},
     }

@@ -30,7 +30,6 @@ typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
 typedef float v16f_t __attribute__((ext_vector_type(16)));
 
 constexpr int kTileRows = 16;
-constexpr int kTileXPieces = 4;         // 16-byte pieces of X a thread may stage when X goes through LDS
 constexpr int kStepCols = 128;          // columns one wave step covers (4 lane groups x 32 ids)
 
 template <bool BF> struct Fmt;
@@ -187,11 +186,12 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
 // slots.  After one barrier the whole workgroup combines the column ranges of each row in a fixed order.
 // The kernel's arguments are 56 bytes of scalars (measured: every further 64 bytes of kernel arguments cost about a
 // microsecond per launch): fin follows loc, n_steps follows P, the small counts share one word.
-template <int NT, int T, bool BF, bool XC, bool XL = false>
+template <int NT, int T, bool BF, bool XC, int XP = 0>
 __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ ids,
                                                    const uint64_t* __restrict__ loc, float* __restrict__ Y, int64_t ids_bytes,
                                                    int Q, int P, uint32_t counts, int TW, int first1, int first2, uint32_t widths) {
     static_assert(!(BF && XC), "narrowing on the way in exists for fp16 operands only");
+    constexpr bool XL = XP > 0;                              // X goes through LDS, XP 16-byte pieces per thread
     TileArgs a;
     a.X = X; a.ids = ids; a.loc = loc; a.fin = reinterpret_cast<const uint4*>(loc + rowinfo_loc_words(Q)); a.Y = Y;
     a.ids_bytes = ids_bytes; a.Q = Q; a.P = P; a.n_steps = P / kStepCols; a.TW = TW;
@@ -217,16 +217,16 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = wave / a.W, wc = wave - g * a.W;
     const int r = lane & 15, kg = lane >> 4;
-    // XL: the whole of X (at most kTileXPieces 16-byte pieces per thread) goes through LDS once: every thread requests its
+    // XL: the whole of X (at most XP 16-byte pieces per thread) goes through LDS once: every thread requests its
     // pieces before anything else, the first tile's ids follow at once, and the workgroup shares X after one barrier --
     // so the trip of the activations and the first trip of the ids overlap, and later panels need no trip for theirs.
     unsigned char* xs = reinterpret_cast<unsigned char*>(part + (size_t)rows_cap * ranges * MS);     // [M][P] in operand format
     const int x_pieces = (a.M * a.P) >> 3;
-    v4u_t xg[kTileXPieces];
+    v4u_t xg[XL ? XP : 1];
     if constexpr (XL) {
         const v4u_t* xsrc = reinterpret_cast<const v4u_t*>(a.X);
 #pragma unroll
-        for (int i = 0; i < kTileXPieces; ++i) xg[i] = xsrc[min(tid + i * (int)blockDim.x, x_pieces - 1)];
+        for (int i = 0; i < XP; ++i) xg[i] = xsrc[min(tid + i * (int)blockDim.x, x_pieces - 1)];
         __builtin_amdgcn_sched_barrier(0);                     // these requests stay where they are: ahead of everything
     }
     // The workgroup's local tile lt is global tile lt * gridDim.x + blockIdx.x: at any moment the workgroups of the
@@ -309,7 +309,7 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
     if constexpr (XL) {
         info = issue_tile(0, wc * T, wlo, whi, n_tiles > 0);   // steps past the row's end read the buffer's start as well
 #pragma unroll
-        for (int i = 0; i < kTileXPieces; ++i) {
+        for (int i = 0; i < XP; ++i) {
             const int idx = tid + i * (int)blockDim.x;
             v4u_t v = xg[i];
             if constexpr (XC) {
@@ -757,7 +757,8 @@ namespace {
 struct TilePlan { int W, G, panels, TW, threads; size_t lds; unsigned blocks; };
 
 constexpr size_t kTileLdsLimit = 128 * 1024;
-constexpr size_t kTileXLdsLimit = 32 * 1024;     // X through LDS: up to this many bytes of activations on top
+constexpr size_t kTileXLdsLimit = 64 * 1024;     // X through LDS: up to this many bytes of activations on top
+constexpr size_t kLdsPerWorkgroup = 160 * 1024;
 
 bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl) {
     const int n_steps = (int)(P / kStepCols);
@@ -799,31 +800,43 @@ bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl) {
     return true;
 }
 
-template <int NT, int T, bool BF, bool XC, bool XL = false>
+template <int NT, int T, bool BF, bool XC, int XP = 0>
 int launch_tile(TileArgs& a, hipStream_t s) {
     TilePlan pl;
     if (!plan_tile(NT, T, a.M, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
-    if constexpr (XL) {
-        const size_t x_bytes = (size_t)a.M * (size_t)a.P * 2;
-        if (x_bytes > kTileXLdsLimit || x_bytes / 16 > (size_t)kTileXPieces * pl.threads) return launch_tile<NT, T, BF, XC, false>(a, s);
-        pl.lds += x_bytes;
-    }
+    if constexpr (XP > 0) pl.lds += (size_t)a.M * (size_t)a.P * 2;
     a.W = pl.W; a.G = pl.G; a.panels = pl.panels; a.TW = pl.TW;
     static bool attr[64] = {false};                           // per device: the attribute belongs to the device's copy of the kernel
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: no current device");
     if (!attr[dev]) {
-        if (hipFuncSetAttribute((const void*)tile_kernel<NT, T, BF, XC, XL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kTileLdsLimit + kTileXLdsLimit)) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)tile_kernel<NT, T, BF, XC, XP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup) != hipSuccess)
             return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: cannot raise the kernel's LDS limit");
         attr[dev] = true;
     }
     if (pl.panels > 0xffff) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: rows too long");
     const uint32_t counts = (uint32_t)a.M | ((uint32_t)a.W << 8) | ((uint32_t)a.G << 12) | ((uint32_t)a.panels << 16);
-    hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC, XL>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s,
+    hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC, XP>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s,
                        a.X, a.ids, a.loc, a.Y, a.ids_bytes, a.Q, a.P, counts, a.TW, a.first1, a.first2,
                        (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16) | ((uint32_t)a.n_classes << 24));
     return host::check_launch("qvb8_mma");
 }
+// One to sixteen rows of X on the NT = 1 kernel: X goes through LDS when all of it fits (64 KB, and the workgroup's LDS),
+// with 1, 4 or 8 pieces of 16 bytes per thread (a request past the end of X would be a wasted one: the count is exact to
+// within those three variants).
+template <int T, bool BF, bool XC>
+int launch_tile_rows16(TileArgs& a, hipStream_t s) {
+    TilePlan pl;
+    if (!plan_tile(1, T, a.M, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
+    const size_t x_bytes = (size_t)a.M * (size_t)a.P * 2;
+    const size_t per_thread = (x_bytes / 16 + pl.threads - 1) / pl.threads;
+    const bool fits = x_bytes <= kTileXLdsLimit && pl.lds + x_bytes <= kLdsPerWorkgroup && host::env_int("QVB8_TILE_X_LDS", 1) != 0;
+    if (fits && per_thread <= 1) return launch_tile<1, T, BF, XC, 1>(a, s);
+    if (fits && per_thread <= 4) return launch_tile<1, T, BF, XC, 4>(a, s);
+    if (fits && per_thread <= 8) return launch_tile<1, T, BF, XC, 8>(a, s);
+    return launch_tile<1, T, BF, XC, 0>(a, s);
+}
+
 struct GemmPlan {
     int MT, tok_blocks, row_blocks, splits, stages_per_split;
     size_t lds;
@@ -996,12 +1009,9 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     // rows of 33..40 steps (P = 5120): one panel of eight waves with five steps each instead of two panels of five waves
     // with four (measured on 27B-class shapes: 16 % faster; more steps per wave did not pay for longer rows)
     const int n_steps_all = (int)(P / kStepCols);
-#define QVB8_TILE_LAUNCH_XL(T_) (mode == 0 ? launch_tile<1, T_, false, false, true>(a, s) : mode == 1 ? launch_tile<1, T_, false, true, true>(a, s) : launch_tile<1, T_, true, false, true>(a, s))
-    const bool x_lds = M <= 16 && M * P * 2 <= (int64_t)kTileXLdsLimit && host::env_int("QVB8_TILE_X_LDS", 1) != 0;
-    if (x_lds) rc = n_steps_all > 32 && n_steps_all <= 40 ? QVB8_TILE_LAUNCH_XL(5) : QVB8_TILE_LAUNCH_XL(4);
-    else if (M <= 16 && n_steps_all > 32 && n_steps_all <= 40) rc = QVB8_TILE_LAUNCH(1, 5);
-#undef QVB8_TILE_LAUNCH_XL
-    else if (M <= 16) rc = QVB8_TILE_LAUNCH(1, 4);
+#define QVB8_TILE_LAUNCH_ROWS16(T_) (mode == 0 ? launch_tile_rows16<T_, false, false>(a, s) : mode == 1 ? launch_tile_rows16<T_, false, true>(a, s) : launch_tile_rows16<T_, true, false>(a, s))
+    if (M <= 16) rc = n_steps_all > 32 && n_steps_all <= 40 ? QVB8_TILE_LAUNCH_ROWS16(5) : QVB8_TILE_LAUNCH_ROWS16(4);
+#undef QVB8_TILE_LAUNCH_ROWS16
     else if (M <= 32) rc = QVB8_TILE_LAUNCH(2, 2);
     else rc = QVB8_TILE_LAUNCH(3, 2);
 #undef QVB8_TILE_LAUNCH
