@@ -47,6 +47,23 @@ def test_mma_all_m(M, dtype):
         _check(H.oracle_view(enc), None, x, y, saturate_ref=False)
 
 
+@pytest.mark.parametrize("M,P", [(1, 4096), (3, 4096), (8, 4096), (1, 12288), (1, 17408), (2, 5120), (1, 28672)])
+def test_activations_through_lds_change_no_bit(M, P, monkeypatch):
+    """Small X is staged through LDS once (1, 4 or 8 sixteen-byte pieces per thread); the same call with that path
+    switched off reads X from global memory per panel.  Same arithmetic in the same order: identical bits."""
+    W = H.synth_weight(80, P, seed=P + M).to(DEV)
+    enc = PK.encode_tensor(W, 1e-3, restore="fp16", force_escapes=[9, P * 79 + P - 1])
+    perm = _perm_by_width(enc["nbits"])
+    for dtype, saturate in ((torch.bfloat16, True), (torch.float16, False), (torch.bfloat16, False)):
+        x = _x(M, P, dtype, 7 * M)
+        monkeypatch.setenv("QVB8_TILE_X_LDS", "1")
+        y1 = ext.mma_tiles(x, *H.pack_args(enc), perm=perm, saturate=saturate)
+        monkeypatch.setenv("QVB8_TILE_X_LDS", "0")
+        y0 = ext.mma_tiles(x, *H.pack_args(enc), perm=perm, saturate=saturate)
+        assert torch.equal(y1, y0), (dtype, saturate)
+    _check(H.oracle_view(enc), None, x, y1, saturate_ref=False)
+
+
 @pytest.mark.parametrize("Q,P,tau", [(1024, 4096, 1e-3), (200, 12288, 1e-3), (130, 768, 2e-3), (96, 2048, 2e-3),
                                      (64, 5120, 2e-3), (40, 17408, 2e-3), (24, 28672, 2e-3), (16, 128, 1e-3), (3, 256, 1e-3)])
 def test_mma_shapes(Q, P, tau):
