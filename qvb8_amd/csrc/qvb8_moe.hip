@@ -20,6 +20,7 @@
 #include "../../include/qvb8_amd.h"
 #include "qvb8_device.h"
 #include "qvb8_host.h"
+#include "qvb8_mma_device.h"
 
 namespace qvb8 {
 
@@ -305,6 +306,213 @@ __global__ void __launch_bounds__(kMoeThreads) moe_gemv_kernel(MoeGemvArgs a) {
     }
 }
 
+// ---- one token: both projections on the matrix cores ------------------------------------------------------------------
+// With a single token every selected expert has exactly one pair, and nothing needs a routing plan: slot j is expert
+// idx[j].  Two launches instead of four.  Both use the tile scheme of the dense kernels: a row tile is 16 rows of one
+// expert, a wave owns T steps of 128 columns of it (W = ceil(steps / T) waves per tile, G = 8 / W tiles at a time),
+// requests its activations and its ids in one burst (no request under a branch), decodes the ids into MFMA operands
+// (ids exact in fp16 next to a bias of 1024, the token in row 0 of the other operand) and leaves its partial sums in LDS.
+//   up:   a workgroup takes `tiles_per_wg` unit tiles (16 outputs of one slot; gated: the 16 gate rows and the 16
+//         matching up rows, so the activation is applied here) and writes H as fp16, saturated like every activation.
+//   down: workgroup b takes rows 16 b .. 16 b + 15 of EVERY slot (the token's H row of that slot as activations) and
+//         adds the slots up in order with their routing weights: the combine needs no launch and no buffer.
+// Rows the slicing cannot read (width outside 4..8, not dword aligned) are redone element by element; an expert number
+// outside the stack gives NaN.
+constexpr int kOneMaxTiles = 16;       // row tiles per workgroup
+constexpr int kOneWaves = 8;
+
+struct MoeOneArgs {
+    const uint16_t* X;             // up: the token's activations (P), fp16 or bf16 bits; down: H (topk, P) fp16 bits
+    const int64_t* idx;            // (topk) selected experts
+    const float* w;                // (topk) routing weights (down)
+    const uint8_t* ids; int64_t ids_bytes;
+    const float* min_s; const float* tau_s; const uint8_t* nbits; const int64_t* bit_off;   // (E, Q)
+    void* out;                     // up: H (topk, units) fp16 bits; down: out (Q) in the caller's dtype
+    int E, Q, P, topk;
+    int units, gated;              // up: outputs per expert; whether the rows come as (gate, up) halves
+    int tiles_per_wg;              // up: unit tiles per workgroup
+};
+
+template <int T, bool DOWN, bool XC, int DT>
+__global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
+    using F = Fmt<false>;
+    using XI = XIn<false, XC>;
+    __shared__ float s_part[kOneMaxTiles][kOneWaves][16];    // [row tile][column range][row]
+    __shared__ float s_sx[kOneMaxTiles][kOneWaves];          // sum of the activations over the column range
+    __shared__ float2 s_fin[kOneMaxTiles][16];               // tau_s, min_s of the tile's rows
+    __shared__ int s_ok[kOneMaxTiles];                       // the slot's expert number is inside the stack
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, kg = lane >> 4;
+    const int n_steps = a.P / kStepCols;
+    const int W = (n_steps + T - 1) / T, G = kOneWaves / W;
+    const int g = wave / W, wc = wave - g * W;
+    const int step0 = wc * T;
+    const int RT = (!DOWN && a.gated) ? 2 : 1;               // row tiles per unit tile
+    const int UT = DOWN ? 1 : a.units / 16;                  // unit tiles per expert
+    const int ut_first = DOWN ? 0 : (int)blockIdx.x * a.tiles_per_wg;
+    const int n_rt = DOWN ? a.topk : min(a.tiles_per_wg, a.topk * UT - ut_first) * RT;
+    auto slot_of = [&](int i) { return DOWN ? i : (ut_first + i / RT) / UT; };
+    auto row0_of = [&](int i) { return DOWN ? (int)blockIdx.x * 16 : ((ut_first + i / RT) % UT) * 16 + (i % RT) * a.units; };
+    const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
+    const v4u_t ones = {F::one_bits, F::one_bits, F::one_bits, F::one_bits};
+
+    // A round = the row tiles the workgroup's waves work on at the same time.  (Two rounds of the up kernel in flight
+    // together were measured: no faster -- a CU's share of the bytes, not the chain of trips, sets the time -- and the
+    // registers cost occupancy.)  The up kernel loads its activations once, the down kernel per round: every slot has
+    // activations of its own.
+    constexpr int R = 1;
+    struct Round { int i; bool has; int nb; int64_t bit0; float ts, mn; bool e_ok, ok, sliced; };
+    Round rd[R];
+    uint4 wlo[R][T], whi[R][T];
+    v4u_t xa[T][4];
+    auto request_x = [&](const uint16_t* xrow) {
+#pragma unroll
+        for (int it = 0; it < T; ++it) {
+            const bool on = (step0 + it) < n_steps;
+            const uint16_t* xp = xrow + (on ? (size_t)(step0 + it) * kStepCols + kg * 32 : (size_t)0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xa[it][j] = *reinterpret_cast<const v4u_t*>(xp + 8 * j);
+        }
+    };
+    // the token sits in row 0 of its operand; narrowed like every activation when it arrives as bf16
+    auto finish_x = [&]() {
+#pragma unroll
+        for (int it = 0; it < T; ++it) {
+            const bool on = (step0 + it) < n_steps && r == 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) xa[it][j][k] = on ? XI::pair(xa[it][j][k]) : 0u;
+        }
+    };
+    // nothing here is under a branch: a wave without a tile in this round reads the metadata of tile 0 and the start of ids
+    auto request_meta = [&](Round& q, int i) {
+        q.has = g < G && i < n_rt;
+        q.i = q.has ? i : 0;
+        const int64_t e = a.idx[slot_of(q.i)];
+        q.e_ok = e >= 0 && e < a.E;
+        const size_t mi = (size_t)(q.e_ok ? e : 0) * a.Q + row0_of(q.i) + r;
+        q.nb = a.nbits[mi];
+        q.bit0 = a.bit_off[mi];
+        q.ts = a.tau_s[mi]; q.mn = a.min_s[mi];
+    };
+    auto request_ids = [&](Round& q, uint4 (&lo)[T], uint4 (&hi)[T]) {
+        q.ok = q.e_ok && q.nb >= 1 && q.nb <= 14 && q.bit0 >= 0 && ((q.bit0 + (int64_t)q.nb * a.P + 7) >> 3) + 8 <= a.ids_bytes;
+        q.sliced = q.ok && q.nb >= 4 && q.nb <= 8 && (q.bit0 & 31) == 0;
+        const uint64_t row_off = (uint64_t)(q.bit0 >> 3) + (uint64_t)(step0 * 4 + kg) * (4u * (uint32_t)q.nb);
+#pragma unroll
+        for (int it = 0; it < T; ++it) {
+            const bool use = q.sliced && (step0 + it) < n_steps;       // a wave without a tile reads tile 0's again: no address shared by the whole chip
+            const uint64_t off = use ? row_off + (uint64_t)it * (16u * (uint32_t)q.nb) : 0;
+            lo[it] = *reinterpret_cast<const uint4*>(a.ids + off);
+            hi[it] = *reinterpret_cast<const uint4*>(a.ids + off + (use ? 4u * (uint32_t)(q.nb - 4) : 16u));
+        }
+    };
+    auto multiply = [&](const Round& q, const uint4 (&lo_)[T], const uint4 (&hi_)[T], const uint16_t* xrow) {
+        const int nb = q.nb;
+        const bool sliced = q.sliced;
+        v4f_t sx = {0.f, 0.f, 0.f, 0.f}, acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int it = 0; it < T; ++it)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sx = F::mfma(xa[it][j], ones, sx);
+        const uint32_t info = sliced ? ((uint32_t)nb | 256u) : 0u;
+        const uint32_t info0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
+        const bool uniform = __builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u;
+#pragma unroll
+        for (int it = 0; it < T; ++it) {
+            v4u_t b[4];
+            const uint4 lo = lo_[it], hi = hi_[it];
+            if (uniform) {
+                switch (info0 & 0xFFu) {
+                    case 7: decode_slice<7, false>(lo, hi, b); break;
+                    case 6: decode_slice<6, false>(lo, hi, b); break;
+                    case 5: decode_slice<5, false>(lo, hi, b); break;
+                    case 4: decode_slice<4, false>(lo, hi, b); break;
+                    default: decode_slice<8, false>(lo, hi, b); break;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) b[j] = v4u_t{F::bias_bits, F::bias_bits, F::bias_bits, F::bias_bits};
+                if (__builtin_amdgcn_ballot_w64(sliced && nb == 7)) { if (sliced && nb == 7) decode_slice<7, false>(lo, hi, b); }
+                if (__builtin_amdgcn_ballot_w64(sliced && nb == 6)) { if (sliced && nb == 6) decode_slice<6, false>(lo, hi, b); }
+                if (__builtin_amdgcn_ballot_w64(sliced && nb == 5)) { if (sliced && nb == 5) decode_slice<5, false>(lo, hi, b); }
+                if (__builtin_amdgcn_ballot_w64(sliced && nb == 4)) { if (sliced && nb == 4) decode_slice<4, false>(lo, hi, b); }
+                if (__builtin_amdgcn_ballot_w64(sliced && nb == 8)) { if (sliced && nb == 8) decode_slice<8, false>(lo, hi, b); }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc = F::mfma(xa[it][j], b[j], acc);
+        }
+        if (!q.has) return;                                   // wave-uniform
+        const int i = q.i;
+        // the token's sums (accumulator register 0 of lane group 0) into the wave's LDS slots
+        if (kg == 0) s_part[i][wc][r] = __builtin_fmaf(-F::bias, sx[0], acc[0]);
+        if (lane == 0) s_sx[i][wc] = sx[0];
+        if (kg == 0 && wc == 0) s_fin[i][r] = float2{q.ts, q.mn};
+        if (lane == 0 && wc == 0) s_ok[i] = q.e_ok ? 1 : 0;
+        // rows the slicing cannot read: element by element over this wave's columns
+        uint64_t odd = __builtin_amdgcn_ballot_w64(kg == 0 && !sliced);
+        while (odd) {
+            const int rr = __builtin_ctzll(odd);
+            odd &= odd - 1;
+            const int nb2 = __shfl(nb, rr, 64);
+            const int64_t bit02 = ((int64_t)__shfl((int)(q.bit0 >> 32), rr, 64) << 32) | (uint32_t)__shfl((int)(uint32_t)q.bit0, rr, 64);
+            const bool ok2 = __shfl((int)q.ok, rr, 64) != 0;
+            const int c_lo = step0 * kStepCols, c_hi = min(a.P, (step0 + T) * kStepCols);
+            float sacc = 0.f;
+            if (ok2) {
+                for (int c = c_lo + lane; c < c_hi; c += kWave)
+                    sacc = __builtin_fmaf(XI::scalar(xrow[c]), (float)load_field(a.ids, bit02 + (int64_t)c * nb2, nb2, clamp_byte), sacc);
+            } else {
+                sacc = __builtin_nanf("");
+            }
+            const float tot = wave_sum(sacc);
+            if (lane == 0) s_part[i][wc][rr] += tot;
+        }
+    };
+
+    const int n_rounds = (n_rt + G - 1) / G;
+    if constexpr (!DOWN) { request_x(a.X); }
+    for (int r0 = 0; r0 < n_rounds; r0 += R) {
+        if constexpr (DOWN) request_x(a.X + (size_t)slot_of(min(g + r0 * G, n_rt - 1) * (g < G ? 1 : 0)) * a.P);
+#pragma unroll
+        for (int k = 0; k < R; ++k) request_meta(rd[k], g + (r0 + k) * G);
+#pragma unroll
+        for (int k = 0; k < R; ++k) request_ids(rd[k], wlo[k], whi[k]);
+        if (DOWN || r0 == 0) finish_x();
+#pragma unroll
+        for (int k = 0; k < R; ++k) multiply(rd[k], wlo[k], whi[k], a.X + (DOWN ? (size_t)slot_of(rd[k].i) * a.P : (size_t)0));
+    }
+    __syncthreads();
+
+    auto row_value = [&](int i, int u) {                      // tau_s * sum(x * id) + min_s * sum(x), the ranges added in order
+        double d = 0.0, xs = 0.0;
+        for (int w = 0; w < W; ++w) { d += (double)s_part[i][w][u]; xs += (double)s_sx[i][w]; }
+        const float2 f = s_fin[i][u];
+        const float y = (float)((double)f.x * d + (double)f.y * xs);
+        return s_ok[i] ? y : __builtin_nanf("");
+    };
+    if constexpr (DOWN) {
+        if (tid < 16) {
+            float acc = 0.f;
+            for (int j = 0; j < a.topk; ++j) acc = __builtin_fmaf(a.w[j], row_value(j, tid), acc);
+            store_from_f32<DT>(a.out, (int64_t)blockIdx.x * 16 + tid, acc);
+        }
+    } else {
+        const int n_ut = n_rt / RT;
+        for (int o = tid; o < n_ut * 16; o += blockDim.x) {
+            const int lut = o >> 4, u = o & 15, i0 = lut * RT;
+            const float y0 = row_value(i0, u);
+            float h;
+            if (a.gated) h = (y0 / (1.0f + __expf(-y0))) * row_value(i0 + 1, u);
+            else { const float p = fmaxf(y0, 0.f); h = y0 != y0 ? y0 : p * p; }
+            const int ut = ut_first + lut;
+            reinterpret_cast<uint16_t*>(a.out)[(size_t)(ut / UT) * a.units + (ut % UT) * 16 + u] = (uint16_t)sat_half_bits(h);
+        }
+    }
+}
+
 template <int DT>
 __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restrict__ Yd, const float* __restrict__ w, void* __restrict__ out,
                                                           int topk, int D, int tokens, const int32_t* __restrict__ n_bad) {
@@ -351,6 +559,29 @@ int launch_moe_gemv(int stage, MoeGemvArgs a, int64_t slots, hipStream_t s) {
     else hipLaunchKernelGGL(moe_gemv_kernel<1>, grid, dim3(kMoeThreads), lds, s, a);
     return host::check_launch("qvb8_moe_experts");
 }
+// The one-token path: what it needs, and its two launches.  H (fp16) takes the place of the fp32 H in the workspace.
+bool moe_one_token_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t Q_up, int64_t P_up, int64_t Q_dn, int64_t P_dn, int act) {
+    if (tokens != 1 || topk > 8 || (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16)) return false;
+    if (P_up % kStepCols != 0 || P_dn % kStepCols != 0 || P_up > 4096 || P_dn > 4096) return false;
+    if (P_dn % 16 != 0 || Q_dn % 16 != 0) return false;
+    (void)Q_up; (void)act;
+    return host::env_int("QVB8_MOE_ONE_TOKEN", 1) != 0;
+}
+
+template <bool DOWN, bool XC, int DT>
+int launch_moe_one(const MoeOneArgs& a, unsigned blocks, hipStream_t s) {
+    const int n_steps = a.P / kStepCols;
+    // six steps per wave only for the down kernel (one round in flight): a whole row of up to 768 columns per wave, so
+    // that eight slots are one round
+    if constexpr (DOWN) {
+        if (n_steps <= 6) {
+            hipLaunchKernelGGL((moe_one_kernel<6, DOWN, XC, DT>), dim3(blocks), dim3(64 * kOneWaves), 0, s, a);
+            return host::check_launch("qvb8_moe_experts");
+        }
+    }
+    hipLaunchKernelGGL((moe_one_kernel<4, DOWN, XC, DT>), dim3(blocks), dim3(64 * kOneWaves), 0, s, a);
+    return host::check_launch("qvb8_moe_experts");
+}
 }  // namespace
 
 extern "C" int64_t qvb8_moe_workspace_bytes(int64_t tokens, int64_t topk, int64_t n_experts, int64_t Q_up, int64_t P_dn, int64_t Q_dn) {
@@ -390,6 +621,29 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
     float* H = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np));
     float* Yd = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np) + align256((size_t)np * P_dn * 4));
 
+    if (moe_one_token_ok(tokens, topk, x_dtype, Q_up, P_up, Q_dn, P_dn, act)) {
+        MoeOneArgs o;
+        o.X = reinterpret_cast<const uint16_t*>(X); o.idx = idx; o.w = w; o.ids = up_ids; o.ids_bytes = up_ids_bytes;
+        o.min_s = up_min; o.tau_s = up_tau; o.nbits = up_nb; o.bit_off = up_off; o.out = H;
+        o.E = (int)n_experts; o.Q = (int)Q_up; o.P = (int)P_up; o.topk = (int)topk; o.units = (int)P_dn; o.gated = act == 0 ? 1 : 0;
+        // unit tiles per workgroup: about one workgroup per CU, within what the rounds of a workgroup can take
+        const int RT = o.gated ? 2 : 1;
+        const int64_t total_ut = topk * (P_dn / 16);
+        int64_t per_wg = (total_ut + host::device_cus() - 1) / host::device_cus();
+        const int64_t cap = kOneMaxTiles / RT;
+        if (per_wg > cap) per_wg = cap;
+        if (per_wg < 1) per_wg = 1;
+        o.tiles_per_wg = (int)per_wg;
+        const unsigned up_blocks = (unsigned)((total_ut + per_wg - 1) / per_wg);
+        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_one<false, true, 0>(o, up_blocks, s) : launch_moe_one<false, false, 0>(o, up_blocks, s)) return rc;
+        o.X = reinterpret_cast<const uint16_t*>(H); o.ids = dn_ids; o.ids_bytes = dn_ids_bytes;
+        o.min_s = dn_min; o.tau_s = dn_tau; o.nbits = dn_nb; o.bit_off = dn_off; o.out = out;
+        o.Q = (int)Q_dn; o.P = (int)P_dn; o.units = (int)Q_dn; o.gated = 0; o.tiles_per_wg = 0;
+        const unsigned dn_blocks = (unsigned)(Q_dn / 16);
+        if (out_dtype == QVB8_F32) return launch_moe_one<true, false, 0>(o, dn_blocks, s);
+        if (out_dtype == QVB8_F16) return launch_moe_one<true, false, 1>(o, dn_blocks, s);
+        return launch_moe_one<true, false, 2>(o, dn_blocks, s);
+    }
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)(n_experts + 8) * 4, s, idx, (int)np, (int)n_experts, pl);
     if (int rc = host::check_launch("qvb8_moe_experts plan")) return rc;
     const int64_t slots = moe_slots(n_experts, np);

@@ -110,6 +110,59 @@ def test_moe_relu2_and_odd_widths():
     _check(out, O.moe_reference(x.float().numpy(), idx, w, Wup, Wdn, act="relu2"), torch.float16)
 
 
+def _hand_made_stack(E, Q, P, widths, seed):
+    """E hand-made experts of (Q, P) with the given row widths, stacked as QVBandExpertsV8.build_stack lays them out;
+    returns the operands after X / idx / w of ext.moe_experts and the restored weights."""
+    lst, Ws = [], []
+    for e in range(E):
+        d = H.mixed_width_pack(Q, P, widths, seed=seed + e)
+        d["tau_s"] = d["tau_s"] * (1.0 / (1 << 6))
+        a = H.to_device_args(d, DEV)
+        lst.append(dict(ids=a[0], min_s=a[1], nbits=a[2], bit_off=a[3], tau_s=a[5]))
+        Ws.append(O.reconstruct(d["min_s"], d["tau_s"], d["ids_dense"], d["esc_idx"], d["esc_vals"]))
+    offs, total = [], 0
+    for t in lst:
+        offs.append(total)
+        total += (t["ids"].numel() + 15) // 16 * 16
+    ids = torch.zeros(total + 64, dtype=torch.uint8, device=DEV)
+    for o, t in zip(offs, lst):
+        ids[o:o + t["ids"].numel()] = t["ids"]
+    ops = (ids, torch.stack([t["min_s"] for t in lst]), torch.stack([t["tau_s"] for t in lst]),
+           torch.stack([t["nbits"] for t in lst]), torch.stack([t["bit_off"] + 8 * o for t, o in zip(lst, offs)]))
+    return ops, Ws
+
+
+@pytest.mark.parametrize("gated", [True, False])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_moe_one_token_on_the_matrix_cores(gated, dtype, monkeypatch):
+    """One token takes two launches (up with the activation, down with the weighted sum) on MFMA tiles.  Rows of every
+    width 1..14 in the up stack (sliced tiles, mixed tiles and element-by-element rows), 4..8 in the down stack; against
+    the oracle, against the general path, run to run, and with an expert number outside the stack."""
+    E, hidden, inter, k = 5, 256, 128, 3
+    Qup = 2 * inter if gated else inter
+    up_ops, Wup = _hand_made_stack(E, Qup, hidden, [6, 6, 6, 6, 6, 6, 6, 6, 6, 6, 6, 6, 6, 6, 6, 6, 7, 5] + list(range(1, 15)), seed=40)
+    dn_ops, Wdn = _hand_made_stack(E, hidden, inter, [4, 5, 6, 7, 8], seed=80)
+    idx, w = _route(1, E, k, seed=11)
+    x = torch.randn(1, hidden, generator=torch.Generator().manual_seed(2)).to(dtype)
+    fn = ext.moe_experts if gated else ext.moe_experts_relu2
+    args = (x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV), *up_ops, Qup, hidden, *dn_ops, hidden, inter)
+    monkeypatch.setenv("QVB8_MOE_ONE_TOKEN", "1")
+    out = fn(*args)
+    assert out.dtype == dtype and out.shape == (1, hidden)
+    ref = O.moe_reference(x.float().numpy(), idx, w, Wup, Wdn, act="silu" if gated else "relu2")
+    _check(out, ref, dtype)
+    assert torch.equal(out, fn(*args))
+    monkeypatch.setenv("QVB8_MOE_ONE_TOKEN", "0")
+    general = fn(*args)
+    _check(general, ref, dtype)
+    scale = float(np.sqrt(np.mean(ref ** 2)))
+    assert float((out.float() - general.float()).abs().max()) <= 4e-3 * scale + 2.0 ** -7 * float(np.abs(ref).max())
+    monkeypatch.setenv("QVB8_MOE_ONE_TOKEN", "1")
+    bad = torch.from_numpy(idx).to(DEV).clone()
+    bad[0, 1] = E + 3
+    assert torch.isnan(fn(args[0], bad, *args[2:]).float()).all()
+
+
 def test_moe_refusals():
     E, hidden, inter = 2, 128, 32
     gu, dn, _, _ = _experts(E, hidden, inter, 2e-3, seed=900)
