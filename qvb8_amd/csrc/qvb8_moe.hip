@@ -344,6 +344,11 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, kg = lane >> 4;
+    // blockIdx.y = token: every token is a problem of its own (its slots, its activations, its output row)
+    const int tok = blockIdx.y;
+    a.idx += (size_t)tok * a.topk; a.w += (size_t)tok * a.topk;
+    if constexpr (DOWN) { a.X += (size_t)tok * a.topk * a.P; a.out = reinterpret_cast<unsigned char*>(a.out) + (size_t)tok * a.Q * (DT == 0 ? 4 : 2); }
+    else { a.X += (size_t)tok * a.P; a.out = reinterpret_cast<uint16_t*>(a.out) + (size_t)tok * a.topk * a.units; }
     const int n_steps = a.P / kStepCols;
     const int W = (n_steps + T - 1) / T, G = kOneWaves / W;
     const int g = wave / W, wc = wave - g * W;
@@ -561,7 +566,7 @@ int launch_moe_gemv(int stage, MoeGemvArgs a, int64_t slots, hipStream_t s) {
 }
 // The one-token path: what it needs, and its two launches.  H (fp16) takes the place of the fp32 H in the workspace.
 bool moe_one_token_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t Q_up, int64_t P_up, int64_t Q_dn, int64_t P_dn, int act) {
-    if (tokens != 1 || topk > 8 || (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16)) return false;
+    if (tokens > host::env_int("QVB8_MOE_TILE_TOKENS", 16) || topk > 8 || (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16)) return false;
     if (P_up % kStepCols != 0 || P_dn % kStepCols != 0 || P_up > 4096 || P_dn > 4096) return false;
     if (P_dn % 16 != 0 || Q_dn % 16 != 0) return false;
     (void)Q_up; (void)act;
@@ -569,17 +574,17 @@ bool moe_one_token_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t Q_up, i
 }
 
 template <bool DOWN, bool XC, int DT>
-int launch_moe_one(const MoeOneArgs& a, unsigned blocks, hipStream_t s) {
+int launch_moe_one(const MoeOneArgs& a, unsigned blocks, unsigned tokens, hipStream_t s) {
     const int n_steps = a.P / kStepCols;
     // six steps per wave only for the down kernel (one round in flight): a whole row of up to 768 columns per wave, so
     // that eight slots are one round
     if constexpr (DOWN) {
         if (n_steps <= 6) {
-            hipLaunchKernelGGL((moe_one_kernel<6, DOWN, XC, DT>), dim3(blocks), dim3(64 * kOneWaves), 0, s, a);
+            hipLaunchKernelGGL((moe_one_kernel<6, DOWN, XC, DT>), dim3(blocks, tokens), dim3(64 * kOneWaves), 0, s, a);
             return host::check_launch("qvb8_moe_experts");
         }
     }
-    hipLaunchKernelGGL((moe_one_kernel<4, DOWN, XC, DT>), dim3(blocks), dim3(64 * kOneWaves), 0, s, a);
+    hipLaunchKernelGGL((moe_one_kernel<4, DOWN, XC, DT>), dim3(blocks, tokens), dim3(64 * kOneWaves), 0, s, a);
     return host::check_launch("qvb8_moe_experts");
 }
 }  // namespace
@@ -635,14 +640,15 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
         if (per_wg < 1) per_wg = 1;
         o.tiles_per_wg = (int)per_wg;
         const unsigned up_blocks = (unsigned)((total_ut + per_wg - 1) / per_wg);
-        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_one<false, true, 0>(o, up_blocks, s) : launch_moe_one<false, false, 0>(o, up_blocks, s)) return rc;
+        const unsigned tk = (unsigned)tokens;
+        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_one<false, true, 0>(o, up_blocks, tk, s) : launch_moe_one<false, false, 0>(o, up_blocks, tk, s)) return rc;
         o.X = reinterpret_cast<const uint16_t*>(H); o.ids = dn_ids; o.ids_bytes = dn_ids_bytes;
         o.min_s = dn_min; o.tau_s = dn_tau; o.nbits = dn_nb; o.bit_off = dn_off; o.out = out;
         o.Q = (int)Q_dn; o.P = (int)P_dn; o.units = (int)Q_dn; o.gated = 0; o.tiles_per_wg = 0;
         const unsigned dn_blocks = (unsigned)(Q_dn / 16);
-        if (out_dtype == QVB8_F32) return launch_moe_one<true, false, 0>(o, dn_blocks, s);
-        if (out_dtype == QVB8_F16) return launch_moe_one<true, false, 1>(o, dn_blocks, s);
-        return launch_moe_one<true, false, 2>(o, dn_blocks, s);
+        if (out_dtype == QVB8_F32) return launch_moe_one<true, false, 0>(o, dn_blocks, tk, s);
+        if (out_dtype == QVB8_F16) return launch_moe_one<true, false, 1>(o, dn_blocks, tk, s);
+        return launch_moe_one<true, false, 2>(o, dn_blocks, tk, s);
     }
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)(n_experts + 8) * 4, s, idx, (int)np, (int)n_experts, pl);
     if (int rc = host::check_launch("qvb8_moe_experts plan")) return rc;
