@@ -219,7 +219,7 @@ def bench_moe(args, dev):
                        "bytes_per_step": step_bytes, "us_per_layer": round(per_layer_us, 2)},
             "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                         "kernel": ("qvb8::moe_one_kernel<4,false,..> + moe_one_kernel<6,true,..> (one layer = 2 launches)" if T == 1 else
+                         "kernel": ("qvb8::moe_one_kernel<4,false,..> + moe_one_kernel<6,true,..> (one layer = 2 launches)" if T <= 16 else
                                     "qvb8::moe_plan_kernel + moe_gemv_kernel<0> + moe_gemv_kernel<1> + moe_combine_kernel "
                                     "(one layer = 4 launches)"),
                          "bytes_per_launch": step_bytes // args.layers, "launch_us": round(per_layer_us, 3)},

@@ -175,8 +175,8 @@ int64_t qvb8_moe_workspace_bytes(int64_t tokens, int64_t topk, int64_t n_experts
  * bit offsets made global; experts carry no escapes.  idx i64 (tokens, topk), w f32 (tokens, topk), X (tokens, P_up)
  * in x_dtype; P_up and P_dn multiples of 32; Q_dn == P_up.  An expert selected by several tokens is read once for up
  * to 8 of them.  An index outside 0..n_experts-1 turns the whole output into NaN.  Four launches, no host round trip.
- * One token (tokens == 1, topk <= 8, fp16 / bf16 X, P_up and P_dn multiples of 128 up to 4096, Q_dn a multiple of 16)
- * takes two launches on the matrix cores instead: the up projection applies the activation and hands H over as
+ * Up to 16 tokens (topk <= 8, fp16 / bf16 X, P_up and P_dn multiples of 128 up to 4096, Q_dn a multiple of 16)
+ * take two launches on the matrix cores instead, every token as a problem of its own: the up projection applies the activation and hands H over as
  * saturated fp16 (the general path keeps H in fp32), the down projection adds the slots up with their routing weights.
  * Replaces: ext.moe_experts  qvb8_moe_experts_forward qvb8_cuda.cu:937-992 (kernels qvb8_moe_gemv :860-907,
  * qvb8_moe_act :910-918, qvb8_moe_combine :924-935) with act QVB8_MOE_SILU_GATED, and ext.moe_experts_relu2
