@@ -1,0 +1,74 @@
+"""GPU: graph replay of blocks built on the compressed operators is bit-identical to eager execution, replay after
+replay, with the program's own eager work and synchronisations in between."""
+import pytest
+import torch
+import torch.nn as nn
+
+from qvb8_amd.formats.qvb8 import pack as PK
+from qvb8_amd.formats.qvb8.backends_experts import QVBandExpertsV8
+from qvb8_amd.formats.qvb8.fuse import fuse_same_input
+from qvb8_amd.formats.qvb8.graph import GraphedBlock, install_block_graphs
+from qvb8_amd.formats.qvb8.module import QVBandLinearV8
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _lin(Q, P, seed):
+    return QVBandLinearV8.from_encoded(PK.encode_tensor(H.synth_weight(Q, P, seed=seed).to(DEV), 1e-3, restore="fp16"))
+
+
+class _Mlp(nn.Module):
+    def __init__(self, h, inter):
+        super().__init__()
+        self.gate_proj, self.up_proj, self.down_proj = _lin(inter, h, 1), _lin(inter, h, 2), _lin(h, inter, 3)
+
+    def forward(self, x):
+        return self.down_proj(torch.nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class _Moe(nn.Module):
+    def __init__(self, h, inter, E, k):
+        super().__init__()
+        gu = [_lin(2 * inter, h, 10 + e) for e in range(E)]
+        dn = [_lin(h, inter, 40 + e) for e in range(E)]
+        self.experts = QVBandExpertsV8(gu, dn, num_experts=E)
+        self.router = nn.Linear(h, E, bias=False).to(DEV).to(torch.bfloat16)
+        self.k = k
+
+    def forward(self, x):
+        p = torch.softmax(self.router(x).float(), -1)
+        w, idx = torch.topk(p, self.k, -1)
+        return self.experts(x, idx, (w / w.sum(-1, keepdim=True)))
+
+
+class _Layer(nn.Module):
+    def __init__(self, block):
+        super().__init__()
+        self.mlp = block
+
+
+@pytest.mark.parametrize("kind", ["mlp", "moe"])
+@torch.no_grad()
+def test_graph_replay_is_bit_identical(kind):
+    torch.manual_seed(0)
+    layer = _Layer(_Mlp(512, 256) if kind == "mlp" else _Moe(256, 128, 6, 2))
+    if kind == "mlp":
+        assert fuse_same_input(layer) == 1                          # gate+up as one launch, inside the graph as well
+    eager = layer.mlp
+    assert install_block_graphs(layer) == 1 and isinstance(layer.mlp, GraphedBlock)
+    assert install_block_graphs(layer) == 0                         # already wrapped
+    h = 512 if kind == "mlp" else 256
+    for rows in (1, 4):
+        xs = [torch.randn(rows, h, device=DEV).to(torch.bfloat16) for _ in range(5)]
+        want = [eager(x).clone() for x in xs]
+        for rep in range(5):                                        # call 1 eager, call 2 captures, 3.. replay
+            got = layer.mlp(xs[rep])
+            torch.cuda.synchronize()
+            _ = (xs[rep].float() @ xs[rep].float().T).sum().item()  # the program's own eager work between replays
+            assert torch.equal(got, want[rep]), (kind, rows, rep)
+    assert sum(1 for v in layer.mlp._graphs.values() if isinstance(v, tuple)) == 2
+    big = torch.randn(64, h, device=DEV).to(torch.bfloat16)         # prefill-sized input: eager, no new graph
+    assert torch.equal(layer.mlp(big), eager(big))
+    assert sum(1 for v in layer.mlp._graphs.values() if isinstance(v, tuple)) == 2
