@@ -129,3 +129,24 @@ def test_embedding_fp16_output_of_a_two_table_pack_needs_its_fp16_list(tmp_path)
 def test_registry_names_the_embedding():
     from qvb8_amd.common.formats import get_format
     assert get_format("qvb8").embedding is QVBandEmbeddingV8 and get_format("qvband").embedding is QVBandEmbeddingV8
+
+
+def test_lookup_rows_refusals_through_the_c_abi():
+    """Argument errors come back as a status and a message, nothing is launched."""
+    from qvb8_amd import _lib
+    lib = _lib.load()
+    d = H.mixed_width_pack(8, 256, [6], seed=1)
+    ids, min_s, nbits, bit_off, P, tau_s, _, _ = H.to_device_args(d, DEV)
+    rows = torch.zeros(4, dtype=torch.int64, device=DEV)
+    out = torch.empty(4 * P + 8, dtype=torch.float32, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+
+    def call(rows_ptr=rows.data_ptr(), n=4, Q=8, out_dtype=_lib.F32, out_ptr=out.data_ptr(), esc=(None, None, 0), ids_ptr=ids.data_ptr()):
+        return lib.qvb8_lookup_rows(rows_ptr, n, ids_ptr, ids.numel(), min_s.data_ptr(), tau_s.data_ptr(), nbits.data_ptr(),
+                                    bit_off.data_ptr(), Q, P, esc[0], esc[1], esc[2], out_dtype, out_ptr, st)
+    assert call() == 0
+    assert call(n=0, rows_ptr=None) == 0                          # nothing to look up
+    for bad in (dict(out_dtype=7), dict(rows_ptr=None), dict(out_ptr=out.data_ptr() + 4), dict(out_ptr=None), dict(n=-1),
+                dict(esc=(None, None, 3)), dict(Q=0), dict(ids_ptr=ids.data_ptr() + 1)):
+        assert call(**bad) != 0, bad
+        assert lib.qvb8_last_error().decode().startswith("qvb8_lookup_rows"), bad
