@@ -235,6 +235,30 @@ int qvb8r_gemv(const void* X, int x_dtype, int64_t M, const qvb8r_core* core, in
 int qvb8r_fix_escapes(const void* X, int x_dtype, int64_t M, const int64_t* uq, const int64_t* ptr, const int64_t* ec,
                       const float* ed, int64_t U, float* Y, int64_t Q, int64_t P, void* stream);
 
+/* Attention of query rows over a banded KV cache whose keys and values stay ids in memory: per split of the key tiles
+ * the unnormalised result and the softmax state, which the caller combines (o * exp(m - max m) summed, over the
+ * likewise weighted l).
+ *   q      fp16, (tokens, q heads, head_dim) with strides sq_r / sq_h in elements, head_dim contiguous; row r of a kv
+ *          head is token r / G, q head h * G + r % G; the token's position is q_pos0 + r / G
+ *   ki, vi ids, (capacity, kv heads, head_dim) with strides s_n / s_h in ids; id_bytes = 1 (uint8) or 2 (uint16)
+ *   kmid, kstep, vmid, vstep  f32 (segments, kv heads, head_dim) contiguous; kc, vc f32 (segments, kv heads):
+ *          k = fp16(kmid + kstep * ((float)id - kc)), one fused multiply-add in fp32; v likewise
+ *   ts, tl, tseg  i32[n_tiles]: first key, length (1..32) and segment of each tile, first keys ascending; split s
+ *          takes tiles s * tps .. min((s + 1) * tps, n_tiles) - 1; a key at position p counts for a row when
+ *          p <= the row's position
+ *   o (n_splits, kv heads, n_rows, head_dim), m and l (n_splits, kv heads, n_rows)  f32, written completely
+ *          (a row that sees no key of a split: m = -inf, l = 0, o = 0)
+ * S = q k^T is accumulated in fp32 from fp16 operands, multiplied by `scale`; the probabilities exp(s - m) are rounded
+ * to fp16 before they are summed into l and multiplied with v (fp32 accumulate).  head_dim 128 or 256.
+ * Replaces: ext.fwd  qvattn_fwd kv/cuda_attn/qvattn_cuda.cu:97-255, host :257-287 (called from attend,
+ * kv/fused_attn.py:246-316, which also does the combination). */
+int qvb8_attn_fwd(const void* q, int64_t sq_r, int64_t sq_h, const void* ki, const void* vi, int id_bytes,
+                  int64_t s_n, int64_t s_h, const float* kmid, const float* kstep, const float* vmid,
+                  const float* vstep, const float* kc, const float* vc, const int32_t* ts, const int32_t* tl,
+                  const int32_t* tseg, int64_t n_tiles, float* o, float* m, float* l, int64_t n_splits,
+                  int64_t n_rows, int64_t n_kv_heads, int64_t head_dim, int64_t q_pos0, int64_t tps,
+                  double scale, int64_t G, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,113 @@
+"""Per-channel affine KV codec (reference: src/qv_band/kv/codec.py): fixed bits per element of a (seq, head_dim)
+segment of one kv head, one (min_s, tau_s) per channel,
+
+    id = round((x - min_c) / step_c),  step_c = (max_c - min_c) / (2^B - 1),  recon = min_c + id * step_c,
+
+no escapes (minimum and maximum cover every value).  The encoder runs as torch ops on the tensor's device; the ids are
+kept bit-packed, LSB first, row-major (codec.py:53-82), as the cache stores them between attention calls.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+
+STEP_FLOOR = 1e-12
+MAX_BITS = 16
+
+
+class KVCertificateError(ValueError):
+    """tau is below what 16 bits per element can certify for a head (codec.py:171-172)."""
+
+
+def pack_ids(ids: torch.Tensor, bits: int) -> torch.Tensor:
+    """Flat ids (< 2^bits) -> uint8, fields LSB first and bit-contiguous (codec.py:53-68)."""
+    n = ids.numel()
+    shifts = torch.arange(bits, device=ids.device, dtype=torch.int64)
+    stream = ((ids.reshape(-1, 1).to(torch.int64) >> shifts) & 1).to(torch.uint8).reshape(-1)
+    pad = (-stream.numel()) % 8
+    if pad:
+        stream = torch.cat([stream, stream.new_zeros(pad)])
+    weights = (1 << torch.arange(8, device=ids.device, dtype=torch.int64)).to(torch.uint8)
+    out = (stream.reshape(-1, 8) * weights).sum(dim=1, dtype=torch.int64).to(torch.uint8)
+    assert out.numel() == (n * bits + 7) // 8
+    return out
+
+
+def unpack_ids(packed: torch.Tensor, bits: int, n: int) -> torch.Tensor:
+    """Inverse of pack_ids: int64[n] (codec.py:71-82)."""
+    shifts = torch.arange(8, device=packed.device, dtype=torch.int64)
+    stream = ((packed.reshape(-1, 1).to(torch.int64) >> shifts) & 1).reshape(-1)[: n * bits].reshape(n, bits)
+    return (stream << torch.arange(bits, device=packed.device, dtype=torch.int64)).sum(dim=1)
+
+
+@dataclass(eq=False)
+class BandedKV:
+    """One kv head of one segment (codec.py:99-166)."""
+    packed: torch.Tensor            # uint8, bits * seq * head_dim bits, row-major
+    min_s: torch.Tensor             # (head_dim,) fp32
+    tau_s: torch.Tensor             # (head_dim,) fp32 step per channel
+    bits: int
+    orig_shape: tuple               # (seq, head_dim)
+    orig_dtype: torch.dtype
+    tau: float
+
+    def nbytes(self) -> int:
+        return int(self.packed.numel() + 4 * (self.min_s.numel() + self.tau_s.numel()))
+
+    @property
+    def max_error(self) -> float:
+        return float(self.tau_s.max()) * 0.5
+
+    def ids(self) -> torch.Tensor:
+        seq, hd = self.orig_shape
+        return unpack_ids(self.packed, self.bits, seq * hd).reshape(seq, hd)
+
+    def decode_all_torch(self, device=None, dtype=torch.float32) -> torch.Tensor:
+        """min_s + id * tau_s in fp32, rounded once to `dtype` (codec.py:117-118)."""
+        dev = self.packed.device if device is None else torch.device(device)
+        ids = self.ids().to(dev)
+        return (self.min_s.to(dev) + ids.to(torch.float32) * self.tau_s.to(dev)).to(dtype)
+
+    def truncate(self, n_rows: int) -> "BandedKV":
+        """The first n_rows tokens, not re-quantised: a byte prefix of `packed` (codec.py:120-139)."""
+        seq, hd = self.orig_shape
+        if not 0 < n_rows <= seq:
+            raise ValueError(f"truncate({n_rows}) outside 1..{seq}")
+        if n_rows == seq:
+            return self
+        nbytes = (n_rows * hd * self.bits + 7) // 8
+        return BandedKV(self.packed[:nbytes].clone(), self.min_s, self.tau_s, self.bits, (n_rows, hd), self.orig_dtype, self.tau)
+
+
+def band_kv_heads(t: torch.Tensor, orig_dtype: torch.dtype, bits: int, tau: float = 0.0, certify: bool = True) -> list:
+    """(heads, seq, head_dim) -> one BandedKV per head (codec.py:175-241).  With certify and tau > 0, `bits` is a floor:
+    a head's width rises (to 16 at most) until the decoder's own expression, rounded to `orig_dtype`, is within tau of
+    every element; KVCertificateError when 16 bits do not reach it."""
+    h, s, d = t.shape
+    x = torch.nan_to_num(t.detach().to(torch.float32), nan=0.0, posinf=0.0, neginf=0.0)
+    mn = x.amin(1, keepdim=True)
+    rng = x.amax(1, keepdim=True) - mn
+    do_cert = certify and tau > 0
+    if do_cert:
+        worst = rng.amax((1, 2)).cpu().tolist()
+        widths = [min(MAX_BITS, max(bits, math.ceil(math.log2(w / (2.0 * tau) + 1.0)))) if w > 0 else bits for w in worst]
+    else:
+        widths = [bits] * h
+    while True:
+        top = torch.tensor([float((1 << b) - 1) for b in widths], device=x.device).view(h, 1, 1)
+        step = (rng / top).clamp_min(STEP_FLOOR)
+        ids = torch.minimum(torch.round((x - mn) / step).clamp_(min=0), top)
+        if not do_cert:
+            break
+        errs = ((mn + ids * step).to(orig_dtype).to(torch.float32) - x).abs().amax((1, 2)).cpu().tolist()
+        bad = [i for i in range(h) if errs[i] > tau]
+        if not bad:
+            break
+        for i in bad:
+            if widths[i] >= MAX_BITS:
+                raise KVCertificateError(f"head {i}: {MAX_BITS}-bit per-channel error {errs[i]:.4g} > tau={tau:g}")
+            widths[i] += 1
+    return [BandedKV(pack_ids(ids[i].to(torch.int64).reshape(-1), widths[i]), mn[i, 0].contiguous(), step[i, 0].contiguous(),
+                     widths[i], (s, d), orig_dtype, tau) for i in range(h)]

@@ -1,0 +1,147 @@
+"""Attention straight over the banded KV cache's ids (reference: src/qv_band/kv/fused_attn.py:155-316): the ids of all
+segments of a layer lie in one (capacity, kv heads, head_dim) buffer, the affine constants per segment / head / channel
+beside them, and the kernel restores keys and values tile by tile -- nothing of the context's size is ever built.
+
+`attend` is the reference's call: it folds the softmax scale into the queries, launches qvb8_attn_fwd through the C ABI
+and combines the splits.  There is no other backend: without the HIP library it raises.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from qvb8_amd import _lib
+
+BLOCK_N = 32          # keys per tile of the table; the kernel takes tiles of at most 32 keys
+ROWS_PER_BLOCK = 16   # query rows one workgroup of the kernel handles
+
+
+class QVLayout:
+    """The id buffers, constants and tile table of one layer (fused_attn.py:155-186).  ki / vi: (capacity, Hkv, D)
+    uint8, or int16 holding 16-bit patterns; kmin / vmin hold the range CENTRE when kc / vc are given."""
+
+    def __init__(self, ki, vi, kmin, kstep, vmin, vstep, seg_len, device, block_n=BLOCK_N, kc=None, vc=None):
+        if block_n > BLOCK_N:
+            raise ValueError(f"tiles of {block_n} keys: the kernel takes at most {BLOCK_N}")
+        self.block_n = block_n
+        n_seg = len(seg_len)
+        zeros = lambda: torch.zeros(n_seg, kmin.shape[1], dtype=torch.float32, device=device)     # noqa: E731
+        self.kc = kc if kc is not None else zeros()
+        self.vc = vc if vc is not None else zeros()
+        self.ki, self.vi = ki, vi
+        self.kmin, self.kstep, self.vmin, self.vstep = kmin, kstep, vmin, vstep
+        self.n = int(sum(seg_len))
+        starts, lens, segs, pos = [], [], [], 0
+        for si, sl in enumerate(seg_len):
+            for a in range(0, sl, block_n):
+                starts.append(pos + a)
+                lens.append(min(block_n, sl - a))
+                segs.append(si)
+            pos += sl
+        table = torch.tensor([starts, lens, segs], dtype=torch.int32).reshape(3, -1).to(device)
+        self.t_start, self.t_len, self.t_seg = table[0].contiguous(), table[1].contiguous(), table[2].contiguous()
+        self.n_tiles = len(starts)
+
+
+def layout_from_segments(segs_k, segs_v, seg_len, device, allow_wide: bool = False):
+    """segs_*: per segment a list with one BandedKV per kv head (fused_attn.py:189-216).  Returns None when a head uses
+    more than 8 bits -- unless allow_wide, which stores every id in 16 bits instead (the kernel reads either)."""
+    nseg, h = len(segs_k), len(segs_k[0])
+    n = sum(seg_len)
+    d = segs_k[0][0].orig_shape[1]
+    wide = any(bk.bits > 8 for store in (segs_k, segs_v) for seg in store for bk in seg)
+    if wide and not allow_wide:
+        return None
+    dt = torch.int16 if wide else torch.uint8
+    ki = torch.empty(n, h, d, dtype=dt, device=device)
+    vi = torch.empty_like(ki)
+    P = [torch.empty(nseg, h, d, dtype=torch.float32, device=device) for _ in range(4)]
+    KC = torch.zeros(nseg, h, dtype=torch.float32, device=device)
+    VC = torch.zeros_like(KC)
+    pos = 0
+    for si in range(nseg):
+        sl = seg_len[si]
+        for hi in range(h):
+            for store, ids_t, mid, st, C in ((segs_k, ki, P[0], P[1], KC), (segs_v, vi, P[2], P[3], VC)):
+                bk = store[si][hi]
+                ids = bk.ids().to(device)
+                ids_t[pos:pos + sl, hi] = (ids.to(torch.int32) - ((ids > 32767).to(torch.int32) << 16)).to(dt) if wide else ids.to(dt)
+                c = ((1 << bk.bits) - 1) / 2.0
+                mid[si, hi] = (bk.min_s + bk.tau_s * c).to(device)      # range centre
+                st[si, hi] = bk.tau_s.to(device)
+                C[si, hi] = c
+        pos += sl
+    return QVLayout(ki, vi, P[0], P[1], P[2], P[3], list(seg_len), device, kc=KC, vc=VC)
+
+
+def fwd(q, ki, vi, kmid, kstep, vmid, vstep, kc, vc, ts, tl, tseg, o, m, l, q_pos0: int, tps: int, scale: float, G: int) -> None:
+    """The compiled kernel's call (ext.fwd, kv/cuda_attn/qvattn_cuda.cu:262-287): fills o (S, Hkv, R, D), m, l (S, Hkv, R)."""
+    if q.dtype != torch.float16 or q.stride(2) != 1:
+        raise RuntimeError("q must be fp16, contiguous in D")
+    wide = ki.dtype == torch.int16
+    if not (wide or ki.dtype == torch.uint8) or vi.dtype != ki.dtype or ki.stride(2) != 1 or ki.stride() != vi.stride():
+        raise RuntimeError("ids layout")
+    for p in (kmid, kstep, vmid, vstep, kc, vc, ts, tl, tseg, o, m, l):
+        if not p.is_contiguous() or p.device != q.device:
+            raise RuntimeError("constants, tile table and outputs must be contiguous and on q's device")
+    if ts.dtype != torch.int32 or tl.dtype != torch.int32 or tseg.dtype != torch.int32 or o.dtype != torch.float32:
+        raise RuntimeError("tile table must be int32, outputs fp32")
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        rc = lib.qvb8_attn_fwd(q.data_ptr(), q.stride(0), q.stride(1), ki.data_ptr(), vi.data_ptr(), 2 if wide else 1,
+                               ki.stride(0), ki.stride(1), kmid.data_ptr(), kstep.data_ptr(), vmid.data_ptr(), vstep.data_ptr(),
+                               kc.data_ptr(), vc.data_ptr(), ts.data_ptr(), tl.data_ptr(), tseg.data_ptr(), ts.numel(),
+                               o.data_ptr(), m.data_ptr(), l.data_ptr(), o.shape[0], o.shape[2], ki.shape[1], q.shape[2],
+                               int(q_pos0), int(tps), float(scale), int(G), torch.cuda.current_stream().cuda_stream)
+    _lib._check(rc, lib)
+
+
+def plan_splits(n_tiles: int, hkv: int, rows: int, device) -> tuple:
+    """(tiles per split, splits): enough workgroups to fill the card (four fit a compute unit), fewer splits for long
+    query blocks (fused_attn.py:259-264, 271-275)."""
+    n_rb = -(-rows // ROWS_PER_BLOCK)
+    want = 4 * torch.cuda.get_device_properties(device).multi_processor_count
+    n_splits = max(1, min(n_tiles, want // max(1, hkv * n_rb)))
+    tps = max(1, math.ceil(n_tiles / n_splits))
+    return tps, max(1, math.ceil(n_tiles / tps))
+
+
+def combine_splits(o, m, l):
+    """Per-split (unnormalised o, running max m, running sum l) -> (normalised result, log-sum-exp) per kv head and row:
+    every split is weighted by exp(m - max over splits); a row no split saw a key for gives 0 and -inf
+    (fused_attn.py:302-314; one split is the same formula with weight 1)."""
+    top = m.amax(dim=0)
+    top = torch.where(torch.isinf(top), torch.zeros_like(top), top)
+    w = torch.exp(m - top)
+    total = (l * w).sum(0)
+    out = (o * w.unsqueeze(-1)).sum(0) / total.clamp_min(1e-30).unsqueeze(-1)
+    lse = torch.where(total > 0, top + torch.log(total.clamp_min(1e-30)), torch.full_like(total, float("-inf")))
+    return out, lse
+
+
+def attend(q, lay: QVLayout, q_pos0: int, scale: float, n_splits: int | None = None):
+    """q: (MQ, Hq, D) bf16 / fp16 queries at positions q_pos0 .. q_pos0 + MQ - 1.  Returns (o (MQ, Hq, D) fp32, lse
+    (MQ, Hq) fp32) over the banded keys with position <= the query's; rows without a visible key get lse = -inf
+    (fused_attn.py:246-316)."""
+    mq, hq, d = q.shape
+    hkv = lay.ki.shape[1]
+    g = hq // hkv
+    rows = mq * g
+    if n_splits is None:
+        tps, n_splits = plan_splits(lay.n_tiles, hkv, rows, q.device)
+    else:
+        tps = max(1, math.ceil(lay.n_tiles / max(1, n_splits)))
+        n_splits = max(1, math.ceil(lay.n_tiles / tps))
+    # fp16 queries: the softmax scale goes in first (|q| shrinks), then they saturate, so that an outlier channel cannot
+    # turn into inf and a row into NaN (fused_attn.py:276-279)
+    q16 = (q.float() * scale).clamp_(-65504.0, 65504.0).to(torch.float16).contiguous()
+    o = torch.empty(n_splits, hkv, rows, d, dtype=torch.float32, device=q.device)
+    m = torch.empty(n_splits, hkv, rows, dtype=torch.float32, device=q.device)
+    l = torch.empty_like(m)
+    fwd(q16, lay.ki, lay.vi, lay.kmin, lay.kstep, lay.vmin, lay.vstep, lay.kc.contiguous(), lay.vc.contiguous(),
+        lay.t_start, lay.t_len, lay.t_seg, o, m, l, q_pos0, tps, 1.0, g)
+    out, lse = combine_splits(o, m, l)
+    out = out.reshape(hkv, mq, g, d).permute(1, 0, 2, 3).reshape(mq, hq, d)
+    lse = lse.reshape(hkv, mq, g).permute(1, 0, 2).reshape(mq, hq)
+    return out, lse
