@@ -380,6 +380,71 @@ def bench_lmhead(args, dev):
             "cpu_baseline": None}
 
 
+def bench_attn(args, dev):
+    """Decode-step attention over a banded KV cache: `--layers` (default 16) distinct caches of `--context` keys (default
+    32768; 4 kv heads x 256 channels, 6-bit ids in bytes, segments of 4096 keys), 24 query heads, `--tokens` query
+    tokens at the end of the context.  A step = per layer one launch of qvb8_attn_fwd plus one of qvb8_attn_combine,
+    all in one graph; the kernel alone is timed by a second graph for the roofline.  Bytes per launch: the
+    ids of K and V once, the per-channel constants, q, and the per-split results written."""
+    import torch
+    from qvb8_amd.kv import codec as KC, fused_attn as FA
+    n, hkv, G, D, seg, MQ = args.context, 4, 6, 256, 4096, args.tokens
+    gen = torch.Generator(device=dev).manual_seed(5)
+    lays = []
+    for li in range(args.layers):
+        segs_k, segs_v, seg_len = [], [], []
+        for a in range(0, n, seg):
+            sl = min(seg, n - a)
+            k = (torch.randn(hkv, sl, D, device=dev, generator=gen) * (0.5 + 2 * torch.rand(hkv, 1, D, device=dev, generator=gen))).to(torch.bfloat16)
+            v = torch.randn(hkv, sl, D, device=dev, generator=gen).to(torch.bfloat16)
+            segs_k.append(KC.band_kv_heads(k, torch.bfloat16, 6, certify=False))
+            segs_v.append(KC.band_kv_heads(v, torch.bfloat16, 6, certify=False))
+            seg_len.append(sl)
+        lays.append(FA.layout_from_segments(segs_k, segs_v, seg_len, dev))
+    lay0 = lays[0]
+    rows = MQ * G
+    tps, n_splits = FA.plan_splits(lay0.n_tiles, hkv, rows, dev)
+    scale = D ** -0.5
+    q = torch.randn(MQ, hkv * G, D, device=dev, generator=gen).to(torch.bfloat16)
+    q16 = (q.float() * scale).clamp_(-65504.0, 65504.0).to(torch.float16).contiguous()
+    o = [torch.empty(n_splits, hkv, rows, D, device=dev) for _ in lays]
+    m = [torch.empty(n_splits, hkv, rows, device=dev) for _ in lays]
+    l = [torch.empty_like(x) for x in m]
+    outs = [None] * len(lays)
+
+    def kernels_only():
+        for i, lay in enumerate(lays):
+            FA.fwd(q16, lay.ki, lay.vi, lay.kmin, lay.kstep, lay.vmin, lay.vstep, lay.kc, lay.vc, lay.t_start, lay.t_len,
+                   lay.t_seg, o[i], m[i], l[i], n - MQ, tps, 1.0, G)
+
+    def step():
+        for i, lay in enumerate(lays):
+            FA.fwd(q16, lay.ki, lay.vi, lay.kmin, lay.kstep, lay.vmin, lay.vstep, lay.kc, lay.vc, lay.t_start, lay.t_len,
+                   lay.t_seg, o[i], m[i], l[i], n - MQ, tps, 1.0, G)
+            outs[i] = FA.combine_splits(o[i], m[i], l[i], G)
+    k_ms, _ = time_graph(kernels_only, args.steps, args.warmup)
+    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
+    ms = max(ev_ms, wall_ms)
+    n_seg = len(lay0.kc)
+    nbytes = int(2 * lay0.ki.numel() * lay0.ki.element_size() + 4 * 4 * n_seg * hkv * D + 2 * MQ * hkv * G * D
+                 + 4 * n_splits * hkv * rows * (D + 2) + 12 * lay0.n_tiles)
+    us = k_ms * 1e3 / len(lays)
+    gbs_kernel = nbytes / (us * 1e-6) / 1e9
+    gbs = nbytes * len(lays) / (ms * 1e-3) / 1e9
+    return {"metric": "banded-KV attention HBM GB/s, decode step over %d keys, 1 MI355X" % n,
+            "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "fp16 restored keys and values, fp32 accumulate", "data": "synthetic",
+            "config": {"workload": "attention of %d query token(s), 24 heads over %d kv heads x 256 channels, %d keys as 6-bit ids "
+                                   "in bytes in segments of %d, %d layers with their own caches, %d splits of %d tiles"
+                                   % (MQ, hkv, n, seg, len(lays), n_splits, tps),
+                       "bytes_per_launch": nbytes, "us_per_layer": round(ms * 1e3 / len(lays), 2)},
+            "roofline": {"bound": "hbm", "achieved": round(gbs_kernel, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs_kernel / HBM_PEAK_GBS, 4), "traffic": None,
+                         "kernel": "qvb8::attn_kernel<256, unsigned char>", "bytes_per_launch": nbytes, "launch_us": round(us, 3)},
+            "cpu_baseline": None}
+
+
 def bench_smallm(args, dev):
     """Config 3: the 9B projections with M = `--tokens` rows (draft-verify / prefill chunk), through QVBandLinearV8's own
     dispatch: M <= 48 the tile kernel (X in registers), 49..256 the workgroup-tiled decode + GEMM kernel (X staged in LDS,
@@ -425,9 +490,10 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=None, help="layers of distinct packs (default 32; moe 4; qvb8r 2)")
-    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead", "embed"), default="decode9b",
+    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead", "embed", "attn"), default="decode9b",
                     help="decode9b (default, the headline metric): 9B-shape decode step; moe: 35B-A3B-shape expert stack; "
                          "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256)")
+    ap.add_argument("--context", type=int, default=32768, help="keys in the cache of the attn workload")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
     ap.add_argument("--model", choices=("9b", "27b"), default="9b",
                     help="decode9b workload only: layer shapes (9b = the headline configuration; 27b = hidden 5120, FFN 17408)")
@@ -454,9 +520,9 @@ def main():
     torch.cuda.set_device(dev)
     lib = _lib.load()                                       # raises when the HIP library is missing: no fallback
     if args.layers is None:
-        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 2, "lmhead": 1, "embed": 1}[args.workload]
+        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 2, "lmhead": 1, "embed": 1, "attn": 16}[args.workload]
     if args.workload != "decode9b":
-        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead, "embed": bench_embed}[args.workload]
+        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead, "embed": bench_embed, "attn": bench_attn}[args.workload]
         print(json.dumps(fn(args, dev)))
         return 0
     if args.no_sort:

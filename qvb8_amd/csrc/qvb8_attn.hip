@@ -10,18 +10,22 @@
 // probabilities rounded to fp16 before they are summed and multiplied; the result per split is the unnormalised
 // accumulator plus (running max, running sum), which the caller combines.
 //
-// Shape of this kernel (gfx950): 128 threads = 2 waves per workgroup, 16 query rows, 32 keys per tile.
-//   * ids are requested one tile ahead into registers: a wave reads whole key rows (64 lanes x 4 ids = 256 channels),
-//     every thread keeps the same four channels for all its keys, so it holds 4 + 4 constants per operand;
+// Shape of this kernel (gfx950): 256 threads = 4 waves per workgroup, 16 query rows, 32 keys per tile.
+//   * ids are requested TWO tiles ahead into two register sets (a trip to memory under load takes longer than one tile's
+//     arithmetic): a wave reads whole key rows (64 lanes x 4 ids = 256 channels), every thread keeps the same four
+//     channels for all its keys, so it holds 4 + 4 constants per operand; no request sits under a branch (a tile past
+//     the split's end re-reads one cached line), so the counted waits leave the younger set in flight;
 //   * restored K goes to LDS as [key][channel], restored V as [channel][key] (a thread owns 4 keys x 4 channels, so the
 //     transposition is free) with the 8-byte cells of a row swizzled by the channel group;
-//   * S = Q K^T: wave w takes keys 16 w .. 16 w + 15 (v_mfma_f32_16x16x16_f16, Q kept in registers as the A operand);
-//   * both waves do the softmax of all 16 rows from S in LDS (same inputs, same results; no state in LDS) in the
+//   * S = Q K^T: wave w takes keys 16 (w % 2) .. + 15 and half w / 2 of the channels (v_mfma_f32_16x16x16_f16, its part
+//     of Q kept in registers as the A operand); the two halves are added when S is read back;
+//   * all waves do the softmax of all 16 rows from S in LDS (same inputs, same results; no state in LDS) in the
 //     A-operand layout of the second product, so P needs no trip through LDS;
-//   * O += P V: wave w owns half of the output channels.
+//   * O += P V: wave w owns a quarter of the output channels.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <algorithm>
+#include <type_traits>
 #include <stdint.h>
 
 #include "qvb8_amd.h"
@@ -35,7 +39,7 @@ typedef float f4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kRows = 16;          // query rows per workgroup
 constexpr int kKeys = 32;          // keys per tile (the table's tiles are never longer)
-constexpr int kAttnThreads = 128;
+constexpr int kAttnThreads = 256;
 constexpr int kSStride = kKeys + 4;
 
 struct AttnArgs {
@@ -59,74 +63,114 @@ template <> struct Quad<uint16_t> {
     static __device__ __forceinline__ float id(type w, int c) { return (float)(((c < 2 ? w.x : w.y) >> (16 * (c & 1))) & 0xFFFFu); }
 };
 
+// One entry of the tile table through the scalar unit.  A plain load would do, but behind a barrier the compiler turns
+// it into a vector load, and waiting for that one (the youngest request) also waits for every id request still in
+// flight -- the prefetch would be worth nothing.
+struct TileRef { int start, nlen, seg; bool ok; };
+__device__ __forceinline__ void tile_entry(const int32_t* ts, const int32_t* tl, const int32_t* tseg, int t, TileRef& r) {
+    const uint32_t off = (uint32_t)__builtin_amdgcn_readfirstlane(t) * 4u;
+    int start, nlen, seg;
+    asm volatile("s_load_dword %0, %3, %6\n\ts_load_dword %1, %4, %6\n\ts_load_dword %2, %5, %6\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(start), "=&s"(nlen), "=&s"(seg) : "s"(ts), "s"(tl), "s"(tseg), "s"(off) : "memory");
+    r.start = start; r.nlen = nlen; r.seg = seg;
+}
+
 template <int D, typename T>
-__global__ __launch_bounds__(kAttnThreads) void attn_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_kernel(const AttnArgs a) {
     constexpr int CG = D / 4;                  // channel groups (four channels each) of a key
     constexpr int KSTEP = kAttnThreads / CG;   // key groups (four keys each) that one pass of the workgroup covers
-    constexpr int UNITS = D / 64;              // (4 keys x 4 channels) units per thread and tile
+    constexpr int UNITS = D / 128;             // (4 keys x 4 channels) units per thread and tile
     constexpr int KROW = D + 8;                // halfs per key in LDS
-    constexpr int NF = D / 32;                 // 16-channel output fragments per wave
+    constexpr int NF = D / 64;                 // 16-channel output fragments per wave
+    constexpr int NKS = D / 32;                // 16-channel steps of S = Q K^T per wave
     using QD = Quad<T>;
     using U = typename QD::type;
     __shared__ __align__(16) _Float16 Ks[kKeys * KROW];
     __shared__ __align__(16) _Float16 Vt[D * kKeys];
-    __shared__ __align__(16) float Ss[kRows * kSStride];
+    __shared__ __align__(16) float Ss[2 * kRows * kSStride];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n16 = lane & 15, kg = lane >> 4;
+    const int kf = wave & 1, dh = wave >> 1;                  // this wave's 16 keys and its half of the channels in S
     const int h = blockIdx.x, sp = blockIdx.y, row0 = blockIdx.z * kRows;
     const int cg = tid % CG, kgp0 = tid / CG;
 
-    // the lane's query row as the A operand of S = Q K^T: Q[row][16 ks + 4 kg .. + 3]
+    // the lane's query row as the A operand of S = Q K^T: Q[row][16 ks + 4 kg .. + 3], ks in the wave's half
     const int row = row0 + n16;
     const bool row_ok = row < a.n_rows;
     const int qpos = a.q_pos0 + (row_ok ? row / a.G : 0);
-    h4_t qa[D / 16];
+    h4_t qa[NKS];
     {
         const int rr = row_ok ? row : 0;
-        const uint16_t* qp = a.q + (int64_t)(rr / a.G) * a.sq_r + (int64_t)(h * a.G + rr % a.G) * a.sq_h + 4 * kg;
+        const uint16_t* qp = a.q + (int64_t)(rr / a.G) * a.sq_r + (int64_t)(h * a.G + rr % a.G) * a.sq_h + dh * (D / 2) + 4 * kg;
 #pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
+        for (int ks = 0; ks < NKS; ++ks) {
             const h4_t v = *reinterpret_cast<const h4_t*>(qp + 16 * ks);
             qa[ks] = row_ok ? v : h4_t{0, 0, 0, 0};
         }
     }
+    const int qmin = a.q_pos0 + row0 / a.G;                                   // first position of the block's rows
     const int qmax = a.q_pos0 + (min(row0 + kRows, a.n_rows) - 1) / a.G;      // last position any row of the block sees
 
     const T* ki = reinterpret_cast<const T*>(a.ki) + (int64_t)h * a.s_h + 4 * cg;
     const T* vi = reinterpret_cast<const T*>(a.vi) + (int64_t)h * a.s_h + 4 * cg;
-    U rk[UNITS][4], rv[UNITS][4];
-    // ids of tile t into registers; keys past the tile's length re-read its last key (never used)
-    auto fetch = [&](int t) {
-        const int start = a.ts[t], nlen = a.tl[t];
+    const int t0 = (int)min((int64_t)sp * a.tps, (int64_t)a.n_tiles), t1 = (int)min((int64_t)t0 + a.tps, (int64_t)a.n_tiles);
+    // ids of tile t into one register set: always 8 UNITS requests, none under a branch; keys past the tile's length
+    // re-read its last key, and a tile that is not wanted -- past the split's end, or starting behind the last visible
+    // position (tiles ascend: so do all after it) -- re-reads key 0 of the head (one cached line); neither is used.
+    // A request's address is the tile's first key (scalar) plus the thread's key offset, fixed for the whole kernel
+    // and clamped to the tile's last key (host-checked: 32 keys' stride fits 31 bits).
+    uint32_t key_off[UNITS][4];
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) key_off[u][j] = (uint32_t)(4 * (kgp0 + KSTEP * u) + j) * (uint32_t)a.s_n * (uint32_t)sizeof(T);
+    const unsigned char* kbytes = reinterpret_cast<const unsigned char*>(ki);
+    const unsigned char* vbytes = reinterpret_cast<const unsigned char*>(vi);
+    auto fetch = [&](int t, U (&rk)[UNITS][4], U (&rv)[UNITS][4], TileRef& ref) {
+        tile_entry(a.ts, a.tl, a.tseg, min(t, t1 - 1), ref);
+        ref.ok = __builtin_amdgcn_readfirstlane((int)(t < t1 && ref.start <= qmax)) != 0;      // scalar: the loop's branches stay uniform
+        const int start = ref.ok ? ref.start : 0, nlen = ref.ok ? ref.nlen : 1;
+        const int64_t tile_byte = (int64_t)start * a.s_n * (int64_t)sizeof(T);
+        const uint32_t last_off = (uint32_t)max(nlen - 1, 0) * (uint32_t)a.s_n * (uint32_t)sizeof(T);
+        const unsigned char* kb = kbytes + tile_byte;
+        const unsigned char* vb = vbytes + tile_byte;
 #pragma unroll
         for (int u = 0; u < UNITS; ++u)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int key = max(0, min(4 * (kgp0 + KSTEP * u) + j, nlen - 1));
-                const int64_t off = (int64_t)(start + key) * a.s_n;
-                rk[u][j] = *reinterpret_cast<const U*>(ki + off);
-                rv[u][j] = *reinterpret_cast<const U*>(vi + off);
+                const uint32_t off = min(key_off[u][j], last_off);
+                rk[u][j] = *reinterpret_cast<const U*>(kb + off);
+                rv[u][j] = *reinterpret_cast<const U*>(vb + off);
             }
     };
 
-    const int t0 = (int)min((int64_t)sp * a.tps, (int64_t)a.n_tiles), t1 = (int)min((int64_t)t0 + a.tps, (int64_t)a.n_tiles);
     float m_run = -INFINITY, l_run = 0.f;
     f4_t acc[NF];
 #pragma unroll
     for (int f = 0; f < NF; ++f) acc[f] = f4_t{0.f, 0.f, 0.f, 0.f};
 
-    bool have = t0 < t1 && a.ts[t0] <= qmax;            // tiles ascend: behind the first masked one all are masked
-    if (have) fetch(t0);
-    for (int t = t0; have; ++t) {
-        const int start = a.ts[t], nlen = a.tl[t], seg = a.tseg[t];
-        {
+    int cur_seg = -1;
+    float km[4] = {0.f, 0.f, 0.f, 0.f}, ks_[4] = {0.f, 0.f, 0.f, 0.f}, vm[4] = {0.f, 0.f, 0.f, 0.f}, vs_[4] = {0.f, 0.f, 0.f, 0.f}, kc = 0.f, vc = 0.f;
+    // One tile: restore the ids of register set (rk, rv) into LDS, refill the set with tile t + 2, S, softmax, O.
+    auto tile = [&](int t, U (&rk)[UNITS][4], U (&rv)[UNITS][4], TileRef& ref) {
+        const int start = ref.start, nlen = ref.nlen, seg = ref.seg;
+        if (seg != cur_seg) {
+            // A new segment (every few thousand keys): its constants for this thread's four channels.  The wait stands
+            // INSIDE the branch: the requests of the next tiles' ids are older than these, and a wait placed where the
+            // constants are first used would hold every tile until its successors' ids had arrived.
             const int64_t pb = ((int64_t)seg * a.nhkv + h) * D + 4 * cg;
             const float4 kmid = *reinterpret_cast<const float4*>(a.kmid + pb), kstep = *reinterpret_cast<const float4*>(a.kstep + pb);
             const float4 vmid = *reinterpret_cast<const float4*>(a.vmid + pb), vstep = *reinterpret_cast<const float4*>(a.vstep + pb);
-            const float kc = a.kc[seg * a.nhkv + h], vc = a.vc[seg * a.nhkv + h];
-            const float km[4] = {kmid.x, kmid.y, kmid.z, kmid.w}, ks_[4] = {kstep.x, kstep.y, kstep.z, kstep.w};
-            const float vm[4] = {vmid.x, vmid.y, vmid.z, vmid.w}, vs_[4] = {vstep.x, vstep.y, vstep.z, vstep.w};
+            kc = a.kc[seg * a.nhkv + h]; vc = a.vc[seg * a.nhkv + h];
+            km[0] = kmid.x; km[1] = kmid.y; km[2] = kmid.z; km[3] = kmid.w;
+            ks_[0] = kstep.x; ks_[1] = kstep.y; ks_[2] = kstep.z; ks_[3] = kstep.w;
+            vm[0] = vmid.x; vm[1] = vmid.y; vm[2] = vmid.z; vm[3] = vmid.w;
+            vs_[0] = vstep.x; vs_[1] = vstep.y; vs_[2] = vstep.z; vs_[3] = vstep.w;
+            __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0)
+            cur_seg = seg;
+        }
+        auto restore = [&](auto full) {
 #pragma unroll
             for (int u = 0; u < UNITS; ++u) {
                 const int kgp = kgp0 + KSTEP * u;
@@ -134,13 +178,13 @@ __global__ __launch_bounds__(kAttnThreads) void attn_kernel(const AttnArgs a) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int key = 4 * kgp + j;
-                    const bool live = key < nlen;
+                    const bool live = decltype(full)::value || key < nlen;
                     h4_t kv;
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        const float kf = __builtin_fmaf(ks_[c], QD::id(rk[u][j], c) - kc, km[c]);
+                        const float kf_ = __builtin_fmaf(ks_[c], QD::id(rk[u][j], c) - kc, km[c]);
                         const float vf = __builtin_fmaf(vs_[c], QD::id(rv[u][j], c) - vc, vm[c]);
-                        kv[c] = live ? (_Float16)kf : (_Float16)0.f;
+                        kv[c] = live ? (_Float16)kf_ : (_Float16)0.f;
                         vcell[c][j] = live ? (_Float16)vf : (_Float16)0.f;
                     }
                     *reinterpret_cast<h4_t*>(Ks + key * KROW + 4 * cg) = kv;
@@ -149,35 +193,39 @@ __global__ __launch_bounds__(kAttnThreads) void attn_kernel(const AttnArgs a) {
                 for (int c = 0; c < 4; ++c)
                     *reinterpret_cast<h4_t*>(Vt + (4 * cg + c) * kKeys + 4 * (kgp ^ (cg & 7))) = vcell[c];
             }
-        }
+        };
+        if (nlen == kKeys) restore(std::true_type{});        // a whole tile: no key to blank out
+        else restore(std::false_type{});
         __syncthreads();
-        const bool more = t + 1 < t1 && a.ts[t + 1] <= qmax;
-        if (more) fetch(t + 1);
+        fetch(t + 2, rk, rv, ref);
 
-        // ---- S = Q K^T for this wave's 16 keys ----
+        // ---- S = Q K^T: this wave's 16 keys, its half of the channels ----
         {
             f4_t s = {0.f, 0.f, 0.f, 0.f};
-            const _Float16* kp = Ks + (16 * wave + n16) * KROW + 4 * kg;
+            const _Float16* kp = Ks + (16 * kf + n16) * KROW + dh * (D / 2) + 4 * kg;
 #pragma unroll
-            for (int ks = 0; ks < D / 16; ++ks)
+            for (int ks = 0; ks < NKS; ++ks)
                 s = __builtin_amdgcn_mfma_f32_16x16x16f16(qa[ks], *reinterpret_cast<const h4_t*>(kp + 16 * ks), s, 0, 0, 0);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) Ss[(4 * kg + e) * kSStride + 16 * wave + n16] = s[e];
+            for (int e = 0; e < 4; ++e) Ss[(dh * kRows + 4 * kg + e) * kSStride + 16 * kf + n16] = s[e];
         }
         __syncthreads();
 
         // ---- softmax of row n16 over the tile: this lane holds keys 16 kk + 4 kg + i ----
         h4_t pa[2];
         float alpha;
+        // every key of the tile counts for every row of the block (rows past n_rows compute on zeros and are never stored)
+        const bool all_seen = nlen == kKeys && start + kKeys - 1 <= qmin;
         {
             float sv[8], mx = -INFINITY;
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
-                const f4_t s4 = *reinterpret_cast<const f4_t*>(Ss + n16 * kSStride + 16 * kk + 4 * kg);
+                const f4_t s4 = *reinterpret_cast<const f4_t*>(Ss + n16 * kSStride + 16 * kk + 4 * kg)
+                                + *reinterpret_cast<const f4_t*>(Ss + (kRows + n16) * kSStride + 16 * kk + 4 * kg);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int n = 16 * kk + 4 * kg + i;
-                    const bool ok = row_ok && n < nlen && start + n <= qpos;
+                    const bool ok = all_seen || (row_ok && n < nlen && start + n <= qpos);
                     sv[4 * kk + i] = ok ? s4[i] * a.scale : -INFINITY;
                     mx = fmaxf(mx, sv[4 * kk + i]);
                 }
@@ -216,12 +264,29 @@ __global__ __launch_bounds__(kAttnThreads) void attn_kernel(const AttnArgs a) {
         for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
             for (int f = 0; f < NF; ++f) {
-                const int ch = wave * (D / 2) + 16 * f + n16;
+                const int ch = wave * (D / 4) + 16 * f + n16;
                 const h4_t b = *reinterpret_cast<const h4_t*>(Vt + ch * kKeys + 4 * ((4 * kk + kg) ^ ((ch >> 2) & 7)));
                 acc[f] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[kk], b, acc[f], 0, 0, 0);
             }
         __syncthreads();                                  // the tile in LDS is free again
-        have = more;
+    };
+
+    if (t0 < t1) {
+        U rk0[UNITS][4], rv0[UNITS][4], rk1[UNITS][4], rv1[UNITS][4];
+        TileRef ref0, ref1;
+        fetch(t0, rk0, rv0, ref0);
+        __builtin_amdgcn_sched_barrier(0);                 // set 0 is the older one, as in every later round of the loop
+        fetch(t0 + 1, rk1, rv1, ref1);
+        __builtin_amdgcn_sched_barrier(0);
+        // The loop has one way out, at its head, and takes tiles in pairs; a last odd tile follows it.  (A way out of the
+        // middle is turned into a path through the loop's end back to its head: on that path set 0 would be the younger
+        // one, and the compiler would make every round wait for both sets.)
+        int t = t0;
+        for (; ref0.ok && ref1.ok; t += 2) {
+            tile(t, rk0, rv0, ref0);
+            tile(t + 1, rk1, rv1, ref1);
+        }
+        if (ref0.ok) tile(t, rk0, rv0, ref0);
     }
 
     const int64_t base = ((int64_t)sp * a.nhkv + h) * a.n_rows;
@@ -230,11 +295,55 @@ __global__ __launch_bounds__(kAttnThreads) void attn_kernel(const AttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int r = row0 + 4 * kg + e;
-            if (r < a.n_rows) a.o[(base + r) * D + wave * (D / 2) + 16 * f + n16] = acc[f][e];
+            if (r < a.n_rows) a.o[(base + r) * D + wave * (D / 4) + 16 * f + n16] = acc[f][e];
         }
     if (wave == 0 && kg == 0 && row_ok) {
         a.m[base + row] = m_run;
         a.l[base + row] = l_run;
+    }
+}
+
+// Splits -> the normalised result and the log-sum-exp.  One workgroup per (kv head, row, 64 channels): 16 groups of 16
+// threads share the splits (group g takes splits g, g + 16, ...), a thread holds four channels; the groups' maxima,
+// sums and partial results meet in LDS.  Every load of a thread is independent of the others, so the launch costs a few
+// trips to memory, not one per split.
+__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ o, const float* __restrict__ m, const float* __restrict__ l,
+                                                            int n_splits, int nhkv, int n_rows, int D, int G,
+                                                            float* __restrict__ out, float* __restrict__ lse) {
+    __shared__ float s_top[16], s_total[16];
+    __shared__ __align__(16) float s_acc[16][64];
+    const int h = blockIdx.x / n_rows, r = blockIdx.x % n_rows;
+    const int grp = threadIdx.x >> 4, cl = threadIdx.x & 15, ch = blockIdx.y * 64 + cl * 4;
+    const int64_t hr = (int64_t)h * n_rows + r, stride = (int64_t)nhkv * n_rows;
+    float top = -INFINITY;
+    for (int s = grp; s < n_splits; s += 16) top = fmaxf(top, m[s * stride + hr]);
+    if (cl == 0) s_top[grp] = top;
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < 16; ++g) top = fmaxf(top, s_top[g]);
+    if (top == -INFINITY) top = 0.f;
+    float total = 0.f;
+    f4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s = grp; s < n_splits; s += 16) {
+        const float w = expf(m[s * stride + hr] - top);
+        total += l[s * stride + hr] * w;
+        if (ch < D) acc += *reinterpret_cast<const f4_t*>(o + (s * stride + hr) * D + ch) * w;
+    }
+    if (cl == 0) s_total[grp] = total;
+    *reinterpret_cast<f4_t*>(&s_acc[grp][cl * 4]) = acc;
+    __syncthreads();
+    if (grp == 0) {
+        total = 0.f;
+        acc = f4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int g = 0; g < 16; ++g) {                    // fixed order: the result does not depend on timing
+            total += s_total[g];
+            acc += *reinterpret_cast<const f4_t*>(&s_acc[g][cl * 4]);
+        }
+        const int tok = r / G, qh = h * G + r % G;
+        const int64_t dst = (int64_t)tok * (nhkv * G) + qh;
+        if (ch < D) *reinterpret_cast<f4_t*>(out + dst * D + ch) = acc * (1.f / fmaxf(total, 1e-30f));
+        if (cl == 0 && blockIdx.y == 0) lse[dst] = total > 0.f ? top + logf(fmaxf(total, 1e-30f)) : -INFINITY;
     }
 }
 
@@ -276,6 +385,7 @@ extern "C" int qvb8_attn_fwd(const void* q, int64_t sq_r, int64_t sq_h, const vo
         if (!aligned(kmid, 16) || !aligned(kstep, 16) || !aligned(vmid, 16) || !aligned(vstep, 16))
             return host::fail(-1, "%s: the per-channel constants must be 16-byte aligned", who);
     }
+    if (n_tiles > 0 && (s_n < 0 || s_n * 32 * id_bytes > INT32_MAX)) return host::fail(-1, "%s: key stride %lld out of range", who, (long long)s_n);
     const int64_t row_blocks = (n_rows + kRows - 1) / kRows;
     if (n_splits > 65535 || row_blocks > 65535 || n_tiles > INT32_MAX || n_rows > INT32_MAX || q_pos0 > INT32_MAX / 2 || q_pos0 < INT32_MIN / 2)
         return host::fail(-1, "%s: size beyond what one launch takes", who);
@@ -289,4 +399,21 @@ extern "C" int qvb8_attn_fwd(const void* q, int64_t sq_r, int64_t sq_h, const vo
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (head_dim == 256) return id_bytes == 1 ? launch_attn<256, uint8_t>(a, n_splits, s) : launch_attn<256, uint16_t>(a, n_splits, s);
     return id_bytes == 1 ? launch_attn<128, uint8_t>(a, n_splits, s) : launch_attn<128, uint16_t>(a, n_splits, s);
+}
+
+extern "C" int qvb8_attn_combine(const float* o, const float* m, const float* l, int64_t n_splits, int64_t n_kv_heads,
+                                 int64_t n_rows, int64_t head_dim, int64_t G, float* out, float* lse, void* stream) {
+    using namespace qvb8;
+    const char* who = "qvb8_attn_combine";
+    if (n_splits < 1 || n_kv_heads < 1 || n_rows < 0 || G < 1 || head_dim < 4 || head_dim % 4 != 0)
+        return host::fail(-1, "%s: bad size (splits %lld, kv heads %lld, rows %lld, G %lld, head_dim %lld)", who, (long long)n_splits,
+                          (long long)n_kv_heads, (long long)n_rows, (long long)G, (long long)head_dim);
+    if (n_rows % G != 0) return host::fail(-1, "%s: %lld rows are not whole tokens of %lld heads", who, (long long)n_rows, (long long)G);
+    if (n_rows == 0) return 0;
+    if (!o || !m || !l || !out || !lse) return host::fail(-1, "%s: null pointer", who);
+    if (!aligned(o, 16) || !aligned(out, 16)) return host::fail(-1, "%s: o and out must be 16-byte aligned", who);
+    if (n_kv_heads * n_rows > INT32_MAX || n_splits > INT32_MAX) return host::fail(-1, "%s: size beyond what one launch takes", who);
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)(n_kv_heads * n_rows), (unsigned)((head_dim + 63) / 64)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       o, m, l, (int)n_splits, (int)n_kv_heads, (int)n_rows, (int)head_dim, (int)G, out, lse);
+    return host::check_launch(who);
 }

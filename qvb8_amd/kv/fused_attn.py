@@ -98,25 +98,28 @@ def fwd(q, ki, vi, kmid, kstep, vmid, vstep, kc, vc, ts, tl, tseg, o, m, l, q_po
 
 
 def plan_splits(n_tiles: int, hkv: int, rows: int, device) -> tuple:
-    """(tiles per split, splits): enough workgroups to fill the card (four fit a compute unit), fewer splits for long
+    """(tiles per split, splits): enough workgroups to fill the card once (three fit a compute unit), fewer splits for long
     query blocks (fused_attn.py:259-264, 271-275)."""
     n_rb = -(-rows // ROWS_PER_BLOCK)
-    want = 4 * torch.cuda.get_device_properties(device).multi_processor_count
+    want = 3 * torch.cuda.get_device_properties(device).multi_processor_count
     n_splits = max(1, min(n_tiles, want // max(1, hkv * n_rb)))
     tps = max(1, math.ceil(n_tiles / n_splits))
     return tps, max(1, math.ceil(n_tiles / tps))
 
 
-def combine_splits(o, m, l):
-    """Per-split (unnormalised o, running max m, running sum l) -> (normalised result, log-sum-exp) per kv head and row:
-    every split is weighted by exp(m - max over splits); a row no split saw a key for gives 0 and -inf
-    (fused_attn.py:302-314; one split is the same formula with weight 1)."""
-    top = m.amax(dim=0)
-    top = torch.where(torch.isinf(top), torch.zeros_like(top), top)
-    w = torch.exp(m - top)
-    total = (l * w).sum(0)
-    out = (o * w.unsqueeze(-1)).sum(0) / total.clamp_min(1e-30).unsqueeze(-1)
-    lse = torch.where(total > 0, top + torch.log(total.clamp_min(1e-30)), torch.full_like(total, float("-inf")))
+def combine_splits(o, m, l, G: int):
+    """Per-split (unnormalised o, running max m, running sum l) of `fwd` -> (out (MQ, Hq, D), lse (MQ, Hq)), one launch
+    of qvb8_attn_combine: every split is weighted by exp(m - max over splits); a row no split saw a key for gives 0
+    and -inf (fused_attn.py:302-316)."""
+    S, hkv, rows, d = o.shape
+    mq = rows // G
+    out = torch.empty(mq, hkv * G, d, dtype=torch.float32, device=o.device)
+    lse = torch.empty(mq, hkv * G, dtype=torch.float32, device=o.device)
+    lib = _lib.load()
+    with torch.cuda.device(o.device):
+        rc = lib.qvb8_attn_combine(o.data_ptr(), m.data_ptr(), l.data_ptr(), S, hkv, rows, d, int(G), out.data_ptr(), lse.data_ptr(),
+                                   torch.cuda.current_stream().cuda_stream)
+    _lib._check(rc, lib)
     return out, lse
 
 
@@ -141,7 +144,4 @@ def attend(q, lay: QVLayout, q_pos0: int, scale: float, n_splits: int | None = N
     l = torch.empty_like(m)
     fwd(q16, lay.ki, lay.vi, lay.kmin, lay.kstep, lay.vmin, lay.vstep, lay.kc.contiguous(), lay.vc.contiguous(),
         lay.t_start, lay.t_len, lay.t_seg, o, m, l, q_pos0, tps, 1.0, g)
-    out, lse = combine_splits(o, m, l)
-    out = out.reshape(hkv, mq, g, d).permute(1, 0, 2, 3).reshape(mq, hq, d)
-    lse = lse.reshape(hkv, mq, g).permute(1, 0, 2).reshape(mq, hq)
-    return out, lse
+    return combine_splits(o, m, l, g)

@@ -219,3 +219,24 @@ def test_attn_refusals_through_the_c_abi():
                 dict(kmid=dl["kmid"].data_ptr() + 4), dict(q_pos0=2 ** 31)):
         assert call(**bad) != 0, bad
         assert lib.qvb8_last_error().decode().startswith("qvb8_attn_fwd"), bad
+
+
+def test_combine_matches_the_oracle():
+    """qvb8_attn_combine against the caller's combination: random splits, rows nobody saw, a single split."""
+    rng = np.random.default_rng(8)
+    for S, hkv, MQ, G, D in ((5, 2, 3, 4, 128), (1, 1, 2, 2, 256), (300, 1, 1, 6, 256)):
+        R = MQ * G
+        o = rng.normal(0, 1, (S, hkv, R, D)).astype(np.float32)
+        m = rng.normal(0, 3, (S, hkv, R)).astype(np.float32)
+        l = rng.uniform(0.5, 30, (S, hkv, R)).astype(np.float32)
+        m[:, 0, 0] = -np.inf; l[:, 0, 0] = 0; o[:, 0, 0] = 0            # a row without a visible key
+        if S > 1:
+            m[1, 0, 1] = -np.inf; l[1, 0, 1] = 0; o[1, 0, 1] = 0        # one empty split among full ones
+        want, want_lse = A.combine(o, m, l, MQ, G)
+        got, lse = FA.combine_splits(torch.from_numpy(o).to(DEV), torch.from_numpy(m).to(DEV), torch.from_numpy(l).to(DEV), G)
+        assert got.shape == (MQ, hkv * G, D) and lse.shape == (MQ, hkv * G)
+        assert np.allclose(got.cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+        assert np.array_equal(np.isneginf(lse.cpu().numpy()), np.isneginf(want_lse))
+        fin = np.isfinite(want_lse)
+        assert np.allclose(lse.cpu().numpy()[fin], want_lse[fin], rtol=1e-6, atol=1e-5)
+        assert np.all(got.cpu().numpy()[0, 0] == 0)
