@@ -440,8 +440,10 @@ def bench_attn(args, dev):
                                    % (MQ, hkv, n, seg, len(lays), n_splits, tps),
                        "bytes_per_launch": nbytes, "us_per_layer": round(ms * 1e3 / len(lays), 2)},
             "roofline": {"bound": "hbm", "achieved": round(gbs_kernel, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs_kernel / HBM_PEAK_GBS, 4), "traffic": None,
-                         "kernel": "qvb8::attn_kernel<256, unsigned char>", "bytes_per_launch": nbytes, "launch_us": round(us, 3)},
+                         "frac": round(gbs_kernel / HBM_PEAK_GBS, 4),
+                         # FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of one launch over 32768 keys (profiles/attn_kernels_*.md)
+                         "traffic": round((2 * 33134.5 + 3120.0) * 1024) if (n, MQ) == (32768, 1) else None,
+                         "kernel": "qvb8::attn_wave_kernel<256>" if tps >= 12 else "qvb8::attn_kernel<256, unsigned char>", "bytes_per_launch": nbytes, "launch_us": round(us, 3)},
             "cpu_baseline": None}
 
 
@@ -492,7 +494,8 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="layers of distinct packs (default 32; moe 4; qvb8r 2)")
     ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead", "embed", "attn"), default="decode9b",
                     help="decode9b (default, the headline metric): 9B-shape decode step; moe: 35B-A3B-shape expert stack; "
-                         "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256)")
+                         "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256); "
+                         "lmhead / embed: the 248320 x 5120 vocabulary table; attn: decode-step attention over a banded KV cache")
     ap.add_argument("--context", type=int, default=32768, help="keys in the cache of the attn workload")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
     ap.add_argument("--model", choices=("9b", "27b"), default="9b",

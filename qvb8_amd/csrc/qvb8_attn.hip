@@ -539,28 +539,28 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_wave_kernel(const AttnAr
     }
 }
 
-// Splits -> the normalised result and the log-sum-exp.  One workgroup per (kv head, row, 64 channels): 16 groups of 16
-// threads share the splits (group g takes splits g, g + 16, ...), a thread holds four channels; the groups' maxima,
-// sums and partial results meet in LDS.  Every load of a thread is independent of the others, so the launch costs a few
-// trips to memory, not one per split.
+// Splits -> the normalised result and the log-sum-exp.  One workgroup per (kv head, row, 16 channels): 64 groups of 4
+// threads share the splits (group g takes splits g, g + 64, ...), a thread holds four channels; the groups' maxima,
+// sums and partial results meet in LDS.  A thread has a few independent loads, so the launch costs a few trips to
+// memory, not one per split.
 __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ o, const float* __restrict__ m, const float* __restrict__ l,
                                                             int n_splits, int nhkv, int n_rows, int D, int G,
                                                             float* __restrict__ out, float* __restrict__ lse) {
-    __shared__ float s_top[16], s_total[16];
-    __shared__ __align__(16) float s_acc[16][64];
+    __shared__ float s_top[64], s_total[64];
+    __shared__ __align__(16) float s_acc[64][16];
     const int h = blockIdx.x / n_rows, r = blockIdx.x % n_rows;
-    const int grp = threadIdx.x >> 4, cl = threadIdx.x & 15, ch = blockIdx.y * 64 + cl * 4;
+    const int grp = threadIdx.x >> 2, cl = threadIdx.x & 3, ch = blockIdx.y * 16 + cl * 4;
     const int64_t hr = (int64_t)h * n_rows + r, stride = (int64_t)nhkv * n_rows;
     float top = -INFINITY;
-    for (int s = grp; s < n_splits; s += 16) top = fmaxf(top, m[s * stride + hr]);
+    for (int s = grp; s < n_splits; s += 64) top = fmaxf(top, m[s * stride + hr]);
     if (cl == 0) s_top[grp] = top;
     __syncthreads();
 #pragma unroll
-    for (int g = 0; g < 16; ++g) top = fmaxf(top, s_top[g]);
+    for (int g = 0; g < 64; ++g) top = fmaxf(top, s_top[g]);
     if (top == -INFINITY) top = 0.f;
     float total = 0.f;
     f4_t acc = {0.f, 0.f, 0.f, 0.f};
-    for (int s = grp; s < n_splits; s += 16) {
+    for (int s = grp; s < n_splits; s += 64) {
         const float w = expf(m[s * stride + hr] - top);
         total += l[s * stride + hr] * w;
         if (ch < D) acc += *reinterpret_cast<const f4_t*>(o + (s * stride + hr) * D + ch) * w;
@@ -571,8 +571,8 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
     if (grp == 0) {
         total = 0.f;
         acc = f4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int g = 0; g < 16; ++g) {                    // fixed order: the result does not depend on timing
+#pragma unroll 8
+        for (int g = 0; g < 64; ++g) {                    // fixed order: the result does not depend on timing
             total += s_total[g];
             acc += *reinterpret_cast<const f4_t*>(&s_acc[g][cl * 4]);
         }
@@ -659,7 +659,7 @@ extern "C" int qvb8_attn_combine(const float* o, const float* m, const float* l,
     if (!o || !m || !l || !out || !lse) return host::fail(-1, "%s: null pointer", who);
     if (!aligned(o, 16) || !aligned(out, 16)) return host::fail(-1, "%s: o and out must be 16-byte aligned", who);
     if (n_kv_heads * n_rows > INT32_MAX || n_splits > INT32_MAX) return host::fail(-1, "%s: size beyond what one launch takes", who);
-    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)(n_kv_heads * n_rows), (unsigned)((head_dim + 63) / 64)), dim3(256), 0, static_cast<hipStream_t>(stream),
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)(n_kv_heads * n_rows), (unsigned)((head_dim + 15) / 16)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        o, m, l, (int)n_splits, (int)n_kv_heads, (int)n_rows, (int)head_dim, (int)G, out, lse);
     return host::check_launch(who);
 }

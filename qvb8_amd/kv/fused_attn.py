@@ -98,10 +98,11 @@ def fwd(q, ki, vi, kmid, kstep, vmid, vstep, kc, vc, ts, tl, tseg, o, m, l, q_po
 
 
 def plan_splits(n_tiles: int, hkv: int, rows: int, device) -> tuple:
-    """(tiles per split, splits): enough workgroups to fill the card once (three fit a compute unit), fewer splits for long
-    query blocks (fused_attn.py:259-264, 271-275)."""
+    """(tiles per split, splits): as many workgroups as the card holds at once -- two per compute unit (measured over
+    32768 and 131072 keys: 512 workgroups 27.9 / 82.6 us, 768 33.9 / 88.9, 1024 30.0 / 85.5, 256 35.4 / 105) -- and
+    fewer splits for long query blocks (fused_attn.py:259-264, 271-275)."""
     n_rb = -(-rows // ROWS_PER_BLOCK)
-    want = 3 * torch.cuda.get_device_properties(device).multi_processor_count
+    want = 2 * torch.cuda.get_device_properties(device).multi_processor_count
     n_splits = max(1, min(n_tiles, want // max(1, hkv * n_rb)))
     tps = max(1, math.ceil(n_tiles / n_splits))
     return tps, max(1, math.ceil(n_tiles / tps))

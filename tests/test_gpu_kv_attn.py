@@ -75,11 +75,15 @@ CASES = [
     (128, 2, 3, 12, [100], 50, 5, 2),                 # 36 rows: three row blocks, causal cut inside the tiles
     (128, 1, 1, 3, [64], -2, 6, 1),                   # the first queries see no key at all
     (256, 2, 2, 1, [1], 0, 6, 1),
+    (256, 1, 6, 1, [500, 17], 516, 6, 7),             # splits of 7 tiles: both register sets and the odd last piece in use
+    (128, 2, 4, 2, [333], 332, 7, 5),
 ]
 
 
+@pytest.mark.parametrize("waves", ["0", "1"])          # both kernels for byte ids: tile shared by the waves / a stream per wave
 @pytest.mark.parametrize("D,Hkv,G,MQ,seg_len,q_pos0,bits,tps", CASES)
-def test_fwd_matches_the_oracle(D, Hkv, G, MQ, seg_len, q_pos0, bits, tps):
+def test_fwd_matches_the_oracle(D, Hkv, G, MQ, seg_len, q_pos0, bits, tps, waves, monkeypatch):
+    monkeypatch.setenv("QVB8_ATTN_WAVES", waves)
     lay = make_layout(D + MQ + G, seg_len, Hkv, D, bits=bits)
     rng = np.random.default_rng(11)
     q = (rng.normal(0, 1, (MQ, Hkv * G, D)) * D ** -0.5).astype(np.float16)
