@@ -1,6 +1,6 @@
 """GPU checks at the full sizes of the benchmark configurations, through size-independent properties (the CPU oracle would
-take minutes there): restore -> certificate, fused product == dense restore + fp32 matmul, linearity, fusion and QVB8R
-restore == QVB8 restore of the same ids."""
+take minutes there): restore -> certificate, fused product == dense restore + fp32 matmul, linearity, fusion, QVB8R
+restore == QVB8 restore of the same ids, and attention over a long banded cache == dense attention, however it is split."""
 import numpy as np
 import pytest
 import torch
@@ -77,3 +77,48 @@ def test_qvb8r_restore_equals_qvb8_restore_at_27b_shape():
     ref = x.float().double() @ w32.t()
     tol = (1e-3 + 2.0 ** -8) * ref.abs() + 1e-3 * w32.norm(dim=1)[None, :] * x.float().double().norm(dim=1)[:, None] / np.sqrt(P)
     assert bool(((y - ref).abs() <= tol).all())
+
+
+@pytest.mark.parametrize("n,MQ", [(32768, 1), (32768, 3), (131072, 1)])
+def test_attention_over_a_long_banded_cache(n, MQ):
+    """The benchmark's cache shape (4 kv heads x 256 channels, 24 query heads, 6-bit ids, segments of 4096 keys): the
+    result does not depend on how the tiles are split (one split, the planner's, twice as many: within the fp16 rounding
+    of the probabilities, 1e-3 * max|v|), equals fp32 attention over the decoded cache (4e-3 * max|v|: that reference
+    keeps bf16-rounded K / V where the kernel restores fp16), and a query placed inside the context ignores every
+    later key."""
+    from qvb8_amd.kv import codec as KC, fused_attn as FA
+    hkv, G, D, seg = 4, 6, 256, 4096
+    g = torch.Generator(device=DEV).manual_seed(n + MQ)
+    segs_k, segs_v, seg_len = [], [], []
+    for a in range(0, n, seg):
+        k = (torch.randn(hkv, seg, D, device=DEV, generator=g) * (0.5 + 2 * torch.rand(hkv, 1, D, device=DEV, generator=g))).to(torch.bfloat16)
+        v = torch.randn(hkv, seg, D, device=DEV, generator=g).to(torch.bfloat16)
+        segs_k.append(KC.band_kv_heads(k, torch.bfloat16, 6, certify=False))
+        segs_v.append(KC.band_kv_heads(v, torch.bfloat16, 6, certify=False))
+        seg_len.append(seg)
+    lay = FA.layout_from_segments(segs_k, segs_v, seg_len, DEV)
+    q = torch.randn(MQ, hkv * G, D, device=DEV, generator=g).to(torch.bfloat16)
+    scale = D ** -0.5
+    vmax = float((lay.vmin.abs() + lay.vstep * 32).max())
+    tps, planned = FA.plan_splits(lay.n_tiles, hkv, MQ * G, DEV)
+    outs = [FA.attend(q, lay, n - MQ, scale, n_splits=s) for s in (1, planned, 2 * planned)]
+    for out, lse in outs[1:]:
+        assert float((out - outs[0][0]).abs().max()) <= 1e-3 * vmax
+        assert float((lse - outs[0][1]).abs().max()) <= 2e-3
+    # dense fp32 attention over the decoded cache, one kv head at a time (the scores of all heads would not fit nicely)
+    q16 = (q.float() * scale).clamp(-65504, 65504).half().float().reshape(MQ, hkv, G, D)
+    mask = torch.arange(n, device=DEV)[None, :] <= (n - MQ + torch.arange(MQ, device=DEV))[:, None]
+    for h in range(hkv):
+        K = torch.cat([s[h].decode_all_torch(DEV) for s in segs_k])
+        V = torch.cat([s[h].decode_all_torch(DEV) for s in segs_v])
+        s = torch.einsum("mgd,nd->mgn", q16[:, h], K).masked_fill(~mask[:, None, :], float("-inf"))
+        ref = torch.einsum("mgn,nd->mgd", torch.softmax(s, -1), V)
+        got = outs[1][0].reshape(MQ, hkv, G, D)[:, h]
+        assert float((got - ref).abs().max()) <= 4e-3 * vmax
+        assert float((outs[1][1].reshape(MQ, hkv, G)[:, h] - torch.logsumexp(s, -1)).abs().max()) <= 2e-2
+    # a query in the middle of the context: the same as attention over the cache cut off behind it
+    cut = n // 2 + 77
+    short = FA.layout_from_segments(segs_k[: cut // seg + 1], segs_v[: cut // seg + 1], seg_len[: cut // seg + 1], DEV)
+    o_mid, l_mid = FA.attend(q[:1], lay, cut, scale)
+    o_cut, l_cut = FA.attend(q[:1], short, cut, scale)
+    assert float((o_mid - o_cut).abs().max()) <= 1e-3 * vmax and float((l_mid - l_cut).abs().max()) <= 2e-3
