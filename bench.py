@@ -443,7 +443,7 @@ def bench_attn(args, dev):
                          "frac": round(gbs_kernel / HBM_PEAK_GBS, 4),
                          # FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of one launch over 32768 keys (profiles/attn_kernels_*.md)
                          "traffic": round((2 * 33134.5 + 3120.0) * 1024) if (n, MQ) == (32768, 1) else None,
-                         "kernel": "qvb8::attn_wave_kernel<256>" if tps >= 12 else "qvb8::attn_kernel<256, unsigned char>", "bytes_per_launch": nbytes, "launch_us": round(us, 3)},
+                         "kernel": "qvb8::attn_kernel<256, unsigned char>", "bytes_per_launch": nbytes, "launch_us": round(us, 3)},
             "cpu_baseline": None}
 
 

@@ -75,8 +75,10 @@ __device__ __forceinline__ void tile_entry(const int32_t* ts, const int32_t* tl,
     r.start = start; r.nlen = nlen; r.seg = seg;
 }
 
+// Three workgroups per compute unit (two with 16-bit ids and 256 channels, whose two register sets are twice as large):
+// the third one is what hides a workgroup's barriers and dependent chains -- 74.9 against 82.3 us over 131072 keys.
 template <int D, typename T>
-__global__ __launch_bounds__(kAttnThreads, 2) void attn_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3) void attn_kernel(const AttnArgs a) {
     constexpr int CG = D / 4;                  // channel groups (four channels each) of a key
     constexpr int KSTEP = kAttnThreads / CG;   // key groups (four keys each) that one pass of the workgroup covers
     constexpr int UNITS = D / 128;             // (4 keys x 4 channels) units per thread and tile
@@ -120,11 +122,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_kernel(const AttnArgs a)
     // position (tiles ascend: so do all after it) -- re-reads key 0 of the head (one cached line); neither is used.
     // A request's address is the tile's first key (scalar) plus the thread's key offset, fixed for the whole kernel
     // and clamped to the tile's last key (host-checked: 32 keys' stride fits 31 bits).
-    uint32_t key_off[UNITS][4];
-#pragma unroll
-    for (int u = 0; u < UNITS; ++u)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) key_off[u][j] = (uint32_t)(4 * (kgp0 + KSTEP * u) + j) * (uint32_t)a.s_n * (uint32_t)sizeof(T);
+    const uint32_t key_stride = (uint32_t)a.s_n * (uint32_t)sizeof(T);      // bytes from one key to the next
+    const uint32_t key_off0 = (uint32_t)(4 * kgp0) * key_stride;            // the thread's first key; its others lie a scalar further
     const unsigned char* kbytes = reinterpret_cast<const unsigned char*>(ki);
     const unsigned char* vbytes = reinterpret_cast<const unsigned char*>(vi);
     auto fetch = [&](int t, U (&rk)[UNITS][4], U (&rv)[UNITS][4], TileRef& ref) {
@@ -139,7 +138,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_kernel(const AttnArgs a)
         for (int u = 0; u < UNITS; ++u)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const uint32_t off = min(key_off[u][j], last_off);
+                const uint32_t off = min(key_off0 + (uint32_t)(4 * KSTEP * u + j) * key_stride, last_off);
                 rk[u][j] = *reinterpret_cast<const U*>(kb + off);
                 rv[u][j] = *reinterpret_cast<const U*>(vb + off);
             }
@@ -154,7 +153,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_kernel(const AttnArgs a)
     float km[4] = {0.f, 0.f, 0.f, 0.f}, ks_[4] = {0.f, 0.f, 0.f, 0.f}, vm[4] = {0.f, 0.f, 0.f, 0.f}, vs_[4] = {0.f, 0.f, 0.f, 0.f}, kc = 0.f, vc = 0.f;
     // One tile: restore the ids of register set (rk, rv) into LDS, refill the set with tile t + 2, S, softmax, O.
     auto tile = [&](int t, U (&rk)[UNITS][4], U (&rv)[UNITS][4], TileRef& ref) {
-        const int start = ref.start, nlen = ref.nlen, seg = ref.seg;
+        const int start = ref.start, nlen = ref.ok ? ref.nlen : 0, seg = ref.seg;      // a tile that is not wanted: no key counts
         if (seg != cur_seg) {
             // A new segment (every few thousand keys): its constants for this thread's four channels.  The wait stands
             // INSIDE the branch: the requests of the next tiles' ids are older than these, and a wait placed where the
@@ -170,32 +169,38 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_kernel(const AttnArgs a)
             __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0)
             cur_seg = seg;
         }
-        auto restore = [&](auto full) {
+        // Keys past the tile's length hold a copy of its last key: their scores are replaced by -inf before any use, so K
+        // needs no blanking; their V must be zero (0 * inf would poison the sums), done on the packed halves.
+        const bool whole = nlen == kKeys;
 #pragma unroll
-            for (int u = 0; u < UNITS; ++u) {
-                const int kgp = kgp0 + KSTEP * u;
-                h4_t vcell[4];
+        for (int u = 0; u < UNITS; ++u) {
+            const int kgp = kgp0 + KSTEP * u;
+            h4_t vcell[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int key = 4 * kgp + j;
-                    const bool live = decltype(full)::value || key < nlen;
-                    h4_t kv;
+            for (int j = 0; j < 4; ++j) {
+                const int key = 4 * kgp + j;
+                h4_t kv;
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const float kf_ = __builtin_fmaf(ks_[c], QD::id(rk[u][j], c) - kc, km[c]);
-                        const float vf = __builtin_fmaf(vs_[c], QD::id(rv[u][j], c) - vc, vm[c]);
-                        kv[c] = live ? (_Float16)kf_ : (_Float16)0.f;
-                        vcell[c][j] = live ? (_Float16)vf : (_Float16)0.f;
-                    }
-                    *reinterpret_cast<h4_t*>(Ks + key * KROW + 4 * cg) = kv;
+                for (int c = 0; c < 4; ++c) {
+                    kv[c] = (_Float16)__builtin_fmaf(ks_[c], QD::id(rk[u][j], c) - kc, km[c]);
+                    vcell[c][j] = (_Float16)__builtin_fmaf(vs_[c], QD::id(rv[u][j], c) - vc, vm[c]);
                 }
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    *reinterpret_cast<h4_t*>(Vt + (4 * cg + c) * kKeys + 4 * (kgp ^ (cg & 7))) = vcell[c];
+                *reinterpret_cast<h4_t*>(Ks + key * KROW + 4 * cg) = kv;
             }
-        };
-        if (nlen == kKeys) restore(std::true_type{});        // a whole tile: no key to blank out
-        else restore(std::false_type{});
+            if (!whole) {
+                const uint32_t m0 = (4 * kgp + 0 < nlen ? 0x0000FFFFu : 0u) | (4 * kgp + 1 < nlen ? 0xFFFF0000u : 0u);
+                const uint32_t m1 = (4 * kgp + 2 < nlen ? 0x0000FFFFu : 0u) | (4 * kgp + 3 < nlen ? 0xFFFF0000u : 0u);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    uint2 w = *reinterpret_cast<uint2*>(&vcell[c]);
+                    w.x &= m0; w.y &= m1;
+                    vcell[c] = *reinterpret_cast<h4_t*>(&w);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                *reinterpret_cast<h4_t*>(Vt + (4 * cg + c) * kKeys + 4 * (kgp ^ (cg & 7))) = vcell[c];
+        }
         __syncthreads();
         fetch(t + 2, rk, rv, ref);
 
@@ -278,264 +283,33 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_kernel(const AttnArgs a)
         __builtin_amdgcn_sched_barrier(0);                 // set 0 is the older one, as in every later round of the loop
         fetch(t0 + 1, rk1, rv1, ref1);
         __builtin_amdgcn_sched_barrier(0);
-        // The loop has one way out, at its head, and takes tiles in pairs; a last odd tile follows it.  (A way out of the
-        // middle is turned into a path through the loop's end back to its head: on that path set 0 would be the younger
-        // one, and the compiler would make every round wait for both sets.)
-        int t = t0;
-        for (; ref0.ok && ref1.ok; t += 2) {
+        // The loop has one way out, at its head, and takes tiles in pairs; when the last pair has no second tile, that
+        // one is run as an empty tile (no key counts: nothing changes).  A way out of the middle would be turned into a
+        // path through the loop's end back to its head, on which set 0 is the younger one, and the compiler would make
+        // every round wait for both sets; a copy of the tile's code behind the loop costs registers that end in scratch.
+        for (int t = t0; ref0.ok; t += 2) {
             tile(t, rk0, rv0, ref0);
             tile(t + 1, rk1, rv1, ref1);
         }
-        if (ref0.ok) tile(t, rk0, rv0, ref0);
     }
 
+    // Where the results go is worked out only now, from a thread index the compiler cannot connect with the one above:
+    // otherwise it computes the addresses before the loop and, short of registers, parks them in scratch memory (measured:
+    // 5.6 MB written and read back per launch).
+    int tid_e = threadIdx.x;
+    asm volatile("" : "+v"(tid_e));
+    const int lane_e = tid_e & 63, wave_e = tid_e >> 6, n16_e = lane_e & 15, kg_e = lane_e >> 4;
     const int64_t base = ((int64_t)sp * a.nhkv + h) * a.n_rows;
 #pragma unroll
     for (int f = 0; f < NF; ++f)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int r = row0 + 4 * kg + e;
-            if (r < a.n_rows) a.o[(base + r) * D + wave * (D / 4) + 16 * f + n16] = acc[f][e];
+            const int r = row0 + 4 * kg_e + e;
+            if (r < a.n_rows) a.o[(base + r) * D + wave_e * (D / 4) + 16 * f + n16_e] = acc[f][e];
         }
-    if (wave == 0 && kg == 0 && row_ok) {
-        a.m[base + row] = m_run;
-        a.l[base + row] = l_run;
-    }
-}
-
-// ---- byte ids: every wave streams its own keys ------------------------------------------------------------------
-// The same arithmetic with no barrier in the loop: a workgroup's four waves take the split's keys in pieces of 16
-// (wave w the pieces w, w + 4, ... -- a 32-key tile is two pieces), each with its own LDS area, its own softmax state
-// and an accumulator over all channels; the four states are merged once, at the end, the way the caller merges splits.
-//   * S^T = K Q^T instead of Q K^T (K from LDS as the A operand, the wave's Q registers as B): the result has row
-//     n16's scores for keys 4 kg .. 4 kg + 3 in lane (n16, kg) -- already the A-operand layout of P V, so neither S nor
-//     P goes through LDS, and the softmax of a key is computed once (lanes hold 4 keys, not 8 on each of 4 waves);
-//   * a lane reads ids of whole key rows (4 channels per lane): with 256 channels one key per request, with 128 two
-//     (the lane's keys are then every second one, and the tile is kept in LDS in the order even keys, odd keys -- P and
-//     V only have to agree on the order);
-//   * V lies in LDS as [4 positions][channel] cells of 8 bytes, a thread's four channels side by side: its writes are
-//     32 contiguous bytes and a fragment's reads 128.
-template <int D>
-__global__ __launch_bounds__(kAttnThreads, 2) void attn_wave_kernel(const AttnArgs a) {
-    constexpr int CG = D / 4;                  // channel groups (four channels each) of a key
-    constexpr int KPL = 64 / CG;               // keys one request of the wave covers (1 or 2)
-    constexpr int NLD = 16 / KPL;              // requests per operand and piece
-    constexpr int KROW = D + 8;                // halfs per key in LDS
-    constexpr int NF = D / 16;                 // 16-channel output fragments
-    constexpr int NKS = D / 16;                // 16-channel steps of S
-    constexpr int kWaveLds = 16 * KROW * 2 + D * 16 * 2;          // bytes: K [16][KROW] + V [4][D][4]
-    constexpr int kArea = kWaveLds > (16 * D + 32) * 4 ? kWaveLds : (16 * D + 32) * 4;
-    __shared__ __align__(16) unsigned char lds[4 * kArea + kRows * KROW * 2];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n16 = lane & 15, kg = lane >> 4;
-    const int h = blockIdx.x, sp = blockIdx.y, row0 = blockIdx.z * kRows;
-    const int cg = lane % CG, par = lane / CG;                  // this lane's channels; which of the request's keys
-    _Float16* Kw = reinterpret_cast<_Float16*>(lds + wave * kArea);
-    _Float16* Vw = Kw + 16 * KROW;
-    // position of the lane's i-th key in the LDS order, and the key at a position
-    auto pos_of = [&](int i) { return KPL == 1 ? i : par * 8 + i; };
-    auto key_at = [&](int pos) { return KPL == 1 ? pos : 2 * (pos & 7) + (pos >> 3); };
-
-    const int row = row0 + n16;
-    const bool row_ok = row < a.n_rows;
-    const int qpos = a.q_pos0 + (row_ok ? row / a.G : 0);
-    // Q of the block's 16 rows in LDS, shared by the four waves (as registers they would not leave room for two sets of
-    // ids in flight): row r at r * KROW halfs, zero for rows past n_rows
-    _Float16* Qs = reinterpret_cast<_Float16*>(lds + 4 * kArea);
-    for (int idx = tid; idx < kRows * (D / 4); idx += kAttnThreads) {
-        const int r = idx / (D / 4), c4 = (idx % (D / 4)) * 4, rr = row0 + r;
-        h4_t v = {0, 0, 0, 0};
-        if (rr < a.n_rows) v = *reinterpret_cast<const h4_t*>(a.q + (int64_t)(rr / a.G) * a.sq_r + (int64_t)(h * a.G + rr % a.G) * a.sq_h + c4);
-        *reinterpret_cast<h4_t*>(Qs + r * KROW + c4) = v;
-    }
-    __syncthreads();
-    const int qmin = a.q_pos0 + row0 / a.G;
-    const int qmax = a.q_pos0 + (min(row0 + kRows, a.n_rows) - 1) / a.G;
-    const unsigned char* kbytes = reinterpret_cast<const unsigned char*>(a.ki) + (int64_t)h * a.s_h + 4 * cg;
-    const unsigned char* vbytes = reinterpret_cast<const unsigned char*>(a.vi) + (int64_t)h * a.s_h + 4 * cg;
-    const int t0 = (int)min((int64_t)sp * a.tps, (int64_t)a.n_tiles), t1 = (int)min((int64_t)t0 + a.tps, (int64_t)a.n_tiles);
-
-    uint32_t key_off[NLD];                     // byte offset of the lane's i-th key from the piece's first key
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) key_off[i] = (uint32_t)(KPL * i + par) * (uint32_t)a.s_n;
-
-    struct Piece { int start, nlen, seg, half; bool ok; };
-    // ids of piece u (tile t0 + u / 2, keys 16 (u % 2) .. + 15 of it): always 2 NLD requests, none under a branch; keys
-    // past the tile's length re-read its last key, a piece that is not wanted re-reads key 0 of the head
-    auto fetch = [&](int u, uint32_t (&rk)[NLD], uint32_t (&rv)[NLD], Piece& pc) {
-        const int t = t0 + (u >> 1);
-        TileRef ref;
-        tile_entry(a.ts, a.tl, a.tseg, min(t, t1 - 1), ref);
-        pc.start = ref.start; pc.nlen = ref.nlen; pc.seg = ref.seg; pc.half = u & 1;
-        pc.ok = __builtin_amdgcn_readfirstlane((int)(t < t1 && ref.start <= qmax)) != 0;
-        const int first = pc.ok ? ref.start + 16 * pc.half : 0;
-        const int last = pc.ok ? max(ref.nlen - 1 - 16 * pc.half, 0) : 0;          // last key of the piece that exists (piece-relative)
-        const int64_t piece_byte = (int64_t)first * a.s_n;
-        const uint32_t last_off = (uint32_t)last * (uint32_t)a.s_n;
-        const unsigned char* kb = kbytes + piece_byte;
-        const unsigned char* vb = vbytes + piece_byte;
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-            const uint32_t off = min(key_off[i], last_off);
-            rk[i] = *reinterpret_cast<const uint32_t*>(kb + off);
-            rv[i] = *reinterpret_cast<const uint32_t*>(vb + off);
-        }
-    };
-
-    float m_run = -INFINITY, l_run = 0.f;
-    f4_t acc[NF];
-#pragma unroll
-    for (int f = 0; f < NF; ++f) acc[f] = f4_t{0.f, 0.f, 0.f, 0.f};
-    int cur_seg = -1;
-    float km[4] = {0.f, 0.f, 0.f, 0.f}, ks_[4] = {0.f, 0.f, 0.f, 0.f}, vm[4] = {0.f, 0.f, 0.f, 0.f}, vs_[4] = {0.f, 0.f, 0.f, 0.f}, kc = 0.f, vc = 0.f;
-
-    auto piece = [&](int u, uint32_t (&rk)[NLD], uint32_t (&rv)[NLD], Piece& pc) {
-        const int start = pc.start + 16 * pc.half, nlen = pc.nlen - 16 * pc.half, seg = pc.seg;     // piece-relative
-        if (seg != cur_seg) {
-            // a new segment's constants; the wait stands inside the branch (the id requests in flight are older)
-            const int64_t pb = ((int64_t)seg * a.nhkv + h) * D + 4 * cg;
-            const float4 kmid = *reinterpret_cast<const float4*>(a.kmid + pb), kstep = *reinterpret_cast<const float4*>(a.kstep + pb);
-            const float4 vmid = *reinterpret_cast<const float4*>(a.vmid + pb), vstep = *reinterpret_cast<const float4*>(a.vstep + pb);
-            kc = a.kc[seg * a.nhkv + h]; vc = a.vc[seg * a.nhkv + h];
-            km[0] = kmid.x; km[1] = kmid.y; km[2] = kmid.z; km[3] = kmid.w;
-            ks_[0] = kstep.x; ks_[1] = kstep.y; ks_[2] = kstep.z; ks_[3] = kstep.w;
-            vm[0] = vmid.x; vm[1] = vmid.y; vm[2] = vmid.z; vm[3] = vmid.w;
-            vs_[0] = vstep.x; vs_[1] = vstep.y; vs_[2] = vstep.z; vs_[3] = vstep.w;
-            __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0)
-            cur_seg = seg;
-        }
-        // ---- restore: K rows in position order, V cells of four positions ----
-#pragma unroll
-        for (int q = 0; q < NLD / 4; ++q) {
-            h4_t vcell[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int i = 4 * q + j;
-                const bool live = KPL * i + par < nlen;
-                h4_t kv;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const float kf_ = __builtin_fmaf(ks_[c], (float)((rk[i] >> (8 * c)) & 0xFFu) - kc, km[c]);
-                    const float vf = __builtin_fmaf(vs_[c], (float)((rv[i] >> (8 * c)) & 0xFFu) - vc, vm[c]);
-                    kv[c] = live ? (_Float16)kf_ : (_Float16)0.f;
-                    vcell[c][j] = live ? (_Float16)vf : (_Float16)0.f;
-                }
-                *reinterpret_cast<h4_t*>(Kw + pos_of(i) * KROW + 4 * cg) = kv;
-            }
-            const int cell = pos_of(4 * q) >> 2;                // positions 4 cell .. 4 cell + 3
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                *reinterpret_cast<h4_t*>(Vw + (cell * D + 4 * cg + c) * 4) = vcell[c];
-        }
-        fetch(u + 8, rk, rv, pc);                                // the piece after next of this wave
-
-        // ---- S^T = K Q^T: lane (row n16, kg) gets the scores of positions 4 kg .. 4 kg + 3 ----
-        f4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-        {
-            const _Float16* kp = Kw + n16 * KROW + 4 * kg;
-            const _Float16* qp = Qs + n16 * KROW + 4 * kg;
-#pragma unroll
-            for (int ks = 0; ks < NKS; ks += 2) {
-                s0 = __builtin_amdgcn_mfma_f32_16x16x16f16(*reinterpret_cast<const h4_t*>(kp + 16 * ks), *reinterpret_cast<const h4_t*>(qp + 16 * ks), s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x16f16(*reinterpret_cast<const h4_t*>(kp + 16 * ks + 16), *reinterpret_cast<const h4_t*>(qp + 16 * ks + 16), s1, 0, 0, 0);
-            }
-        }
-        const f4_t s4 = s0 + s1;
-        // ---- softmax of row n16 over the piece ----
-        h4_t pa;
-        float alpha;
-        const bool all_seen = nlen >= 16 && start + 15 <= qmin;
-        {
-            float sv[4], mx = -INFINITY;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int key = key_at(4 * kg + e);
-                const bool ok = all_seen || (row_ok && key < nlen && start + key <= qpos);
-                sv[e] = ok ? s4[e] * a.scale : -INFINITY;
-                mx = fmaxf(mx, sv[e]);
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run, mx);
-            const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-            float sum = 0.f;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const _Float16 p = (_Float16)(sv[e] == -INFINITY ? 0.f : __expf(sv[e] - m_safe));
-                pa[e] = p;
-                sum += (float)p;
-            }
-            sum += __shfl_xor(sum, 16);
-            sum += __shfl_xor(sum, 32);
-            alpha = m_run == -INFINITY ? 0.f : (m_new == m_run ? 1.f : __expf(m_run - m_safe));
-            l_run = l_run * alpha + sum;
-            m_run = m_new;
-        }
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
-            float ae[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) ae[e] = __shfl(alpha, 4 * kg + e);
-#pragma unroll
-            for (int f = 0; f < NF; ++f)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[f][e] *= ae[e];
-        }
-        // ---- O += P V: fragment f = channels 16 f .. 16 f + 15 ----
-#pragma unroll
-        for (int f = 0; f < NF; ++f) {
-            const h4_t b = *reinterpret_cast<const h4_t*>(Vw + (kg * D + 16 * f + n16) * 4);
-            acc[f] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa, b, acc[f], 0, 0, 0);
-        }
-    };
-
-    if (t0 < t1) {
-        uint32_t rk0[NLD], rv0[NLD], rk1[NLD], rv1[NLD];
-        Piece pc0, pc1;
-        fetch(wave, rk0, rv0, pc0);
-        __builtin_amdgcn_sched_barrier(0);                 // set 0 is the older one, as in every later round of the loop
-        fetch(wave + 4, rk1, rv1, pc1);
-        __builtin_amdgcn_sched_barrier(0);
-        int u = wave;
-        for (; pc0.ok && pc1.ok; u += 8) {                 // one way out, at the head; a last odd piece follows
-            piece(u, rk0, rv0, pc0);
-            piece(u + 4, rk1, rv1, pc1);
-        }
-        if (pc0.ok) piece(u, rk0, rv0, pc0);
-    }
-
-    // ---- merge the four waves' states (each in its own LDS area: [16][D] results, then m, then l) ----
-    {
-        float* area = reinterpret_cast<float*>(lds + wave * kArea);
-#pragma unroll
-        for (int f = 0; f < NF; ++f)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) area[(4 * kg + e) * D + 16 * f + n16] = acc[f][e];
-        if (kg == 0) { area[16 * D + n16] = m_run; area[16 * D + 16 + n16] = l_run; }
-    }
-    __syncthreads();
-    {
-        const int64_t base = ((int64_t)sp * a.nhkv + h) * a.n_rows;
-        auto area_of = [&](int w) { return reinterpret_cast<const float*>(lds + w * kArea); };
-        for (int idx = tid; idx < 16 * D; idx += kAttnThreads) {
-            const int r = idx / D, ch = idx % D;
-            float top = -INFINITY;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) top = fmaxf(top, area_of(w)[16 * D + r]);
-            const float safe = top == -INFINITY ? 0.f : top;
-            float o = 0.f, l = 0.f;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const float mw = area_of(w)[16 * D + r];
-                const float wgt = mw == -INFINITY ? 0.f : (mw == top ? 1.f : __expf(mw - safe));
-                o += area_of(w)[r * D + ch] * wgt;
-                l += area_of(w)[16 * D + 16 + r] * wgt;
-            }
-            if (row0 + r < a.n_rows) {
-                a.o[(base + row0 + r) * D + ch] = o;
-                if (ch == 0) { a.m[base + row0 + r] = top; a.l[base + row0 + r] = l; }
-            }
-        }
+    if (wave_e == 0 && kg_e == 0 && row0 + n16_e < a.n_rows) {
+        a.m[base + row0 + n16_e] = m_run;
+        a.l[base + row0 + n16_e] = l_run;
     }
 }
 
@@ -586,16 +360,6 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
 template <int D, typename T>
 int launch_attn(const AttnArgs& a, int64_t n_splits, hipStream_t s) {
     const dim3 grid((unsigned)a.nhkv, (unsigned)n_splits, (unsigned)((a.n_rows + kRows - 1) / kRows));
-    if constexpr (sizeof(T) == 1) {
-        // Splits of a dozen tiles and more go to the kernel whose waves stream on their own (measured: 94.7 against
-        // 103.3 us over 131072 keys); shorter ones to the kernel that shares a tile among the four waves, whose start
-        // and end are cheaper (34.2 against 39.3 us over 32768 keys in splits of 6 tiles).  QVB8_ATTN_WAVES=0 / 1 forces one.
-        const int pick = host::env_int("QVB8_ATTN_WAVES", -1);
-        if (pick > 0 || (pick < 0 && a.tps >= 12)) {
-            hipLaunchKernelGGL((attn_wave_kernel<D>), grid, dim3(kAttnThreads), 0, s, a);
-            return host::check_launch("qvb8_attn_fwd");
-        }
-    }
     hipLaunchKernelGGL((attn_kernel<D, T>), grid, dim3(kAttnThreads), 0, s, a);
     return host::check_launch("qvb8_attn_fwd");
 }

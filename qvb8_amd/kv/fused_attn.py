@@ -8,6 +8,7 @@ and combines the splits.  There is no other backend: without the HIP library it 
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 
@@ -97,12 +98,14 @@ def fwd(q, ki, vi, kmid, kstep, vmid, vstep, kc, vc, ts, tl, tseg, o, m, l, q_po
     _lib._check(rc, lib)
 
 
-def plan_splits(n_tiles: int, hkv: int, rows: int, device) -> tuple:
-    """(tiles per split, splits): as many workgroups as the card holds at once -- two per compute unit (measured over
-    32768 and 131072 keys: 512 workgroups 27.9 / 82.6 us, 768 33.9 / 88.9, 1024 30.0 / 85.5, 256 35.4 / 105) -- and
-    fewer splits for long query blocks (fused_attn.py:259-264, 271-275)."""
+def plan_splits(n_tiles: int, hkv: int, rows: int, device, per_cu: int = 3) -> tuple:
+    """(tiles per split, splits): as many workgroups as the card holds at once -- `per_cu` per compute unit: three, or
+    two for 16-bit ids with 256 channels (the kernel's registers) -- and fewer splits for long query blocks
+    (fused_attn.py:259-264, 271-275).  Measured over 32768 / 131072 keys with three resident workgroups: 768 workgroups
+    27.2 / 74.9 us, 512 27.7 / 86.1, 1024 28.5 / 81.8, 1536 29.5 / 76.5."""
     n_rb = -(-rows // ROWS_PER_BLOCK)
-    want = 2 * torch.cuda.get_device_properties(device).multi_processor_count
+    per_cu = int(os.environ.get("QVB8_ATTN_WG_PER_CU", per_cu))          # a knob for measurements
+    want = per_cu * torch.cuda.get_device_properties(device).multi_processor_count
     n_splits = max(1, min(n_tiles, want // max(1, hkv * n_rb)))
     tps = max(1, math.ceil(n_tiles / n_splits))
     return tps, max(1, math.ceil(n_tiles / tps))
@@ -133,7 +136,7 @@ def attend(q, lay: QVLayout, q_pos0: int, scale: float, n_splits: int | None = N
     g = hq // hkv
     rows = mq * g
     if n_splits is None:
-        tps, n_splits = plan_splits(lay.n_tiles, hkv, rows, q.device)
+        tps, n_splits = plan_splits(lay.n_tiles, hkv, rows, q.device, 2 if (lay.ki.dtype == torch.int16 and d == 256) else 3)
     else:
         tps = max(1, math.ceil(lay.n_tiles / max(1, n_splits)))
         n_splits = max(1, math.ceil(lay.n_tiles / tps))

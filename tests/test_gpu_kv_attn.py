@@ -80,10 +80,8 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("waves", ["0", "1"])          # both kernels for byte ids: tile shared by the waves / a stream per wave
 @pytest.mark.parametrize("D,Hkv,G,MQ,seg_len,q_pos0,bits,tps", CASES)
-def test_fwd_matches_the_oracle(D, Hkv, G, MQ, seg_len, q_pos0, bits, tps, waves, monkeypatch):
-    monkeypatch.setenv("QVB8_ATTN_WAVES", waves)
+def test_fwd_matches_the_oracle(D, Hkv, G, MQ, seg_len, q_pos0, bits, tps):
     lay = make_layout(D + MQ + G, seg_len, Hkv, D, bits=bits)
     rng = np.random.default_rng(11)
     q = (rng.normal(0, 1, (MQ, Hkv * G, D)) * D ** -0.5).astype(np.float16)
