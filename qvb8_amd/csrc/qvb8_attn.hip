@@ -63,6 +63,17 @@ template <> struct Quad<uint16_t> {
     static __device__ __forceinline__ float id(type w, int c) { return (float)(((c < 2 ? w.x : w.y) >> (16 * (c & 1))) & 0xFFFFu); }
 };
 
+// Two restored values as one dword of fp16: lo = fp16(fma(s0, d0, m0)), hi = fp16(fma(s1, d1, m1)), the fused
+// multiply-add rounded to fp32 FIRST and then to fp16, as the reference's `__floats2half2_rn(md + sp * (v - c))` does.
+// Written as `(_Float16)fmaf(...)` the compiler emits v_fma_mixlo_f16, which rounds the exact sum to fp16 in one step:
+// one fp16 ulp off in about one value of 4000 (measured against the oracle).  The conversion is kept out of its sight.
+__device__ __forceinline__ uint32_t restore_pair(float s0, float d0, float m0, float s1, float d1, float m1) {
+    const float lo = __builtin_fmaf(s0, d0, m0), hi = __builtin_fmaf(s1, d1, m1);
+    uint32_t r;
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    return r;
+}
+
 // One entry of the tile table through the scalar unit.  A plain load would do, but behind a barrier the compiler turns
 // it into a vector load, and waiting for that one (the youngest request) also waits for every id request still in
 // flight -- the prefetch would be worth nothing.
@@ -175,31 +186,33 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
 #pragma unroll
         for (int u = 0; u < UNITS; ++u) {
             const int kgp = kgp0 + KSTEP * u;
-            h4_t vcell[4];
+            uint2 vcell[4];
+            float dv[4][4];                                         // [key j][channel c]: id - centre of V
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int key = 4 * kgp + j;
-                h4_t kv;
+                float dk[4];
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    kv[c] = (_Float16)__builtin_fmaf(ks_[c], QD::id(rk[u][j], c) - kc, km[c]);
-                    vcell[c][j] = (_Float16)__builtin_fmaf(vs_[c], QD::id(rv[u][j], c) - vc, vm[c]);
-                }
-                *reinterpret_cast<h4_t*>(Ks + key * KROW + 4 * cg) = kv;
+                for (int c = 0; c < 4; ++c) { dk[c] = QD::id(rk[u][j], c) - kc; dv[j][c] = QD::id(rv[u][j], c) - vc; }
+                uint2 kv;
+                kv.x = restore_pair(ks_[0], dk[0], km[0], ks_[1], dk[1], km[1]);
+                kv.y = restore_pair(ks_[2], dk[2], km[2], ks_[3], dk[3], km[3]);
+                *reinterpret_cast<uint2*>(Ks + key * KROW + 4 * cg) = kv;
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                vcell[c].x = restore_pair(vs_[c], dv[0][c], vm[c], vs_[c], dv[1][c], vm[c]);
+                vcell[c].y = restore_pair(vs_[c], dv[2][c], vm[c], vs_[c], dv[3][c], vm[c]);
             }
             if (!whole) {
                 const uint32_t m0 = (4 * kgp + 0 < nlen ? 0x0000FFFFu : 0u) | (4 * kgp + 1 < nlen ? 0xFFFF0000u : 0u);
                 const uint32_t m1 = (4 * kgp + 2 < nlen ? 0x0000FFFFu : 0u) | (4 * kgp + 3 < nlen ? 0xFFFF0000u : 0u);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    uint2 w = *reinterpret_cast<uint2*>(&vcell[c]);
-                    w.x &= m0; w.y &= m1;
-                    vcell[c] = *reinterpret_cast<h4_t*>(&w);
-                }
+                for (int c = 0; c < 4; ++c) { vcell[c].x &= m0; vcell[c].y &= m1; }
             }
 #pragma unroll
             for (int c = 0; c < 4; ++c)
-                *reinterpret_cast<h4_t*>(Vt + (4 * cg + c) * kKeys + 4 * (kgp ^ (cg & 7))) = vcell[c];
+                *reinterpret_cast<uint2*>(Vt + (4 * cg + c) * kKeys + 4 * (kgp ^ (cg & 7))) = vcell[c];
         }
         __syncthreads();
         fetch(t + 2, rk, rv, ref);

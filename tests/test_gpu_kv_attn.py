@@ -242,3 +242,34 @@ def test_combine_matches_the_oracle():
         fin = np.isfinite(want_lse)
         assert np.allclose(lse.cpu().numpy()[fin], want_lse[fin], rtol=1e-6, atol=1e-5)
         assert np.all(got.cpu().numpy()[0, 0] == 0)
+
+
+@pytest.mark.parametrize("D,bits,wide", [(128, 6, False), (256, 8, False), (128, 11, True), (256, 9, True)])
+def test_restored_keys_and_values_are_the_oracles_bits(D, bits, wide):
+    """Read the kernel's restored K and V back, bit for bit: every key is a tile and a split of its own, so a split's
+    p is exp(0) = 1 and its output row IS the restored V of that key, and with a one-hot query its running maximum IS
+    one restored K element (1.0 * k, alone in an fp32 sum)."""
+    Hkv, n = 2, 37
+    lay = make_layout(D + bits, [20, 17], Hkv, D, bits=bits, spread=3.0)
+    lay["ts"] = np.arange(n, dtype=np.int32)
+    lay["tl"] = np.ones(n, np.int32)
+    lay["tseg"] = (np.arange(n) >= 20).astype(np.int32)
+    dl = to_device(lay, wide=wide)
+    G = 16
+    K = np.zeros((n, Hkv, D), np.float32)
+    V = np.zeros_like(K)
+    for c0 in range(0, D, G):
+        q = np.zeros((1, Hkv * G, D), np.float16)
+        for g in range(G):
+            q[0, np.arange(Hkv) * G + g, c0 + g] = 1.0
+        o, m, l = run_fwd(lay, dl, torch.from_numpy(q).to(DEV), n - 1, 1, G)        # (n splits, Hkv, G, ...)
+        assert np.all(l == 1.0)
+        K[:, :, c0:c0 + G] = m
+        V = o[:, :, 0, :]
+        assert np.array_equal(o, np.broadcast_to(o[:, :, :1, :], o.shape))
+    for h in range(Hkv):
+        for a, b, seg in ((0, 20, 0), (20, 37, 1)):
+            wk = A.restore_tile(lay["ki"][a:b, h], lay["kmid"][seg, h], lay["kstep"][seg, h], lay["kc"][seg, h])
+            wv = A.restore_tile(lay["vi"][a:b, h], lay["vmid"][seg, h], lay["vstep"][seg, h], lay["vc"][seg, h])
+            assert np.array_equal(K[a:b, h].view(np.uint32), wk.view(np.uint32))
+            assert np.array_equal(V[a:b, h].view(np.uint32), wv.view(np.uint32))
