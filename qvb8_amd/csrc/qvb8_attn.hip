@@ -14,7 +14,8 @@
 //   * ids are requested TWO tiles ahead into two register sets (a trip to memory under load takes longer than one tile's
 //     arithmetic): a wave reads whole key rows (64 lanes x 4 ids = 256 channels), every thread keeps the same four
 //     channels for all its keys, so it holds 4 + 4 constants per operand; no request sits under a branch (a tile past
-//     the split's end re-reads one cached line), so the counted waits leave the younger set in flight;
+//     the split's end re-reads one cached line), so the counted waits leave the younger set in flight; the tile table
+//     comes through the scalar unit;
 //   * restored K goes to LDS as [key][channel], restored V as [channel][key] (a thread owns 4 keys x 4 channels, so the
 //     transposition is free) with the 8-byte cells of a row swizzled by the channel group;
 //   * S = Q K^T: wave w takes keys 16 (w % 2) .. + 15 and half w / 2 of the channels (v_mfma_f32_16x16x16_f16, its part
