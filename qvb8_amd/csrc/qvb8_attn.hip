@@ -102,6 +102,9 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
     __shared__ __align__(16) _Float16 Ks[kKeys * KROW];
     __shared__ __align__(16) _Float16 Vt[D * kKeys];
     __shared__ __align__(16) float Ss[2 * kRows * kSStride];
+    constexpr int kPStride = kKeys + 8;                       // halfs per row of P
+    __shared__ __align__(16) _Float16 Ps[kRows * kPStride];
+    __shared__ __align__(16) float Al[kRows];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n16 = lane & 15, kg = lane >> 4;
@@ -124,6 +127,10 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
         }
     }
     const int qmin = a.q_pos0 + row0 / a.G;                                   // first position of the block's rows
+    // the softmax's own split of the block: this lane's row and pair of keys
+    const int srow = 4 * wave + (lane >> 4), kpair = lane & 15;
+    const bool srow_ok = row0 + srow < a.n_rows;
+    const int sqpos = a.q_pos0 + (srow_ok ? (row0 + srow) / a.G : 0);
     const int qmax = a.q_pos0 + (min(row0 + kRows, a.n_rows) - 1) / a.G;      // last position any row of the block sees
 
     const T* ki = reinterpret_cast<const T*>(a.ki) + (int64_t)h * a.s_h + 4 * cg;
@@ -230,54 +237,46 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
         }
         __syncthreads();
 
-        // ---- softmax of row n16 over the tile: this lane holds keys 16 kk + 4 kg + i ----
-        h4_t pa[2];
-        float alpha;
-        // every key of the tile counts for every row of the block (rows past n_rows compute on zeros and are never stored)
-        const bool all_seen = nlen == kKeys && start + kKeys - 1 <= qmin;
+        // ---- softmax, once per workgroup: wave w takes rows 4 w .. 4 w + 3, sixteen lanes a row, two keys a lane; the
+        //      probabilities (fp16) and the rows' rescale factors go to LDS for all four waves ----
         {
-            float sv[8], mx = -INFINITY;
+            // every key of the tile counts for every row of the block (rows past n_rows compute on zeros, never stored)
+            const bool all_seen = nlen == kKeys && start + kKeys - 1 <= qmin;
+            const float2 sa = *reinterpret_cast<const float2*>(Ss + srow * kSStride + 2 * kpair);
+            const float2 sb = *reinterpret_cast<const float2*>(Ss + (kRows + srow) * kSStride + 2 * kpair);
+            const bool ok0 = all_seen || (srow_ok && 2 * kpair < nlen && start + 2 * kpair <= sqpos);
+            const bool ok1 = all_seen || (srow_ok && 2 * kpair + 1 < nlen && start + 2 * kpair + 1 <= sqpos);
+            const float sv0 = ok0 ? (sa.x + sb.x) * a.scale : -INFINITY, sv1 = ok1 ? (sa.y + sb.y) * a.scale : -INFINITY;
+            float mx = fmaxf(sv0, sv1);
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-                const f4_t s4 = *reinterpret_cast<const f4_t*>(Ss + n16 * kSStride + 16 * kk + 4 * kg)
-                                + *reinterpret_cast<const f4_t*>(Ss + (kRows + n16) * kSStride + 16 * kk + 4 * kg);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int n = 16 * kk + 4 * kg + i;
-                    const bool ok = all_seen || (row_ok && n < nlen && start + n <= qpos);
-                    sv[4 * kk + i] = ok ? s4[i] * a.scale : -INFINITY;
-                    mx = fmaxf(mx, sv[4 * kk + i]);
-                }
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            for (int d = 1; d < 16; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
             const float m_new = fmaxf(m_run, mx);
             const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-            float sum = 0.f;
+            const _Float16 p0 = (_Float16)(sv0 == -INFINITY ? 0.f : __expf(sv0 - m_safe));
+            const _Float16 p1 = (_Float16)(sv1 == -INFINITY ? 0.f : __expf(sv1 - m_safe));
+            float sum = (float)p0 + (float)p1;                  // the rounded p, as the second product sees it
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float x = sv[4 * kk + i];
-                    const _Float16 p = (_Float16)(x == -INFINITY ? 0.f : __expf(x - m_safe));
-                    pa[kk][i] = p;
-                    sum += (float)p;                    // the rounded p, as the second product sees it
-                }
-            sum += __shfl_xor(sum, 16);
-            sum += __shfl_xor(sum, 32);
-            alpha = m_run == -INFINITY ? 0.f : (m_new == m_run ? 1.f : __expf(m_run - m_safe));
+            for (int d = 1; d < 16; d <<= 1) sum += __shfl_xor(sum, d);
+            const float alpha = m_run == -INFINITY ? 0.f : (m_new == m_run ? 1.f : __expf(m_run - m_safe));
             l_run = l_run * alpha + sum;
             m_run = m_new;
+            typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+            *reinterpret_cast<h2_t*>(Ps + srow * kPStride + 2 * kpair) = h2_t{p0, p1};
+            if (kpair == 0) Al[srow] = alpha;
         }
+        __syncthreads();
         // ---- O = alpha O + P V; the accumulator holds rows 4 kg + e of channel n16 of each fragment ----
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
-            float ae[4];
+        h4_t pa[2];
+        pa[0] = *reinterpret_cast<const h4_t*>(Ps + n16 * kPStride + 4 * kg);
+        pa[1] = *reinterpret_cast<const h4_t*>(Ps + n16 * kPStride + 16 + 4 * kg);
+        {
+            const f4_t ae = *reinterpret_cast<const f4_t*>(Al + 4 * kg);
+            if (__builtin_amdgcn_ballot_w64(ae[0] != 1.f || ae[1] != 1.f || ae[2] != 1.f || ae[3] != 1.f)) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) ae[e] = __shfl(alpha, 4 * kg + e);
+                for (int f = 0; f < NF; ++f)
 #pragma unroll
-            for (int f = 0; f < NF; ++f)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[f][e] *= ae[e];
+                    for (int e = 0; e < 4; ++e) acc[f][e] *= ae[e];
+            }
         }
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
@@ -321,9 +320,10 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
             const int r = row0 + 4 * kg_e + e;
             if (r < a.n_rows) a.o[(base + r) * D + wave_e * (D / 4) + 16 * f + n16_e] = acc[f][e];
         }
-    if (wave_e == 0 && kg_e == 0 && row0 + n16_e < a.n_rows) {
-        a.m[base + row0 + n16_e] = m_run;
-        a.l[base + row0 + n16_e] = l_run;
+    const int srow_e = 4 * wave_e + kg_e;                    // the row whose softmax state this lane holds
+    if (n16_e == 0 && row0 + srow_e < a.n_rows) {
+        a.m[base + row0 + srow_e] = m_run;
+        a.l[base + row0 + srow_e] = l_run;
     }
 }
 
