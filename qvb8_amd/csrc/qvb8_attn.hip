@@ -75,6 +75,19 @@ __device__ __forceinline__ uint32_t restore_pair(float s0, float d0, float m0, f
     return r;
 }
 
+// The value of the lane N places further on in its row of 16 lanes (a data-parallel move inside the vector unit; four of
+// them -- 8, 4, 2, 1 -- leave a row's maximum or sum in every lane, without the LDS trips of a general shuffle).
+template <int N>
+__device__ __forceinline__ float row_rotate(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float row_max16(float v) {
+    v = fmaxf(v, row_rotate<8>(v)); v = fmaxf(v, row_rotate<4>(v)); v = fmaxf(v, row_rotate<2>(v)); return fmaxf(v, row_rotate<1>(v));
+}
+__device__ __forceinline__ float row_sum16(float v) {
+    v += row_rotate<8>(v); v += row_rotate<4>(v); v += row_rotate<2>(v); return v + row_rotate<1>(v);
+}
+
 // One entry of the tile table through the scalar unit.  A plain load would do, but behind a barrier the compiler turns
 // it into a vector load, and waiting for that one (the youngest request) also waits for every id request still in
 // flight -- the prefetch would be worth nothing.
@@ -247,16 +260,12 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
             const bool ok0 = all_seen || (srow_ok && 2 * kpair < nlen && start + 2 * kpair <= sqpos);
             const bool ok1 = all_seen || (srow_ok && 2 * kpair + 1 < nlen && start + 2 * kpair + 1 <= sqpos);
             const float sv0 = ok0 ? (sa.x + sb.x) * a.scale : -INFINITY, sv1 = ok1 ? (sa.y + sb.y) * a.scale : -INFINITY;
-            float mx = fmaxf(sv0, sv1);
-#pragma unroll
-            for (int d = 1; d < 16; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+            const float mx = row_max16(fmaxf(sv0, sv1));
             const float m_new = fmaxf(m_run, mx);
             const float m_safe = m_new == -INFINITY ? 0.f : m_new;
             const _Float16 p0 = (_Float16)(sv0 == -INFINITY ? 0.f : __expf(sv0 - m_safe));
             const _Float16 p1 = (_Float16)(sv1 == -INFINITY ? 0.f : __expf(sv1 - m_safe));
-            float sum = (float)p0 + (float)p1;                  // the rounded p, as the second product sees it
-#pragma unroll
-            for (int d = 1; d < 16; d <<= 1) sum += __shfl_xor(sum, d);
+            const float sum = row_sum16((float)p0 + (float)p1);    // the rounded p, as the second product sees it
             const float alpha = m_run == -INFINITY ? 0.f : (m_new == m_run ? 1.f : __expf(m_run - m_safe));
             l_run = l_run * alpha + sum;
             m_run = m_new;
