@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
     constexpr int CG = D / 4;                  // channel groups (four channels each) of a key
     constexpr int KSTEP = kAttnThreads / CG;   // key groups (four keys each) that one pass of the workgroup covers
     constexpr int UNITS = D / 128;             // (4 keys x 4 channels) units per thread and tile
-    constexpr int KROW = D + 8;                // halfs per key in LDS
+    constexpr int KROW = D + 4;                // halfs per key in LDS: 16 keys' 8-byte reads fall on all banks once
     constexpr int NF = D / 64;                 // 16-channel output fragments per wave
     constexpr int NKS = D / 32;                // 16-channel steps of S = Q K^T per wave
     using QD = Quad<T>;
@@ -146,8 +146,10 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
     const int sqpos = a.q_pos0 + (srow_ok ? (row0 + srow) / a.G : 0);
     const int qmax = a.q_pos0 + (min(row0 + kRows, a.n_rows) - 1) / a.G;      // last position any row of the block sees
 
-    const T* ki = reinterpret_cast<const T*>(a.ki) + (int64_t)h * a.s_h + 4 * cg;
-    const T* vi = reinterpret_cast<const T*>(a.vi) + (int64_t)h * a.s_h + 4 * cg;
+    // the head's ids: a scalar base; the thread's four channels are part of its (32-bit) offset
+    const T* ki = reinterpret_cast<const T*>(a.ki) + (int64_t)h * a.s_h;
+    const T* vi = reinterpret_cast<const T*>(a.vi) + (int64_t)h * a.s_h;
+    const uint32_t cg_off = (uint32_t)(4 * cg) * (uint32_t)sizeof(T);
     const int t0 = (int)min((int64_t)sp * a.tps, (int64_t)a.n_tiles), t1 = (int)min((int64_t)t0 + a.tps, (int64_t)a.n_tiles);
     // ids of tile t into one register set: always 8 UNITS requests, none under a branch; keys past the tile's length
     // re-read its last key, and a tile that is not wanted -- past the split's end, or starting behind the last visible
@@ -170,7 +172,7 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
         for (int u = 0; u < UNITS; ++u)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const uint32_t off = min(key_off0 + (uint32_t)(4 * KSTEP * u + j) * key_stride, last_off);
+                const uint32_t off = min(key_off0 + (uint32_t)(4 * KSTEP * u + j) * key_stride, last_off) + cg_off;
                 rk[u][j] = *reinterpret_cast<const U*>(kb + off);
                 rv[u][j] = *reinterpret_cast<const U*>(vb + off);
             }
