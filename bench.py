@@ -442,7 +442,7 @@ def bench_attn(args, dev):
             "roofline": {"bound": "hbm", "achieved": round(gbs_kernel, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs_kernel / HBM_PEAK_GBS, 4),
                          # FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of one launch over 32768 keys (profiles/attn_kernels_*.md)
-                         "traffic": round((2 * 33143.4 + 4168.1) * 1024) if (n, MQ) == (32768, 1) else None,
+                         "traffic": round((2 * 33133.0 + 4168.1) * 1024) if (n, MQ) == (32768, 1) else None,
                          "kernel": "qvb8::attn_kernel<256, unsigned char>", "bytes_per_launch": nbytes, "launch_us": round(us, 3)},
             "cpu_baseline": None}
 

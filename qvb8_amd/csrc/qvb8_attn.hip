@@ -20,8 +20,9 @@
 //     transposition is free) with the 8-byte cells of a row swizzled by the channel group;
 //   * S = Q K^T: wave w takes keys 16 (w % 2) .. + 15 and half w / 2 of the channels (v_mfma_f32_16x16x16_f16, its part
 //     of Q kept in registers as the A operand); the two halves are added when S is read back;
-//   * all waves do the softmax of all 16 rows from S in LDS (same inputs, same results; no state in LDS) in the
-//     A-operand layout of the second product, so P needs no trip through LDS;
+//   * the softmax is computed once per workgroup (wave w rows 4 w .. 4 w + 3, sixteen lanes a row, two keys a lane, row
+//     maxima and sums by data-parallel rotations inside the row); the probabilities, rounded to fp16, and the rows'
+//     rescale factors reach the four waves through LDS in the A-operand layout of the second product;
 //   * O += P V: wave w owns a quarter of the output channels.
 #include <hip/hip_runtime.h>
 #include <math.h>
