@@ -10,7 +10,7 @@
 // probabilities rounded to fp16 before they are summed and multiplied; the result per split is the unnormalised
 // accumulator plus (running max, running sum), which the caller combines.
 //
-// Shape of this kernel (gfx950): 256 threads = 4 waves per workgroup, 16 query rows, 32 keys per tile.
+// Shape of this kernel (gfx950): 256 threads = 4 waves per workgroup, 16 query rows (or 2 / 4 blocks of 16), 32 keys per tile.
 //   * ids are requested TWO tiles ahead into two register sets (a trip to memory under load takes longer than one tile's
 //     arithmetic): a wave reads whole key rows (64 lanes x 4 ids = 256 channels), every thread keeps the same four
 //     channels for all its keys, so it holds 4 + 4 constants per operand; no request sits under a branch (a tile past
@@ -103,8 +103,10 @@ __device__ __forceinline__ void tile_entry(const int32_t* ts, const int32_t* tl,
 
 // Three workgroups per compute unit (two with 16-bit ids and 256 channels, whose two register sets are twice as large):
 // the third one is what hides a workgroup's barriers and dependent chains -- 74.9 against 82.3 us over 131072 keys.
-template <int D, typename T>
-__global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3) void attn_kernel(const AttnArgs a) {
+// RB = blocks of 16 query rows a workgroup serves from one restored tile (1, 2 or 4): the restore, most of the work, is
+// shared; every block has its own Q registers, scores, softmax state and accumulators (two workgroups per CU then).
+template <int D, typename T, int RB>
+__global__ __launch_bounds__(kAttnThreads, ((D == 256 && sizeof(T) == 2) || RB > 1) ? 2 : 3) void attn_kernel(const AttnArgs a) {
     constexpr int CG = D / 4;                  // channel groups (four channels each) of a key
     constexpr int KSTEP = kAttnThreads / CG;   // key groups (four keys each) that one pass of the workgroup covers
     constexpr int UNITS = D / 128;             // (4 keys x 4 channels) units per thread and tile
@@ -115,37 +117,35 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
     using U = typename QD::type;
     __shared__ __align__(16) _Float16 Ks[kKeys * KROW];
     __shared__ __align__(16) _Float16 Vt[D * kKeys];
-    __shared__ __align__(16) float Ss[2 * kRows * kSStride];
+    __shared__ __align__(16) float Ss[RB * 2 * kRows * kSStride];
     constexpr int kPStride = kKeys + 8;                       // halfs per row of P
-    __shared__ __align__(16) _Float16 Ps[kRows * kPStride];
-    __shared__ __align__(16) float Al[kRows];
+    __shared__ __align__(16) _Float16 Ps[RB * kRows * kPStride];
+    __shared__ __align__(16) float Al[RB * kRows];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n16 = lane & 15, kg = lane >> 4;
     const int kf = wave & 1, dh = wave >> 1;                  // this wave's 16 keys and its half of the channels in S
-    const int h = blockIdx.x, sp = blockIdx.y, row0 = blockIdx.z * kRows;
+    const int h = blockIdx.x, sp = blockIdx.y, row0 = blockIdx.z * (RB * kRows);
     const int cg = tid % CG, kgp0 = tid / CG;
 
-    // the lane's query row as the A operand of S = Q K^T: Q[row][16 ks + 4 kg .. + 3], ks in the wave's half
-    const int row = row0 + n16;
-    const bool row_ok = row < a.n_rows;
-    const int qpos = a.q_pos0 + (row_ok ? row / a.G : 0);
-    h4_t qa[NKS];
-    {
+    // the lane's query rows (one per block) as the A operand of S = Q K^T: Q[row][16 ks + 4 kg .. + 3], ks in the wave's half
+    h4_t qa[RB][NKS];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        const int row = row0 + rb * kRows + n16;
+        const bool row_ok = row < a.n_rows;
         const int rr = row_ok ? row : 0;
         const uint16_t* qp = a.q + (int64_t)(rr / a.G) * a.sq_r + (int64_t)(h * a.G + rr % a.G) * a.sq_h + dh * (D / 2) + 4 * kg;
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) {
             const h4_t v = *reinterpret_cast<const h4_t*>(qp + 16 * ks);
-            qa[ks] = row_ok ? v : h4_t{0, 0, 0, 0};
+            qa[rb][ks] = row_ok ? v : h4_t{0, 0, 0, 0};
         }
     }
     const int qmin = a.q_pos0 + row0 / a.G;                                   // first position of the block's rows
     // the softmax's own split of the block: this lane's row and pair of keys
-    const int srow = 4 * wave + (lane >> 4), kpair = lane & 15;
-    const bool srow_ok = row0 + srow < a.n_rows;
-    const int sqpos = a.q_pos0 + (srow_ok ? (row0 + srow) / a.G : 0);
-    const int qmax = a.q_pos0 + (min(row0 + kRows, a.n_rows) - 1) / a.G;      // last position any row of the block sees
+    const int srow = 4 * wave + (lane >> 4), kpair = lane & 15;             // row within a block
+    const int qmax = a.q_pos0 + (min(row0 + RB * kRows, a.n_rows) - 1) / a.G; // last position any row of the workgroup sees
 
     // the head's ids: a scalar base; the thread's four channels are part of its (32-bit) offset
     const T* ki = reinterpret_cast<const T*>(a.ki) + (int64_t)h * a.s_h;
@@ -179,10 +179,14 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
             }
     };
 
-    float m_run = -INFINITY, l_run = 0.f;
-    f4_t acc[NF];
+    float m_run[RB], l_run[RB];
+    f4_t acc[RB][NF];
 #pragma unroll
-    for (int f = 0; f < NF; ++f) acc[f] = f4_t{0.f, 0.f, 0.f, 0.f};
+    for (int rb = 0; rb < RB; ++rb) {
+        m_run[rb] = -INFINITY; l_run[rb] = 0.f;
+#pragma unroll
+        for (int f = 0; f < NF; ++f) acc[rb][f] = f4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     int cur_seg = -1;
     float km[4] = {0.f, 0.f, 0.f, 0.f}, ks_[4] = {0.f, 0.f, 0.f, 0.f}, vm[4] = {0.f, 0.f, 0.f, 0.f}, vs_[4] = {0.f, 0.f, 0.f, 0.f}, kc = 0.f, vc = 0.f;
@@ -241,53 +245,68 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
         __syncthreads();
         fetch(t + 2, rk, rv, ref);
 
-        // ---- S = Q K^T: this wave's 16 keys, its half of the channels ----
+        // ---- S = Q K^T: this wave's 16 keys, its half of the channels; a K operand serves every row block ----
         {
-            f4_t s = {0.f, 0.f, 0.f, 0.f};
+            f4_t sc[RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) sc[rb] = f4_t{0.f, 0.f, 0.f, 0.f};
             const _Float16* kp = Ks + (16 * kf + n16) * KROW + dh * (D / 2) + 4 * kg;
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks)
-                s = __builtin_amdgcn_mfma_f32_16x16x16f16(qa[ks], *reinterpret_cast<const h4_t*>(kp + 16 * ks), s, 0, 0, 0);
+            for (int ks = 0; ks < NKS; ++ks) {
+                const h4_t kb = *reinterpret_cast<const h4_t*>(kp + 16 * ks);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) Ss[(dh * kRows + 4 * kg + e) * kSStride + 16 * kf + n16] = s[e];
+                for (int rb = 0; rb < RB; ++rb) sc[rb] = __builtin_amdgcn_mfma_f32_16x16x16f16(qa[rb][ks], kb, sc[rb], 0, 0, 0);
+            }
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) Ss[((2 * rb + dh) * kRows + 4 * kg + e) * kSStride + 16 * kf + n16] = sc[rb][e];
         }
         __syncthreads();
 
-        // ---- softmax, once per workgroup: wave w takes rows 4 w .. 4 w + 3, sixteen lanes a row, two keys a lane; the
-        //      probabilities (fp16) and the rows' rescale factors go to LDS for all four waves ----
+        // ---- softmax, once per workgroup: wave w takes rows 4 w .. 4 w + 3 of every block, sixteen lanes a row, two keys
+        //      a lane; the probabilities (fp16) and the rows' rescale factors go to LDS for all four waves ----
         {
-            // every key of the tile counts for every row of the block (rows past n_rows compute on zeros, never stored)
+            // every key of the tile counts for every row of the workgroup (rows past n_rows compute on zeros, never stored)
             const bool all_seen = nlen == kKeys && start + kKeys - 1 <= qmin;
-            const float2 sa = *reinterpret_cast<const float2*>(Ss + srow * kSStride + 2 * kpair);
-            const float2 sb = *reinterpret_cast<const float2*>(Ss + (kRows + srow) * kSStride + 2 * kpair);
-            const bool ok0 = all_seen || (srow_ok && 2 * kpair < nlen && start + 2 * kpair <= sqpos);
-            const bool ok1 = all_seen || (srow_ok && 2 * kpair + 1 < nlen && start + 2 * kpair + 1 <= sqpos);
-            const float sv0 = ok0 ? (sa.x + sb.x) * a.scale : -INFINITY, sv1 = ok1 ? (sa.y + sb.y) * a.scale : -INFINITY;
-            const float mx = row_max16(fmaxf(sv0, sv1));
-            const float m_new = fmaxf(m_run, mx);
-            const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-            const _Float16 p0 = (_Float16)(sv0 == -INFINITY ? 0.f : __expf(sv0 - m_safe));
-            const _Float16 p1 = (_Float16)(sv1 == -INFINITY ? 0.f : __expf(sv1 - m_safe));
-            const float sum = row_sum16((float)p0 + (float)p1);    // the rounded p, as the second product sees it
-            const float alpha = m_run == -INFINITY ? 0.f : (m_new == m_run ? 1.f : __expf(m_run - m_safe));
-            l_run = l_run * alpha + sum;
-            m_run = m_new;
-            typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-            *reinterpret_cast<h2_t*>(Ps + srow * kPStride + 2 * kpair) = h2_t{p0, p1};
-            if (kpair == 0) Al[srow] = alpha;
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                const int prow = rb * kRows + srow;                // row within the workgroup
+                const bool srow_ok = row0 + prow < a.n_rows;
+                const int sqpos = a.q_pos0 + (srow_ok ? (row0 + prow) / a.G : 0);
+                const float2 sa = *reinterpret_cast<const float2*>(Ss + ((2 * rb) * kRows + srow) * kSStride + 2 * kpair);
+                const float2 sb = *reinterpret_cast<const float2*>(Ss + ((2 * rb + 1) * kRows + srow) * kSStride + 2 * kpair);
+                const bool ok0 = all_seen || (srow_ok && 2 * kpair < nlen && start + 2 * kpair <= sqpos);
+                const bool ok1 = all_seen || (srow_ok && 2 * kpair + 1 < nlen && start + 2 * kpair + 1 <= sqpos);
+                const float sv0 = ok0 ? (sa.x + sb.x) * a.scale : -INFINITY, sv1 = ok1 ? (sa.y + sb.y) * a.scale : -INFINITY;
+                const float mx = row_max16(fmaxf(sv0, sv1));
+                const float m_new = fmaxf(m_run[rb], mx);
+                const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+                const _Float16 p0 = (_Float16)(sv0 == -INFINITY ? 0.f : __expf(sv0 - m_safe));
+                const _Float16 p1 = (_Float16)(sv1 == -INFINITY ? 0.f : __expf(sv1 - m_safe));
+                const float sum = row_sum16((float)p0 + (float)p1);    // the rounded p, as the second product sees it
+                const float alpha = m_run[rb] == -INFINITY ? 0.f : (m_new == m_run[rb] ? 1.f : __expf(m_run[rb] - m_safe));
+                l_run[rb] = l_run[rb] * alpha + sum;
+                m_run[rb] = m_new;
+                typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+                *reinterpret_cast<h2_t*>(Ps + prow * kPStride + 2 * kpair) = h2_t{p0, p1};
+                if (kpair == 0) Al[prow] = alpha;
+            }
         }
         __syncthreads();
-        // ---- O = alpha O + P V; the accumulator holds rows 4 kg + e of channel n16 of each fragment ----
-        h4_t pa[2];
-        pa[0] = *reinterpret_cast<const h4_t*>(Ps + n16 * kPStride + 4 * kg);
-        pa[1] = *reinterpret_cast<const h4_t*>(Ps + n16 * kPStride + 16 + 4 * kg);
-        {
-            const f4_t ae = *reinterpret_cast<const f4_t*>(Al + 4 * kg);
+        // ---- O = alpha O + P V; the accumulator holds rows 4 kg + e of channel n16 of each fragment; a V operand serves
+        //      every row block ----
+        h4_t pa[RB][2];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            pa[rb][0] = *reinterpret_cast<const h4_t*>(Ps + (rb * kRows + n16) * kPStride + 4 * kg);
+            pa[rb][1] = *reinterpret_cast<const h4_t*>(Ps + (rb * kRows + n16) * kPStride + 16 + 4 * kg);
+            const f4_t ae = *reinterpret_cast<const f4_t*>(Al + rb * kRows + 4 * kg);
             if (__builtin_amdgcn_ballot_w64(ae[0] != 1.f || ae[1] != 1.f || ae[2] != 1.f || ae[3] != 1.f)) {
 #pragma unroll
                 for (int f = 0; f < NF; ++f)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[f][e] *= ae[e];
+                    for (int e = 0; e < 4; ++e) acc[rb][f][e] *= ae[e];
             }
         }
 #pragma unroll
@@ -296,7 +315,8 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
             for (int f = 0; f < NF; ++f) {
                 const int ch = wave * (D / 4) + 16 * f + n16;
                 const h4_t b = *reinterpret_cast<const h4_t*>(Vt + ch * kKeys + 4 * ((4 * kk + kg) ^ ((ch >> 2) & 7)));
-                acc[f] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[kk], b, acc[f], 0, 0, 0);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) acc[rb][f] = __builtin_amdgcn_mfma_f32_16x16x16f16(pa[rb][kk], b, acc[rb][f], 0, 0, 0);
             }
         __syncthreads();                                  // the tile in LDS is free again
     };
@@ -325,17 +345,21 @@ __global__ __launch_bounds__(kAttnThreads, (D == 256 && sizeof(T) == 2) ? 2 : 3)
     asm volatile("" : "+v"(tid_e));
     const int lane_e = tid_e & 63, wave_e = tid_e >> 6, n16_e = lane_e & 15, kg_e = lane_e >> 4;
     const int64_t base = ((int64_t)sp * a.nhkv + h) * a.n_rows;
+    const int srow_e = 4 * wave_e + kg_e;                    // the row (of every block) whose softmax state this lane holds
 #pragma unroll
-    for (int f = 0; f < NF; ++f)
+    for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int r = row0 + 4 * kg_e + e;
-            if (r < a.n_rows) a.o[(base + r) * D + wave_e * (D / 4) + 16 * f + n16_e] = acc[f][e];
+        for (int f = 0; f < NF; ++f)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int r = row0 + rb * kRows + 4 * kg_e + e;
+                if (r < a.n_rows) a.o[(base + r) * D + wave_e * (D / 4) + 16 * f + n16_e] = acc[rb][f][e];
+            }
+        const int r = row0 + rb * kRows + srow_e;
+        if (n16_e == 0 && r < a.n_rows) {
+            a.m[base + r] = m_run[rb];
+            a.l[base + r] = l_run[rb];
         }
-    const int srow_e = 4 * wave_e + kg_e;                    // the row whose softmax state this lane holds
-    if (n16_e == 0 && row0 + srow_e < a.n_rows) {
-        a.m[base + row0 + srow_e] = m_run;
-        a.l[base + row0 + srow_e] = l_run;
     }
 }
 
@@ -385,8 +409,17 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
 
 template <int D, typename T>
 int launch_attn(const AttnArgs& a, int64_t n_splits, hipStream_t s) {
-    const dim3 grid((unsigned)a.nhkv, (unsigned)n_splits, (unsigned)((a.n_rows + kRows - 1) / kRows));
-    hipLaunchKernelGGL((attn_kernel<D, T>), grid, dim3(kAttnThreads), 0, s, a);
+    // up to 16 rows: one block per workgroup; up to 32: two; beyond: four with 128 channels, two with 256 (four blocks'
+    // accumulators and Q do not fit the registers there).  QVB8_ATTN_ROW_BLOCKS forces 1, 2 or 4.
+    int rb = a.n_rows <= kRows ? 1 : a.n_rows <= 2 * kRows ? 2 : 4;
+    const int forced = host::env_int("QVB8_ATTN_ROW_BLOCKS", 0);
+    if (forced == 1 || forced == 2 || forced == 4) rb = forced;
+    if (D == 256 && rb > 2) rb = 2;
+    const dim3 grid((unsigned)a.nhkv, (unsigned)n_splits, (unsigned)((a.n_rows + rb * kRows - 1) / (rb * kRows)));
+    if (grid.z > 65535u) return host::fail(-1, "qvb8_attn_fwd: %d rows are more than one launch takes", a.n_rows);
+    if (rb == 1) hipLaunchKernelGGL((attn_kernel<D, T, 1>), grid, dim3(kAttnThreads), 0, s, a);
+    else if (rb == 2) hipLaunchKernelGGL((attn_kernel<D, T, 2>), grid, dim3(kAttnThreads), 0, s, a);
+    else if constexpr (D == 128) hipLaunchKernelGGL((attn_kernel<D, T, 4>), grid, dim3(kAttnThreads), 0, s, a);
     return host::check_launch("qvb8_attn_fwd");
 }
 

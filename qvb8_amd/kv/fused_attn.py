@@ -15,7 +15,6 @@ import torch
 from qvb8_amd import _lib
 
 BLOCK_N = 32          # keys per tile of the table; the kernel takes tiles of at most 32 keys
-ROWS_PER_BLOCK = 16   # query rows one workgroup of the kernel handles
 
 
 class QVLayout:
@@ -98,13 +97,22 @@ def fwd(q, ki, vi, kmid, kstep, vmid, vstep, kc, vc, ts, tl, tseg, o, m, l, q_po
     _lib._check(rc, lib)
 
 
-def plan_splits(n_tiles: int, hkv: int, rows: int, device, per_cu: int = 3) -> tuple:
-    """(tiles per split, splits): as many workgroups as the card holds at once -- `per_cu` per compute unit: three, or
-    two for 16-bit ids with 256 channels (the kernel's registers) -- and fewer splits for long query blocks
-    (fused_attn.py:259-264, 271-275).  Measured over 32768 / 131072 keys with three resident workgroups: 768 workgroups
-    27.2 / 74.9 us, 512 27.7 / 86.1, 1024 28.5 / 81.8, 1536 29.5 / 76.5."""
-    n_rb = -(-rows // ROWS_PER_BLOCK)
+def rows_per_workgroup(rows: int, d: int) -> int:
+    """Query rows one workgroup of the kernel serves from a restored tile: 16, 32 from 17 rows on, 64 from 33 rows on
+    when the heads have 128 channels (qvb8_attn.hip, launch_attn)."""
+    return 16 if rows <= 16 else 32 if (rows <= 32 or d == 256) else 64
+
+
+def plan_splits(n_tiles: int, hkv: int, rows: int, device, per_cu: int | None = None, d: int = 256, wide: bool = False) -> tuple:
+    """(tiles per split, splits): as many workgroups as the card holds at once -- three per compute unit, two when a
+    workgroup serves more than 16 rows or reads 16-bit ids with 256 channels (the kernel's registers) -- and fewer
+    splits for long query blocks (fused_attn.py:259-264, 271-275).  Measured over 32768 / 131072 keys with three
+    resident workgroups of 16 rows: 768 workgroups 27.2 / 74.9 us, 512 27.7 / 86.1, 1024 28.5 / 81.8, 1536 29.5 / 76.5."""
+    block = rows_per_workgroup(rows, d)
+    if per_cu is None:
+        per_cu = 2 if (block > 16 or (wide and d == 256)) else 3
     per_cu = int(os.environ.get("QVB8_ATTN_WG_PER_CU", per_cu))          # a knob for measurements
+    n_rb = -(-rows // block)
     want = per_cu * torch.cuda.get_device_properties(device).multi_processor_count
     n_splits = max(1, min(n_tiles, want // max(1, hkv * n_rb)))
     tps = max(1, math.ceil(n_tiles / n_splits))
@@ -136,7 +144,7 @@ def attend(q, lay: QVLayout, q_pos0: int, scale: float, n_splits: int | None = N
     g = hq // hkv
     rows = mq * g
     if n_splits is None:
-        tps, n_splits = plan_splits(lay.n_tiles, hkv, rows, q.device, 2 if (lay.ki.dtype == torch.int16 and d == 256) else 3)
+        tps, n_splits = plan_splits(lay.n_tiles, hkv, rows, q.device, d=d, wide=lay.ki.dtype == torch.int16)
     else:
         tps = max(1, math.ceil(lay.n_tiles / max(1, n_splits)))
         n_splits = max(1, math.ceil(lay.n_tiles / tps))

@@ -77,6 +77,11 @@ CASES = [
     (256, 2, 2, 1, [1], 0, 6, 1),
     (256, 1, 6, 1, [500, 17], 516, 6, 7),             # splits of 7 tiles: both register sets and the odd last piece in use
     (128, 2, 4, 2, [333], 332, 7, 5),
+    # more than 16 rows: a workgroup serves two or four blocks of 16 rows from one restored tile
+    (256, 1, 6, 4, [90, 40], 126, 6, 2),              # 24 rows: two blocks, the second half empty
+    (256, 2, 8, 5, [70], 65, 6, 1),                   # 40 rows: two workgroups of two blocks, causal cut inside
+    (128, 1, 8, 3, [64, 3], 64, 6, 2),                # 24 rows, 128 channels
+    (128, 2, 6, 11, [100], 95, 6, 3),                 # 66 rows: four blocks + a second workgroup with two rows
 ]
 
 
@@ -273,3 +278,16 @@ def test_restored_keys_and_values_are_the_oracles_bits(D, bits, wide):
             wv = A.restore_tile(lay["vi"][a:b, h], lay["vmid"][seg, h], lay["vstep"][seg, h], lay["vc"][seg, h])
             assert np.array_equal(K[a:b, h].view(np.uint32), wk.view(np.uint32))
             assert np.array_equal(V[a:b, h].view(np.uint32), wv.view(np.uint32))
+
+
+@pytest.mark.parametrize("blocks", ["1", "2", "4"])
+def test_row_blocks_per_workgroup_do_not_change_the_result(blocks, monkeypatch):
+    """The same 36 rows served as three workgroups of one block, two of two, one of four (128 channels)."""
+    lay = make_layout(21, [100], 2, 128)
+    rng = np.random.default_rng(5)
+    q = (rng.normal(0, 1, (12, 6, 128)) * 128 ** -0.5).astype(np.float16)
+    want = A.fwd_split(q, lay["ki"], lay["vi"], lay["kmid"], lay["kstep"], lay["vmid"], lay["vstep"], lay["kc"], lay["vc"],
+                       lay["ts"], lay["tl"], lay["tseg"], 88, 2, 1.0, 3)
+    monkeypatch.setenv("QVB8_ATTN_ROW_BLOCKS", blocks)
+    got = run_fwd(lay, to_device(lay), torch.from_numpy(q).to(DEV), 88, 2, 3)
+    check_split_outputs(got, want, lay)
