@@ -388,7 +388,7 @@ def bench_attn(args, dev):
     ids of K and V once, the per-channel constants, q, and the per-split results written."""
     import torch
     from qvb8_amd.kv import codec as KC, fused_attn as FA
-    n, hkv, G, D, seg, MQ = args.context, 4, 6, 256, 4096, args.tokens
+    n, hkv, G, D, seg, MQ = args.context, 4, 6, args.head_dim, 4096, args.tokens
     gen = torch.Generator(device=dev).manual_seed(5)
     lays = []
     for li in range(args.layers):
@@ -403,7 +403,7 @@ def bench_attn(args, dev):
         lays.append(FA.layout_from_segments(segs_k, segs_v, seg_len, dev))
     lay0 = lays[0]
     rows = MQ * G
-    tps, n_splits = FA.plan_splits(lay0.n_tiles, hkv, rows, dev)
+    tps, n_splits = FA.plan_splits(lay0.n_tiles, hkv, rows, dev, d=D)
     scale = D ** -0.5
     q = torch.randn(MQ, hkv * G, D, device=dev, generator=gen).to(torch.bfloat16)
     q16 = (q.float() * scale).clamp_(-65504.0, 65504.0).to(torch.float16).contiguous()
@@ -435,15 +435,15 @@ def bench_attn(args, dev):
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "fp16 restored keys and values, fp32 accumulate", "data": "synthetic",
-            "config": {"workload": "attention of %d query token(s), 24 heads over %d kv heads x 256 channels, %d keys as 6-bit ids "
+            "config": {"workload": "attention of %d query token(s), 24 heads over %d kv heads x %d channels, %d keys as 6-bit ids "
                                    "in bytes in segments of %d, %d layers with their own caches, %d splits of %d tiles"
-                                   % (MQ, hkv, n, seg, len(lays), n_splits, tps),
+                                   % (MQ, hkv, D, n, seg, len(lays), n_splits, tps),
                        "bytes_per_launch": nbytes, "us_per_layer": round(ms * 1e3 / len(lays), 2)},
             "roofline": {"bound": "hbm", "achieved": round(gbs_kernel, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs_kernel / HBM_PEAK_GBS, 4),
                          # FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 of one launch over 32768 keys (profiles/attn_kernels_*.md)
-                         "traffic": round((2 * 33133.0 + 4168.1) * 1024) if (n, MQ) == (32768, 1) else None,
-                         "kernel": "qvb8::attn_kernel<256, unsigned char>", "bytes_per_launch": nbytes, "launch_us": round(us, 3)},
+                         "traffic": round((2 * 33133.0 + 4168.1) * 1024) if (n, MQ, D) == (32768, 1, 256) else None,
+                         "kernel": "qvb8::attn_kernel<%d, unsigned char, %d>" % (D, 1 if MQ * G <= 16 else 2 if (MQ * G <= 32 or D == 256) else 4), "bytes_per_launch": nbytes, "launch_us": round(us, 3)},
             "cpu_baseline": None}
 
 
@@ -497,6 +497,7 @@ def main():
                          "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256); "
                          "lmhead / embed: the 248320 x 5120 vocabulary table; attn: decode-step attention over a banded KV cache")
     ap.add_argument("--context", type=int, default=32768, help="keys in the cache of the attn workload")
+    ap.add_argument("--head-dim", type=int, default=256, choices=(128, 256), help="channels per head of the attn workload")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
     ap.add_argument("--model", choices=("9b", "27b"), default="9b",
                     help="decode9b workload only: layer shapes (9b = the headline configuration; 27b = hidden 5120, FFN 17408)")

@@ -104,13 +104,14 @@ def rows_per_workgroup(rows: int, d: int) -> int:
 
 
 def plan_splits(n_tiles: int, hkv: int, rows: int, device, per_cu: int | None = None, d: int = 256, wide: bool = False) -> tuple:
-    """(tiles per split, splits): as many workgroups as the card holds at once -- three per compute unit, two when a
-    workgroup serves more than 16 rows or reads 16-bit ids with 256 channels (the kernel's registers) -- and fewer
+    """(tiles per split, splits): as many workgroups as the card holds at once -- three per compute unit (four with byte ids and
+    128 channels), two when a workgroup serves more than 16 rows or reads 16-bit ids with 256 channels (the kernel's
+    registers) -- and fewer
     splits for long query blocks (fused_attn.py:259-264, 271-275).  Measured over 32768 / 131072 keys with three
     resident workgroups of 16 rows: 768 workgroups 27.2 / 74.9 us, 512 27.7 / 86.1, 1024 28.5 / 81.8, 1536 29.5 / 76.5."""
     block = rows_per_workgroup(rows, d)
     if per_cu is None:
-        per_cu = 2 if (block > 16 or (wide and d == 256)) else 3
+        per_cu = 2 if (block > 16 or (wide and d == 256)) else 4 if (d == 128 and not wide) else 3
     per_cu = int(os.environ.get("QVB8_ATTN_WG_PER_CU", per_cu))          # a knob for measurements
     n_rb = -(-rows // block)
     want = per_cu * torch.cuda.get_device_properties(device).multi_processor_count
