@@ -291,3 +291,23 @@ def test_row_blocks_per_workgroup_do_not_change_the_result(blocks, monkeypatch):
     monkeypatch.setenv("QVB8_ATTN_ROW_BLOCKS", blocks)
     got = run_fwd(lay, to_device(lay), torch.from_numpy(q).to(DEV), 88, 2, 3)
     check_split_outputs(got, want, lay)
+
+
+def test_random_shapes_match_the_oracle():
+    """Sixty seeded random caches and query blocks: head_dim, heads, group size, tokens, ragged segments, id width, the
+    first query position (before, inside and behind the cache), tiles per split, embedded buffers."""
+    rng = np.random.default_rng(12345)
+    for it in range(60):
+        D = int(rng.choice([128, 256])); Hkv = int(rng.integers(1, 4)); G = int(rng.choice([1, 2, 3, 4, 6, 8])); MQ = int(rng.integers(1, 14))
+        seg_len = [int(rng.integers(1, 120)) for _ in range(int(rng.integers(1, 4)))]
+        n = sum(seg_len); bits = int(rng.choice([4, 6, 8, 10]))
+        q_pos0 = int(rng.integers(-3, n + 5)); tps = int(rng.choice([1, 2, 3, 5, 8, 1000]))
+        lay = make_layout(1000 + it, seg_len, Hkv, D, bits=bits)
+        q = (rng.normal(0, 1, (MQ, Hkv * G, D)) * D ** -0.5).astype(np.float16)
+        want = A.fwd_split(q, lay["ki"], lay["vi"], lay["kmid"], lay["kstep"], lay["vmid"], lay["vstep"], lay["kc"], lay["vc"],
+                           lay["ts"], lay["tl"], lay["tseg"], q_pos0, tps, 1.0, G)
+        got = run_fwd(lay, to_device(lay, wide=bits > 8, slack=int(rng.integers(0, 3))), torch.from_numpy(q).to(DEV), q_pos0, tps, G)
+        try:
+            check_split_outputs(got, want, lay)
+        except AssertionError as ex:
+            raise AssertionError(f"case {it}: D={D} Hkv={Hkv} G={G} MQ={MQ} seg_len={seg_len} bits={bits} q_pos0={q_pos0} tps={tps}") from ex
