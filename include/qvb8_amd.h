@@ -83,6 +83,11 @@ int qvb8_certify(const void* restored, int restored_dtype, const void* original,
 /* out_f16[i] = fp16(clamp(x[i], -65504, 65504)), NaN kept.  Replaces saturating_half  qvb8_cuda.cu:761-841. */
 int qvb8_sat_half(const void* x, int x_dtype, int64_t n, void* out_f16, void* stream);
 
+/* out_f16[i] = fp16(clamp((float)x[i] * scale, -65504, 65504)), NaN kept: the queries of the banded-KV attention with the
+ * softmax scale folded in, one launch.  Replaces `(q.float() * scale).clamp_(-65504.0, 65504.0).to(torch.float16)` of
+ * attend  kv/fused_attn.py:276-279. */
+int qvb8_scale_sat_half(const void* x, int x_dtype, int64_t n, float scale, void* out_f16, void* stream);
+
 /* ---- fused decode + GEMV, M = 1..8 ---------------------------------------------------------------------- */
 
 /* Bytes of workspace qvb8_gemv needs for this shape (0 is possible). */

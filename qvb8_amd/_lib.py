@@ -17,7 +17,7 @@ _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 # every symbol include/qvb8_amd.h declares
 SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_lookup_rows", "qvb8_scatter_escapes", "qvb8_certify",
-           "qvb8_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma",
+           "qvb8_sat_half", "qvb8_scale_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma",
            "qvb8_moe_workspace_bytes", "qvb8_moe_experts",
            "qvb8r_decode", "qvb8r_gemv_workspace_bytes", "qvb8r_gemv", "qvb8r_fix_escapes", "qvb8_attn_fwd", "qvb8_attn_combine")
 
@@ -55,6 +55,7 @@ def load(build_if_missing: bool = True):
     lib.qvb8_scatter_escapes.argtypes = [vp, i32, i64, vp, vp, i64, vp]
     lib.qvb8_certify.argtypes = [vp, i32, vp, i32, i64, ctypes.c_float, vp, vp]
     lib.qvb8_sat_half.argtypes = [vp, i32, i64, vp, vp]
+    lib.qvb8_scale_sat_half.argtypes = [vp, i32, i64, ctypes.c_float, vp, vp]
     lib.qvb8_gemv_workspace_bytes.argtypes = [i64, i64, i64]
     lib.qvb8_gemv_workspace_bytes.restype = i64
     lib.qvb8_gemv.argtypes = [vp, i32, i64, vp, i64, vp, vp, vp, vp, i64, i64, vp, vp, i64, vp, vp, i64, vp]

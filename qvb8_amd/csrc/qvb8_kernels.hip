@@ -204,6 +204,12 @@ __global__ void __launch_bounds__(256) sat_half_kernel(const void* __restrict__ 
     if (i < n) out[i] = (uint16_t)sat_half_bits(load_as_f32<DT>(x, i));
 }
 
+template <int DT>
+__global__ void __launch_bounds__(256) scale_sat_half_kernel(const void* __restrict__ x, float scale, uint16_t* __restrict__ out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (uint16_t)sat_half_bits(load_as_f32<DT>(x, i) * scale);
+}
+
 // ===========================================================================================================
 // fused decode + GEMV, M = MB rows of X (1..8)
 // ===========================================================================================================
@@ -634,6 +640,21 @@ extern "C" int qvb8_sat_half(const void* x, int x_dtype, int64_t n, void* out_f1
         default: hipLaunchKernelGGL(sat_half_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, s, x, (uint16_t*)out_f16, n); break;
     }
     return host::check_launch("qvb8_sat_half");
+}
+
+extern "C" int qvb8_scale_sat_half(const void* x, int x_dtype, int64_t n, float scale, void* out_f16, void* stream) {
+    if (x_dtype < 0 || x_dtype > 2 || n < 0) return host::fail(QVB8_ERR_ARG, "qvb8_scale_sat_half: bad argument");
+    if (n == 0) return QVB8_OK;
+    if (!x || !out_f16) return host::fail(QVB8_ERR_ARG, "qvb8_scale_sat_half: null pointer");
+    const int64_t blocks = (n + 255) / 256;
+    if (blocks > 0x7fffffff) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_scale_sat_half: too large");
+    hipStream_t s = (hipStream_t)stream;
+    switch (x_dtype) {
+        case QVB8_F32: hipLaunchKernelGGL(scale_sat_half_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, s, x, scale, (uint16_t*)out_f16, n); break;
+        case QVB8_F16: hipLaunchKernelGGL(scale_sat_half_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, s, x, scale, (uint16_t*)out_f16, n); break;
+        default: hipLaunchKernelGGL(scale_sat_half_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, s, x, scale, (uint16_t*)out_f16, n); break;
+    }
+    return host::check_launch("qvb8_scale_sat_half");
 }
 
 // ---- GEMV launch plan --------------------------------------------------------------------------------------

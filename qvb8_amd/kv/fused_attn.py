@@ -151,7 +151,14 @@ def attend(q, lay: QVLayout, q_pos0: int, scale: float, n_splits: int | None = N
         n_splits = max(1, math.ceil(lay.n_tiles / tps))
     # fp16 queries: the softmax scale goes in first (|q| shrinks), then they saturate, so that an outlier channel cannot
     # turn into inf and a row into NaN (fused_attn.py:276-279)
-    q16 = (q.float() * scale).clamp_(-65504.0, 65504.0).to(torch.float16).contiguous()
+    qc = q.contiguous()
+    if qc.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        qc = qc.float()
+    q16 = torch.empty(qc.shape, dtype=torch.float16, device=qc.device)
+    lib = _lib.load()
+    with torch.cuda.device(qc.device):
+        _lib._check(lib.qvb8_scale_sat_half(qc.data_ptr(), _lib.dtype_code(qc.dtype), qc.numel(), float(scale), q16.data_ptr(),
+                                            torch.cuda.current_stream().cuda_stream), lib)
     o = torch.empty(n_splits, hkv, rows, d, dtype=torch.float32, device=q.device)
     m = torch.empty(n_splits, hkv, rows, dtype=torch.float32, device=q.device)
     l = torch.empty_like(m)

@@ -311,3 +311,21 @@ def test_random_shapes_match_the_oracle():
             check_split_outputs(got, want, lay)
         except AssertionError as ex:
             raise AssertionError(f"case {it}: D={D} Hkv={Hkv} G={G} MQ={MQ} seg_len={seg_len} bits={bits} q_pos0={q_pos0} tps={tps}") from ex
+
+
+def test_query_preparation_is_the_callers_expression():
+    """qvb8_scale_sat_half == (q.float() * scale).clamp(-65504, 65504).to(fp16), bit for bit, NaN and overflow included."""
+    from qvb8_amd import _lib
+    lib = _lib.load()
+    g = torch.Generator(device=DEV).manual_seed(3)
+    for dt in (torch.bfloat16, torch.float16, torch.float32):
+        x = (torch.randn(5, 12, 128, device=DEV, generator=g) * 300).to(dt)
+        x.view(-1)[:4] = torch.tensor([float("nan"), float("inf"), -float("inf"), 6e4], device=DEV).to(dt)
+        for scale in (128 ** -0.5, 1.0, 40.0):
+            out = torch.empty(x.shape, dtype=torch.float16, device=DEV)
+            rc = lib.qvb8_scale_sat_half(x.data_ptr(), _lib.dtype_code(dt), x.numel(), scale, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+            assert rc == 0
+            want = (x.float() * scale).clamp(-65504.0, 65504.0).to(torch.float16)
+            assert torch.equal(out.view(torch.int16)[~torch.isnan(want)], want.view(torch.int16)[~torch.isnan(want)])
+            assert torch.equal(torch.isnan(out), torch.isnan(want))
+    assert lib.qvb8_scale_sat_half(None, 0, 4, 1.0, None, None) != 0 and lib.qvb8_scale_sat_half(None, 0, 0, 1.0, None, None) == 0
