@@ -38,7 +38,8 @@ enum qvb8_status {
     QVB8_ERR_UNSUPPORTED = -4 /* configuration this build does not cover */
 };
 
-/* Library identification: ABI version (bumped on any signature change). */
+/* Library identification: ABI version, bumped on any signature change or new entry point (3: row lookup, attention over
+ * the banded KV cache, query preparation). */
 int qvb8_abi_version(void);
 /* Message of the calling thread's most recent failure ("" if none). Valid until that thread's next call. */
 const char* qvb8_last_error(void);
