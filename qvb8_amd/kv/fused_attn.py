@@ -21,7 +21,11 @@ class QVLayout:
     """The id buffers, constants and tile table of one layer (fused_attn.py:155-186).  ki / vi: (capacity, Hkv, D)
     uint8, or int16 holding 16-bit patterns; kmin / vmin hold the range CENTRE when kc / vc are given."""
 
-    def __init__(self, ki, vi, kmin, kstep, vmin, vstep, seg_len, device, block_n=BLOCK_N, kc=None, vc=None):
+    def __init__(self, ki, vi, kmin, kstep, vmin, vstep, seg_len, device, block_n=BLOCK_N, kc=None, vc=None,
+                 hk=None, hv=None, hrow=None):
+        if hk is not None or hv is not None or hrow is not None:
+            raise NotImplementedError("the high-byte pool of 9..16-bit heads is not read: store such layers' ids in 16 bits "
+                                      "(layout_from_segments(..., allow_wide=True))")
         if block_n > BLOCK_N:
             raise ValueError(f"tiles of {block_n} keys: the kernel takes at most {BLOCK_N}")
         self.block_n = block_n
@@ -136,10 +140,13 @@ def combine_splits(o, m, l, G: int):
     return out, lse
 
 
-def attend(q, lay: QVLayout, q_pos0: int, scale: float, n_splits: int | None = None):
+def attend(q, lay: QVLayout, q_pos0: int, scale: float, n_splits: int | None = None,
+           num_warps: int = 4, num_stages: int = 1, block_m: int | None = None):
     """q: (MQ, Hq, D) bf16 / fp16 queries at positions q_pos0 .. q_pos0 + MQ - 1.  Returns (o (MQ, Hq, D) fp32, lse
     (MQ, Hq) fp32) over the banded keys with position <= the query's; rows without a visible key get lse = -inf
-    (fused_attn.py:246-316)."""
+    (fused_attn.py:246-316).  num_warps / num_stages / block_m are the reference's tuning knobs of its other kernel;
+    they are accepted and have no meaning here."""
+    del num_warps, num_stages, block_m
     mq, hq, d = q.shape
     hkv = lay.ki.shape[1]
     g = hq // hkv
