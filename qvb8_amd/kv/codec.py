@@ -81,6 +81,38 @@ class BandedKV:
         return BandedKV(self.packed[:nbytes].clone(), self.min_s, self.tau_s, self.bits, (n_rows, hd), self.orig_dtype, self.tau)
 
 
+    def take_rows(self, rows: torch.Tensor) -> "BandedKV":
+        """Only the given token rows (indices inside 0..seq-1), not re-quantised: the ids are unpacked, selected and
+        packed again at the same width with the same constants (codec.py:141-158)."""
+        seq, hd = self.orig_shape
+        rows = rows.to(torch.int64)
+        if rows.numel() == 0 or int(rows.min()) < 0 or int(rows.max()) >= seq:
+            raise ValueError(f"take_rows indices must lie in 0..{seq - 1} and be non-empty")
+        if rows.numel() == seq and bool((rows == torch.arange(seq, device=rows.device)).all()):
+            return self
+        kept = self.ids()[rows.to(self.packed.device)]
+        return BandedKV(pack_ids(kept.reshape(-1), self.bits), self.min_s, self.tau_s, self.bits, (int(rows.numel()), hd),
+                        self.orig_dtype, self.tau)
+
+    def decode_all(self) -> torch.Tensor:
+        return self.decode_all_torch("cpu", torch.float32)
+
+    def decode_row(self, row_idx: int) -> torch.Tensor:
+        return self.decode_all()[row_idx]
+
+    outlier_count = property(lambda s: 0)           # minimum and maximum cover every value: there are no escapes
+    outlier_ratio = property(lambda s: 0.0)
+
+
+def unband_kv_4d(banded: list, batch: int, heads: int, device="cpu") -> torch.Tensor:
+    """(batch, heads, seq, head_dim) in the cache's dtype from one BandedKV per head (codec.py:252-262)."""
+    if not banded:
+        return torch.empty(batch, heads, 0, 0, device=device)
+    seq, dim = banded[0].orig_shape
+    mats = [bk.decode_all_torch(device, banded[0].orig_dtype) for bk in banded]
+    return torch.stack(mats, dim=0).reshape(batch, heads, seq, dim)
+
+
 def band_kv_heads(t: torch.Tensor, orig_dtype: torch.dtype, bits: int, tau: float = 0.0, certify: bool = True) -> list:
     """(heads, seq, head_dim) -> one BandedKV per head (codec.py:175-241).  With certify and tau > 0, `bits` is a floor:
     a head's width rises (to 16 at most) until the decoder's own expression, rounded to `orig_dtype`, is within tau of

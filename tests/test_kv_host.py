@@ -84,3 +84,21 @@ def test_layout_and_tile_table_from_segments():
 def test_split_planner_rules():
     assert FA.rows_per_workgroup(6, 256) == 16 and FA.rows_per_workgroup(24, 256) == 32 and FA.rows_per_workgroup(96, 256) == 32
     assert FA.rows_per_workgroup(96, 128) == 64 and FA.rows_per_workgroup(17, 128) == 32
+
+
+def test_take_rows_and_unband_keep_every_value():
+    torch.manual_seed(8)
+    x = torch.randn(2, 30, 16).to(torch.bfloat16)
+    heads = C.band_kv_heads(x, torch.bfloat16, 6, tau=0.1)
+    full = C.unband_kv_4d(heads, 1, 2)
+    assert full.shape == (1, 2, 30, 16) and full.dtype == torch.bfloat16
+    assert float((full[0].float() - x.float()).abs().max()) <= 0.1
+    rows = torch.tensor([0, 3, 4, 29])
+    sub = heads[0].take_rows(rows)
+    assert sub.orig_shape == (4, 16) and sub.bits == heads[0].bits and sub.min_s is heads[0].min_s
+    assert torch.equal(sub.decode_all(), heads[0].decode_all()[rows])          # the same values, bit for bit
+    assert torch.equal(heads[0].decode_row(3), heads[0].decode_all()[3])
+    assert heads[0].take_rows(torch.arange(30)) is heads[0] and heads[0].outlier_count == 0
+    with pytest.raises(ValueError):
+        heads[0].take_rows(torch.tensor([30]))
+    assert C.unband_kv_4d([], 1, 2).shape == (1, 2, 0, 0)
