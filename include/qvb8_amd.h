@@ -269,7 +269,10 @@ int qvb8_attn_fwd(const void* q, int64_t sq_r, int64_t sq_h, const void* ki, con
  * and w_s = exp(m_s - top):  total = sum_s l_s w_s,  out = sum_s o_s w_s / max(total, 1e-30),
  * lse = top + log(total) when total > 0, else -inf.  o / m / l as qvb8_attn_fwd writes them; out (tokens, q heads,
  * head_dim) and lse (tokens, q heads) f32 contiguous, row r of kv head h going to token r / G, q head h * G + r % G.
- * head_dim a multiple of 4; o and out 16-byte aligned.  Replaces the torch expressions of attend  kv/fused_attn.py:302-316. */
+ * head_dim a multiple of 4; o and out 16-byte aligned.  l may be null: every l_s is then 1, which merges NORMALISED partial
+ * results by their log-sum-exp (m = lse_s) -- the banded part and the dense residual of a layer, or the blocks of a
+ * tiered cache (_merge_lse / _merge_lse_all  kv/fused_attn.py:769-788; n_kv_heads = 1, G = n_rows keeps the row order).
+ * Replaces the torch expressions of attend  kv/fused_attn.py:302-316. */
 int qvb8_attn_combine(const float* o, const float* m, const float* l, int64_t n_splits, int64_t n_kv_heads,
                       int64_t n_rows, int64_t head_dim, int64_t G, float* out, float* lse, void* stream);
 

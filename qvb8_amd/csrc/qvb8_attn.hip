@@ -386,7 +386,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
     f4_t acc = {0.f, 0.f, 0.f, 0.f};
     for (int s = grp; s < n_splits; s += 64) {
         const float w = expf(m[s * stride + hr] - top);
-        total += l[s * stride + hr] * w;
+        total += (l ? l[s * stride + hr] : 1.f) * w;
         if (ch < D) acc += *reinterpret_cast<const f4_t*>(o + (s * stride + hr) * D + ch) * w;
     }
     if (cl == 0) s_total[grp] = total;
@@ -479,7 +479,7 @@ extern "C" int qvb8_attn_combine(const float* o, const float* m, const float* l,
                           (long long)n_kv_heads, (long long)n_rows, (long long)G, (long long)head_dim);
     if (n_rows % G != 0) return host::fail(-1, "%s: %lld rows are not whole tokens of %lld heads", who, (long long)n_rows, (long long)G);
     if (n_rows == 0) return 0;
-    if (!o || !m || !l || !out || !lse) return host::fail(-1, "%s: null pointer", who);
+    if (!o || !m || !out || !lse) return host::fail(-1, "%s: null pointer", who);
     if (!aligned(o, 16) || !aligned(out, 16)) return host::fail(-1, "%s: o and out must be 16-byte aligned", who);
     if (n_kv_heads * n_rows > INT32_MAX || n_splits > INT32_MAX) return host::fail(-1, "%s: size beyond what one launch takes", who);
     hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)(n_kv_heads * n_rows), (unsigned)((head_dim + 15) / 16)), dim3(256), 0, static_cast<hipStream_t>(stream),

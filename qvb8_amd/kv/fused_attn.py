@@ -140,6 +140,28 @@ def combine_splits(o, m, l, G: int):
     return out, lse
 
 
+def merge_lse_all(o, lse):
+    """n normalised partial results o (n, ..., D) with their log-sum-exps lse (n, ...) -> (merged result, merged lse), one
+    launch (fused_attn.py:769-778: the banded part and the dense residual of a layer, the blocks of a tiered cache)."""
+    n, d = o.shape[0], o.shape[-1]
+    rows = lse[0].numel()
+    oc = o.to(torch.float32).contiguous()
+    mc = lse.to(torch.float32).contiguous()
+    out = torch.empty(o.shape[1:], dtype=torch.float32, device=o.device)
+    lse_out = torch.empty(lse.shape[1:], dtype=torch.float32, device=o.device)
+    lib = _lib.load()
+    with torch.cuda.device(o.device):
+        rc = lib.qvb8_attn_combine(oc.data_ptr(), mc.data_ptr(), None, n, 1, rows, d, max(rows, 1), out.data_ptr(), lse_out.data_ptr(),
+                                   torch.cuda.current_stream().cuda_stream)
+    _lib._check(rc, lib)
+    return out, lse_out
+
+
+def merge_lse(o1, lse1, o2, lse2):
+    """Two partial results (fused_attn.py:781-788)."""
+    return merge_lse_all(torch.stack([o1, o2]), torch.stack([lse1, lse2]))
+
+
 def attend(q, lay: QVLayout, q_pos0: int, scale: float, n_splits: int | None = None,
            num_warps: int = 4, num_stages: int = 1, block_m: int | None = None):
     """q: (MQ, Hq, D) bf16 / fp16 queries at positions q_pos0 .. q_pos0 + MQ - 1.  Returns (o (MQ, Hq, D) fp32, lse

@@ -329,3 +329,39 @@ def test_query_preparation_is_the_callers_expression():
             assert torch.equal(out.view(torch.int16)[~torch.isnan(want)], want.view(torch.int16)[~torch.isnan(want)])
             assert torch.equal(torch.isnan(out), torch.isnan(want))
     assert lib.qvb8_scale_sat_half(None, 0, 4, 1.0, None, None) != 0 and lib.qvb8_scale_sat_half(None, 0, 0, 1.0, None, None) == 0
+
+
+def test_merge_by_log_sum_exp_is_attention_over_the_union():
+    """Attention over two halves of a cache, merged by their log-sum-exps, equals attention over the whole; a part that
+    saw no key (lse = -inf) drops out; the formulas of the reference's merge give the same numbers."""
+    torch.manual_seed(9)
+    Hkv, G, D, MQ = 2, 3, 128, 2
+    parts = []
+    for sl in (70, 45):
+        k = C.band_kv_heads((torch.randn(Hkv, sl, D, device=DEV) * 2).to(torch.bfloat16), torch.bfloat16, 6)
+        v = C.band_kv_heads(torch.randn(Hkv, sl, D, device=DEV).to(torch.bfloat16), torch.bfloat16, 6)
+        parts.append((k, v, sl))
+    whole = FA.layout_from_segments([p[0] for p in parts], [p[1] for p in parts], [p[2] for p in parts], DEV)
+    first = FA.layout_from_segments([parts[0][0]], [parts[0][1]], [70], DEV)
+    second = FA.layout_from_segments([parts[1][0]], [parts[1][1]], [45], DEV)
+    q = torch.randn(MQ, Hkv * G, D, device=DEV).to(torch.bfloat16)
+    scale = D ** -0.5
+    o_all, l_all = FA.attend(q, whole, 115 - MQ, scale)
+    o1, l1 = FA.attend(q, first, 115 - MQ, scale)
+    o2, l2 = FA.attend(q, second, 45 - MQ, scale)             # positions relative to the second part's first key
+    o, l = FA.merge_lse(o1, l1, o2, l2)
+    assert o.shape == o_all.shape and l.shape == l_all.shape
+    assert float((o - o_all).abs().max()) <= 2e-3 * float(whole.vmin.abs().max() + 32 * whole.vstep.max())
+    assert float((l - l_all).abs().max()) <= 2e-3
+    # the reference's expressions
+    m = torch.maximum(l1, l2)
+    w1, w2 = torch.exp(l1 - m), torch.exp(l2 - m)
+    assert torch.allclose(o, (o1 * w1[..., None] + o2 * w2[..., None]) / (w1 + w2)[..., None], rtol=1e-5, atol=1e-6)
+    assert torch.allclose(l, m + torch.log(w1 + w2), rtol=1e-6, atol=1e-5)
+    # a part without a visible key
+    o0, l0 = FA.attend(q, second, -5, scale)
+    assert torch.isneginf(l0).all()
+    o, l = FA.merge_lse_all(torch.stack([o1, o0, o2]), torch.stack([l1, l0, l2]))
+    assert float((o - o_all).abs().max()) <= 2e-3 * float(whole.vmin.abs().max() + 32 * whole.vstep.max())
+    on, ln = FA.merge_lse(o0, l0, o0, l0)
+    assert torch.isneginf(ln).all() and (on == 0).all()
