@@ -249,8 +249,9 @@ def test_combine_matches_the_oracle():
         assert np.all(got.cpu().numpy()[0, 0] == 0)
 
 
-@pytest.mark.parametrize("D,bits,wide", [(128, 6, False), (256, 8, False), (128, 11, True), (256, 9, True)])
-def test_restored_keys_and_values_are_the_oracles_bits(D, bits, wide):
+@pytest.mark.parametrize("D,bits,wide,shift", [(128, 6, False, 0.0), (256, 8, False, 0.0), (128, 11, True, 0.0), (256, 9, True, 0.0),
+                                               (256, 6, False, 0.3), (128, 5, False, -7.0)])
+def test_restored_keys_and_values_are_the_oracles_bits(D, bits, wide, shift):
     """Read the kernel's restored K and V back, bit for bit: every key is a tile and a split of its own, so a split's
     p is exp(0) = 1 and its output row IS the restored V of that key, and with a one-hot query its running maximum IS
     one restored K element (1.0 * k, alone in an fp32 sum)."""
@@ -259,6 +260,9 @@ def test_restored_keys_and_values_are_the_oracles_bits(D, bits, wide):
     lay["ts"] = np.arange(n, dtype=np.int32)
     lay["tl"] = np.ones(n, np.int32)
     lay["tseg"] = (np.arange(n) >= 20).astype(np.int32)
+    # id centres other than (2^B - 1) / 2 as well: moved by an integer, moved by 0.3
+    lay["kc"] = (lay["kc"] + np.float32(shift)).astype(np.float32)
+    lay["vc"] = (lay["vc"] - np.float32(shift)).astype(np.float32)
     dl = to_device(lay, wide=wide)
     G = 16
     K = np.zeros((n, Hkv, D), np.float32)
