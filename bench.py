@@ -400,7 +400,11 @@ def bench_attn(args, dev):
             segs_k.append(KC.band_kv_heads(k, torch.bfloat16, 6, certify=False))
             segs_v.append(KC.band_kv_heads(v, torch.bfloat16, 6, certify=False))
             seg_len.append(sl)
-        lays.append(FA.layout_from_segments(segs_k, segs_v, seg_len, dev))
+        lay = FA.layout_from_segments(segs_k, segs_v, seg_len, dev)
+        if args.head_major:                                  # the same ids, every kv head's keys contiguous in memory
+            lay.ki = lay.ki.permute(1, 0, 2).contiguous().permute(1, 0, 2)
+            lay.vi = lay.vi.permute(1, 0, 2).contiguous().permute(1, 0, 2)
+        lays.append(lay)
     lay0 = lays[0]
     rows = MQ * G
     tps, n_splits = FA.plan_splits(lay0.n_tiles, hkv, rows, dev, d=D)
@@ -436,8 +440,8 @@ def bench_attn(args, dev):
             "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "fp16 restored keys and values, fp32 accumulate", "data": "synthetic",
             "config": {"workload": "attention of %d query token(s), 24 heads over %d kv heads x %d channels, %d keys as 6-bit ids "
-                                   "in bytes in segments of %d, %d layers with their own caches, %d splits of %d tiles"
-                                   % (MQ, hkv, D, n, seg, len(lays), n_splits, tps),
+                                   "in bytes in segments of %d, %d layers with their own caches, %d splits of %d tiles%s"
+                                   % (MQ, hkv, D, n, seg, len(lays), n_splits, tps, ", head-major ids" if args.head_major else ""),
                        "bytes_per_launch": nbytes, "us_per_layer": round(ms * 1e3 / len(lays), 2)},
             "roofline": {"bound": "hbm", "achieved": round(gbs_kernel, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs_kernel / HBM_PEAK_GBS, 4),
@@ -497,6 +501,8 @@ def main():
                          "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256); "
                          "lmhead / embed: the 248320 x 5120 vocabulary table; attn: decode-step attention over a banded KV cache")
     ap.add_argument("--context", type=int, default=32768, help="keys in the cache of the attn workload")
+    ap.add_argument("--head-major", action="store_true",
+                    help="attn workload: ids stored (kv heads, keys, channels) instead of the reference's (keys, kv heads, channels)")
     ap.add_argument("--head-dim", type=int, default=256, choices=(128, 256), help="channels per head of the attn workload")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
     ap.add_argument("--model", choices=("9b", "27b"), default="9b",
