@@ -37,19 +37,30 @@ def sources() -> list[str]:
 
 
 def build(verbose: bool = True) -> str:
+    """Compiles every source to an object (in parallel, one hipcc each) and links them into the library."""
+    from concurrent.futures import ThreadPoolExecutor
     os.makedirs(LIB_DIR, exist_ok=True)
+    obj_dir = os.path.join(LIB_DIR, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    common = [hipcc_path(), f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-sanitize", *DEVICE_FLAGS,
+              "-I", os.path.join(os.path.dirname(HERE), "include")]
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        out = "\n".join(l for l in r.stdout.splitlines() if "is not a recognized feature" not in l)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed ({r.returncode}):\n{out}")
+        if verbose and out.strip():
+            print(out)
+
+    srcs = sources()
+    objs = [os.path.join(obj_dir, os.path.basename(s) + ".o") for s in srcs]
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        list(pool.map(lambda so: run([*common, "-c", so[0], "-o", so[1]]), zip(srcs, objs)))
     tmp = LIB_PATH + ".tmp"
-    cmd = [hipcc_path(), f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
-           "-fno-gpu-sanitize", *DEVICE_FLAGS, "-I", os.path.join(os.path.dirname(HERE), "include"),
-           "-o", tmp, *sources()]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in r.stdout.splitlines() if "is not a recognized feature" not in l)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({r.returncode}):\n{out}")
-    if verbose and out.strip():
-        print(out)
+    run([hipcc_path(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-sanitize", "-o", tmp, *objs])
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
 

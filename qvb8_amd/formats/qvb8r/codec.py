@@ -114,27 +114,40 @@ def encode_ids(ids: np.ndarray, *, n_classes: int | None = None, rows_per_tile: 
     if ids.ndim != 2 or ids.shape[1] % 128 != 0 or ids.shape[0] == 0:
         raise QVB8RFormatError("qvb8r: ids must be (Q, P) with P % 128 == 0 and Q > 0")
     Q, P = ids.shape
-    ids = ids.astype(np.int64)
-    lo, hi = ids.min(1), ids.max(1)
-    med = np.median(ids, 1).astype(np.int64)
+    # row statistics and the symbols, a block of rows at a time (the temporaries of a whole 200-million-id tensor at once
+    # would be gigabytes)
+    RB = max(1, (1 << 22) // P)
+    lo, hi, med = np.zeros(Q, np.int64), np.zeros(Q, np.int64), np.zeros(Q, np.int64)
+    for r in range(0, Q, RB):
+        blk = ids[r:r + RB].astype(np.int32)
+        lo[r:r + RB], hi[r:r + RB] = blk.min(1), blk.max(1)
+        med[r:r + RB] = np.median(blk, 1).astype(np.int64)
     drow = med - CENTRE
     drow = np.where(lo - drow < 0, lo, drow)              # symbols must not be negative
     if np.any(hi - drow >= MAX_ID) or np.any(np.abs(drow) > 32767):
         raise QVB8RFormatError("qvb8r: a row's ids span more than 2048 symbols: keep this tensor as QVB8")
-    sym_orig = (ids - drow[:, None]).astype(np.int16)
-    N = int(sym_orig.max()) + 1
+    sym_orig = np.empty((Q, P), np.int16)
+    spread = np.zeros(Q, np.float64)
+    for r in range(0, Q, RB):
+        blk = ids[r:r + RB].astype(np.int32) - drow[r:r + RB, None].astype(np.int32)
+        sym_orig[r:r + RB] = blk
+        spread[r:r + RB] = blk.astype(np.float64).std(1)
+    N = int((hi - drow).max()) + 1
     # classes: rows of similar spread share a frequency table
     K = n_classes if n_classes is not None else (1 if Q < 64 else min(8, max(1, Q // 256)))
     K = max(1, min(K, Q))
-    spread = sym_orig.astype(np.float64).std(1)
     order = np.argsort(spread, kind="stable")
     cls_of_sorted = (np.arange(Q) * K) // Q               # equal-size groups along the sorted spread
     perm = order.astype(np.int32)                         # sorted row -> original row
     sym = sym_orig[order]
+    del sym_orig
     F = np.zeros((K, N), np.int64)
     for k in range(K):
-        rows_k = sym[cls_of_sorted == k]
-        F[k] = quantise_frequencies(np.bincount(rows_k.reshape(-1).astype(np.int64), minlength=N))
+        rows_k = np.nonzero(cls_of_sorted == k)[0]
+        hist = np.zeros(N, np.int64)
+        for r in range(0, len(rows_k), RB):
+            hist += np.bincount(sym[rows_k[r]:rows_k[min(r + RB, len(rows_k)) - 1] + 1].reshape(-1), minlength=N)
+        F[k] = quantise_frequencies(hist)
     C = np.concatenate([np.zeros((K, 1), np.int64), np.cumsum(F, 1)[:, :-1]], 1)
     T = rows_per_tile if rows_per_tile is not None else max(1, ROWS_PER_TILE_DIV // P)
     tiles = []

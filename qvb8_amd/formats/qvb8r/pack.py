@@ -13,7 +13,7 @@ def transcode(enc: dict, *, n_classes: int | None = None, rows_per_tile: int | N
     if "ids_dense" not in enc:
         raise ValueError("transcode needs the unpacked ids: encode_tensor(..., keep_ids=True)")
     Q, P = int(enc["Q"]), int(enc["P"])
-    ids = enc["ids_dense"].cpu().numpy().astype(np.int64)
+    ids = enc["ids_dense"].cpu().numpy()
     r = codec.encode_ids(ids, n_classes=n_classes, rows_per_tile=rows_per_tile)
     min_s = enc["min_s"].cpu().numpy().astype(np.float32)
     tau_s = enc["tau_s"].cpu().numpy().astype(np.float32)
@@ -21,7 +21,7 @@ def transcode(enc: dict, *, n_classes: int | None = None, rows_per_tile: int | N
     esc_val = enc["esc_vals_bf16"].cpu().numpy().astype(np.float32)
     q, c = esc_idx // P, esc_idx % P
     # exact - fp32 band value, the band value with ONE rounding (fused multiply-add), via float64: id * tau_s is exact there
-    band = (ids[q, c].astype(np.float64) * tau_s[q].astype(np.float64) + min_s[q].astype(np.float64)).astype(np.float32)
+    band = (ids[q, c].astype(np.int64).astype(np.float64) * tau_s[q].astype(np.float64) + min_s[q].astype(np.float64)).astype(np.float32)
     esc_delta = (esc_val - band).astype(np.float32)
     cert = dict(tau=float(enc["tau"]), max_err=float(enc["max_err"]), restore=enc["restore"], source=enc["source"])
     d = dict(r, Q=Q, P=P, PB=codec.PB, cert=cert, min_s=min_s, tau_s=tau_s, esc_idx=esc_idx, esc_val=esc_val, esc_delta=esc_delta)

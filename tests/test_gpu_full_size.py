@@ -79,6 +79,35 @@ def test_qvb8r_restore_equals_qvb8_restore_at_27b_shape():
     assert bool(((y - ref).abs() <= tol).all())
 
 
+@pytest.mark.parametrize("Q,P", [(28672, 8192), (8192, 28672)])
+def test_qvb8r_at_the_65b_shapes(Q, P):
+    """The large-dense configuration at its full shapes (hidden 8192, FFN 28672, tau = 2e-3): the walk gives back the
+    encoder's ids, the restore equals the QVB8 restore of the same ids, the certificate holds, and the products of 1 and
+    16 rows equal dense restore + float64 matmul."""
+    from qvb8_amd import ext_qvb8r
+    from qvb8_amd.formats.qvb8r import pack as RP
+    from qvb8_amd.formats.qvb8r.module import QVBandLinearV8R
+    W = _weight(Q, P, seed=Q // 7 + P)
+    enc = PK.encode_tensor(W, 2e-3, keep_ids=True)
+    lin = QVBandLinearV8R(RP.transcode(enc), device=DEV)
+    assert torch.equal(ext_qvb8r.ids(P, *lin._core(), T=lin.T), enc["ids_dense"])
+    w32 = lin.dense(torch.float32)
+    assert torch.equal(w32, ext.decode_f32(*_args(enc)))
+    w16 = lin.dense(torch.float16)
+    assert torch.equal(w16, ext.decode(*_args(enc)))
+    max_err, bad = ext.certify(w16, W, 2e-3)
+    assert bad == 0 and max_err < 2e-3
+    del w16, W
+    w64 = w32.double()
+    wn = w64.norm(dim=1)[None, :]
+    for M in (1, 16):
+        x = torch.randn(M, P, device=DEV, generator=torch.Generator(device=DEV).manual_seed(M)).to(torch.bfloat16)
+        y = lin(x).float().double()
+        ref = x.float().double() @ w64.t()
+        tol = (1e-3 + 2.0 ** -8) * ref.abs() + 1e-3 * wn * x.float().double().norm(dim=1)[:, None] / np.sqrt(P)
+        assert bool(((y - ref).abs() <= tol).all()), (M, float(((y - ref).abs() / tol).max()))
+
+
 @pytest.mark.parametrize("n,MQ", [(32768, 1), (32768, 3), (131072, 1)])
 def test_attention_over_a_long_banded_cache(n, MQ):
     """The benchmark's cache shape (4 kv heads x 256 channels, 24 query heads, 6-bit ids, segments of 4096 keys): the

@@ -76,6 +76,29 @@ def test_product_small_m(M, dtype):
     assert torch.equal(y, lin(x))                                             # reproducible
 
 
+@pytest.mark.parametrize("Q,P", [(12, 28672), (40, 8192)])
+def test_65b_row_lengths_against_the_oracle(Q, P):
+    """Rows as long as the large-dense configuration's (hidden 8192, FFN 28672; one row per tile there): ids and restore
+    bit for bit against the oracle's walk, the product of 1 and 16 rows against restore + float64 matmul."""
+    W, enc, d = _make(Q, P, 2e-3, seed=Q + P, force=[5, P * (Q - 1) + P - 1])
+    assert d["T"] == 1
+    lin = QVBandLinearV8R(d, device=DEV)
+    want_ids = R.ids(d)
+    assert np.array_equal(want_ids, enc["ids_dense"].cpu().numpy().astype(np.int64))
+    assert np.array_equal(ext.ids(P, *lin._core(), T=lin.T).cpu().numpy().astype(np.int64), want_ids)
+    Wr = R.reconstruct(d, enc["esc_idx"].cpu().numpy(), enc["esc_vals"].cpu().numpy())
+    assert np.array_equal(lin.dense(torch.float32).cpu().numpy().view(np.uint32), Wr.view(np.uint32))
+    assert np.array_equal(lin.dense(torch.float16).cpu().numpy().view(np.uint16), O.narrow_fp16(Wr).astype(np.float16).view(np.uint16))
+    for M in (1, 16):
+        x = torch.randn(M, P, generator=torch.Generator().manual_seed(M)).to(torch.bfloat16).to(DEV)
+        y = lin(x)
+        xs = x.float().cpu().numpy()
+        ref = O.linear_f64(xs, Wr)
+        tol = H.gemv_tolerance(ref, Wr, xs) + 2.0 ** -8 * np.abs(ref)
+        diff = np.abs(y.float().cpu().numpy().astype(np.float64) - ref)
+        assert np.all(diff <= tol), (M, float((diff / tol).max()))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_matrix_core_rows_agree_with_single_row_walk(dtype):
     """Every row of a many-row call against the one-row kernel on the same row: the two differ only in the order of the
