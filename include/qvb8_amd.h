@@ -39,7 +39,9 @@ enum qvb8_status {
 };
 
 /* Library identification: ABI version, bumped on any signature change or new entry point (3: row lookup, attention over
- * the banded KV cache, query preparation). */
+ * the banded KV cache, query preparation; 4: qvb8_moe_experts_static).  A binding compares the loaded library's answer
+ * with the QVB8_ABI_VERSION it was written for before it makes any other call. */
+#define QVB8_ABI_VERSION 4
 int qvb8_abi_version(void);
 /* Message of the calling thread's most recent failure ("" if none). Valid until that thread's next call. */
 const char* qvb8_last_error(void);
@@ -194,6 +196,24 @@ int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, const int64_t* 
                      const uint8_t* dn_ids, int64_t dn_ids_bytes, const float* dn_min, const float* dn_tau,
                      const uint8_t* dn_nb, const int64_t* dn_off, int64_t Q_dn, int64_t P_dn,
                      int act, void* out, int out_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* qvb8_moe_experts for callers that cannot allocate device memory or bring a workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  Same operands, same kernels and the same results bit for bit; the
+ * workspace is an array of QVB8_MOE_STATIC_SCRATCH_BYTES inside the library's device image (one copy per GPU, held until
+ * the process ends).  A call that would need more (qvb8_moe_workspace_bytes) fails with QVB8_ERR_WORKSPACE: 2 MiB covers
+ * 16 tokens x top-8 of a 2048 / 768 expert stack.  The call allocates and frees nothing.  All calls on one GPU share the
+ * array: calls that overlap on one GPU (two streams, two threads) race; calls in stream order do not.  The first call on a
+ * device looks the array's address up (make that call outside a stream capture).
+ * No counterpart in the reference, whose extension allocates its temporaries with torch on every call
+ * (qvb8_cuda.cu:958-960). */
+#define QVB8_MOE_STATIC_SCRATCH_BYTES (2 * 1024 * 1024)
+int qvb8_moe_experts_static(const void* X, int x_dtype, int64_t tokens, const int64_t* idx, const float* w, int64_t topk,
+                            int64_t n_experts,
+                            const uint8_t* up_ids, int64_t up_ids_bytes, const float* up_min, const float* up_tau,
+                            const uint8_t* up_nb, const int64_t* up_off, int64_t Q_up, int64_t P_up,
+                            const uint8_t* dn_ids, int64_t dn_ids_bytes, const float* dn_min, const float* dn_tau,
+                            const uint8_t* dn_nb, const int64_t* dn_off, int64_t Q_dn, int64_t P_dn,
+                            int act, void* out, int out_dtype, void* stream);
 
 /* ---- QVB8R: the same band ids, rANS-coded (32 interleaved streams per tile) ---------------------------------------- */
 

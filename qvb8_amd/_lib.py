@@ -12,13 +12,14 @@ import torch
 from .common.errors import NativeLibraryError
 
 _LIB = None
+EXPECTED_ABI = 4            # QVB8_ABI_VERSION of include/qvb8_amd.h that the argument lists below were written for
 F32, F16, BF16 = 0, 1, 2
 _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 # every symbol include/qvb8_amd.h declares
 SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_lookup_rows", "qvb8_scatter_escapes", "qvb8_certify",
            "qvb8_sat_half", "qvb8_scale_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma",
-           "qvb8_moe_workspace_bytes", "qvb8_moe_experts",
+           "qvb8_moe_workspace_bytes", "qvb8_moe_experts", "qvb8_moe_experts_static",
            "qvb8r_decode", "qvb8r_gemv_workspace_bytes", "qvb8r_gemv", "qvb8r_fix_escapes", "qvb8_attn_fwd", "qvb8_attn_combine")
 
 
@@ -36,7 +37,7 @@ def load(build_if_missing: bool = True):
         return _LIB
     path = lib_path()
     if not os.path.exists(path):
-        if not build_if_missing:
+        if not build_if_missing or os.environ.get("QVB8_AMD_LIB"):
             raise NativeLibraryError(f"{path} is missing: run `python -m qvb8_amd.build`")
         from . import build as _b
         try:
@@ -47,6 +48,11 @@ def load(build_if_missing: bool = True):
         lib = ctypes.CDLL(path)
     except OSError as ex:
         raise NativeLibraryError(f"cannot load {path}: {ex}") from None
+    lib.qvb8_abi_version.restype = ctypes.c_int
+    found = lib.qvb8_abi_version()
+    if found != EXPECTED_ABI:
+        raise NativeLibraryError(f"{path} has ABI version {found}, this binding was written for {EXPECTED_ABI}: "
+                                 "rebuild it with `python -m qvb8_amd.build`")
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     lib.qvb8_abi_version.restype = i32
     lib.qvb8_last_error.restype = ctypes.c_char_p
@@ -69,6 +75,8 @@ def load(build_if_missing: bool = True):
     lib.qvb8_moe_workspace_bytes.restype = i64
     lib.qvb8_moe_experts.argtypes = ([vp, i32, i64, vp, vp, i64, i64] + [vp, i64, vp, vp, vp, vp, i64, i64] * 2
                                      + [i32, vp, i32, vp, i64, vp])
+    lib.qvb8_moe_experts_static.argtypes = ([vp, i32, i64, vp, vp, i64, i64] + [vp, i64, vp, vp, vp, vp, i64, i64] * 2
+                                            + [i32, vp, i32, vp])
     lib.qvb8r_decode.argtypes = [vp, i64, i32, i64, i64, i64, vp, i64, vp]
     lib.qvb8r_gemv_workspace_bytes.argtypes = [i64, i64]
     lib.qvb8r_gemv_workspace_bytes.restype = i64

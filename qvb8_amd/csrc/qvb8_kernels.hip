@@ -530,7 +530,7 @@ __global__ void __launch_bounds__(256) gemv_fix_escapes_kernel(const void* __res
 // ===========================================================================================================
 using namespace qvb8;
 
-extern "C" int qvb8_abi_version(void) { return 3; }
+extern "C" int qvb8_abi_version(void) { return QVB8_ABI_VERSION; }
 extern "C" const char* qvb8_last_error(void) { return host::last_error().c_str(); }
 
 static int check_pack(const uint8_t* ids, int64_t ids_bytes, const float* min_s, const float* tau_s, const uint8_t* nbits,

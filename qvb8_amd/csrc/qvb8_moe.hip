@@ -15,6 +15,7 @@
 // sum, and the two terms joined in double: reproducible, and within rounding of  sum(x * fmaf(id, tau_s, min_s)).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <mutex>
 #include <type_traits>
 
 #include "../../include/qvb8_amd.h"
@@ -668,4 +669,49 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
     else if (out_dtype == QVB8_F16) hipLaunchKernelGGL(moe_combine_kernel<1>, grid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
     else hipLaunchKernelGGL(moe_combine_kernel<2>, grid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
     return host::check_launch("qvb8_moe_experts combine");
+}
+
+// ---- the same call for callers that cannot allocate ------------------------------------------------------------------
+// The workspace of qvb8_moe_experts (routing plan, H, Yd) as a fixed array in the device image: every GPU the library
+// runs on holds its own copy at its own address until the process ends.  Host code never uses the array's name as an
+// address (there it is only a handle for the runtime): the device address is looked up once per device.
+static __device__ __align__(256) unsigned char scratch[QVB8_MOE_STATIC_SCRATCH_BYTES];
+
+namespace {
+// device address of `scratch` on the current device, looked up on the first call there (with that device current)
+int moe_static_scratch(void** out) {
+    static void* ptr[64] = {nullptr};
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_moe_experts_static: no current device");
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return host::fail(QVB8_ERR_LAUNCH, "qvb8_moe_experts_static: cannot find the scratch array on device %d: %s", dev, hipGetErrorString(e));
+        ptr[dev] = p;
+    }
+    *out = ptr[dev];
+    return QVB8_OK;
+}
+}  // namespace
+
+extern "C" int qvb8_moe_experts_static(const void* X, int x_dtype, int64_t tokens, const int64_t* idx, const float* w, int64_t topk, int64_t n_experts,
+                                       const uint8_t* up_ids, int64_t up_ids_bytes, const float* up_min, const float* up_tau,
+                                       const uint8_t* up_nb, const int64_t* up_off, int64_t Q_up, int64_t P_up,
+                                       const uint8_t* dn_ids, int64_t dn_ids_bytes, const float* dn_min, const float* dn_tau,
+                                       const uint8_t* dn_nb, const int64_t* dn_off, int64_t Q_dn, int64_t P_dn,
+                                       int act, void* out, int out_dtype, void* stream) {
+    const int64_t need = qvb8_moe_workspace_bytes(tokens, topk, n_experts, Q_up, P_dn, Q_dn);
+    if (need > (int64_t)QVB8_MOE_STATIC_SCRATCH_BYTES)
+        return host::fail(QVB8_ERR_WORKSPACE, "qvb8_moe_experts_static: this call needs %lld bytes of scratch, the built-in array holds %lld "
+                          "(fewer tokens per call, or qvb8_moe_experts with a workspace)", (long long)need, (long long)QVB8_MOE_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if (int rc = moe_static_scratch(&ws)) return rc;
+    // nothing in the workspace has to start at zero: the plan kernel writes its counter before it is read, and H and Yd
+    // are written completely before the next step reads them
+    return qvb8_moe_experts(X, x_dtype, tokens, idx, w, topk, n_experts, up_ids, up_ids_bytes, up_min, up_tau, up_nb, up_off, Q_up, P_up,
+                            dn_ids, dn_ids_bytes, dn_min, dn_tau, dn_nb, dn_off, Q_dn, P_dn, act, out, out_dtype, ws,
+                            (int64_t)QVB8_MOE_STATIC_SCRATCH_BYTES, stream);
 }

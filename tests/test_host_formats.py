@@ -143,7 +143,8 @@ def test_library_loads_and_exports_every_declared_symbol():
     for name in sorted(declared):
         assert hasattr(lib, name), name
     lib.qvb8_abi_version.restype = ctypes.c_int
-    assert lib.qvb8_abi_version() >= 1
+    m = re.search(r"#define\s+QVB8_ABI_VERSION\s+(\d+)", header)
+    assert m and lib.qvb8_abi_version() == int(m.group(1)) == _lib.EXPECTED_ABI
     lib.qvb8_last_error.restype = ctypes.c_char_p
     assert lib.qvb8_last_error() is not None
     # size queries are host-only arithmetic: callable without a GPU
