@@ -42,7 +42,8 @@ MMA_FLAGS = int(os.environ.get("QVB8_BENCH_MMA_FLAGS", "1"))     # 1 = QVB8_MMA_
 
 def algorithmic_bytes(enc, M):
     """Bytes one product has to move: packed ids, 17 bytes of row metadata per row (min_s, tau_s, nbits, bit_off), 12
-    per escape, the bf16 activations in and the bf16 results out."""
+    per escape, the bf16 activations in and the results counted as bf16 (2 bytes each; the timed kernel writes them as
+    fp32, 4 bytes each, which is more than is counted here -- 0.03 % of a projection's bytes)."""
     ids = enc["ids"] if "ids" in enc else enc["ids_host"]
     return int(ids.numel() + 17 * enc["Q"] + 12 * enc["esc_idx"].numel() + 2 * M * enc["P"] + 2 * M * enc["Q"])
 
@@ -187,16 +188,22 @@ def bench_moe(args, dev):
     x = torch.randn(T, hidden, device=dev, generator=torch.Generator(device=dev).manual_seed(7)).to(torch.bfloat16)
     out = torch.empty(T, hidden, dtype=torch.bfloat16, device=dev)
     ws = torch.empty(lib.qvb8_moe_workspace_bytes(T, k, E, 2 * inter, inter, hidden), dtype=torch.uint8, device=dev)
-    routes, step_bytes = [], 0
-    for g_, d_ in stacks:
-        idx, w = synthetic_routing(rng.normal(size=(T, E)), k)
-        routes.append((torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)))
-        per_expert = (g_["ids"].numel() + d_["ids"].numel()) // E + 17 * (g_["Q"] + d_["Q"])
-        step_bytes += len(np.unique(idx)) * per_expert + 2 * T * hidden * 2
+    # Every layer is called with several routings in turn (each its own random draw), until a step touches more than
+    # 512 MB of distinct expert bytes: a replay then cannot be served from the 256 MB last-level cache.
+    calls, step_bytes = [], 0
+    per_expert = (stacks[0][0]["ids"].numel() + stacks[0][1]["ids"].numel()) // E + 17 * (stacks[0][0]["Q"] + stacks[0][1]["Q"])
+    rounds = 0
+    while step_bytes < (512 << 20) and rounds < 16:
+        for g_, d_ in stacks:
+            idx, w = synthetic_routing(rng.normal(size=(T, E)), k)
+            calls.append((g_, d_, torch.from_numpy(idx).to(dev), torch.from_numpy(w).to(dev)))
+            step_bytes += len(np.unique(idx)) * per_expert + 2 * T * hidden * 2
+        rounds += 1
+    n_calls = len(calls)
 
     def step():
         s = torch.cuda.current_stream().cuda_stream
-        for (g_, d_), (idx, w) in zip(stacks, routes):
+        for g_, d_, idx, w in calls:
             rc = lib.qvb8_moe_experts(x.data_ptr(), 2, T, idx.data_ptr(), w.data_ptr(), k, E,
                                       g_["ids"].data_ptr(), g_["ids"].numel(), g_["min_s"].data_ptr(), g_["tau_s"].data_ptr(),
                                       g_["nbits"].data_ptr(), g_["bit_off"].data_ptr(), g_["Q"], g_["P"],
@@ -208,28 +215,33 @@ def bench_moe(args, dev):
     ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
     ms = max(ev_ms, wall_ms)
     gbs = step_bytes / (ms * 1e-3) / 1e9
-    per_layer_us = ev_ms * 1e3 / args.layers
+    per_layer_us = ev_ms * 1e3 / n_calls
     return {"metric": "expert-gathered fused decode-GEMV GB/s on the bytes of the unique selected experts, 35B-A3B-shape MoE "
                       "layer, 1 MI355X",
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16 activations narrowed to fp16 x fp32 band value, fp32 accumulate", "data": "synthetic",
             "config": {"workload": "MoE layer: hidden 2048, 128 experts gate/up 2048->768 + down 768->2048, top-8, QVB8 "
-                                   "tau=2e-3, %d token(s), %d layers" % (T, args.layers),
+                                   "tau=2e-3, %d token(s), %d layers x %d routings per step" % (T, args.layers, rounds),
                        "bytes_per_step": step_bytes, "us_per_layer": round(per_layer_us, 2)},
             "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                          "kernel": ("qvb8::moe_one_kernel<4,false,..> + moe_one_kernel<6,true,..> (one layer = 2 launches)" if T <= 16 else
                                     "qvb8::moe_plan_kernel + moe_gemv_kernel<0> + moe_gemv_kernel<1> + moe_combine_kernel "
                                     "(one layer = 4 launches)"),
-                         "bytes_per_launch": step_bytes // args.layers, "launch_us": round(per_layer_us, 3)},
+                         "bytes_per_launch": step_bytes // n_calls, "launch_us": round(per_layer_us, 3)},
             "cpu_baseline": None}
 
 
-def bench_qvb8r(args, dev):
-    """Config 5 (27B-class shapes): hidden 5120, FFN 17408, QVB8R at tau = 2e-3, `--tokens` rows (1..48).  A step = gate,
-    up (17408 x 5120) and down (5120 x 17408) of `--layers` layers through qvb8r_gemv; bytes = coded words + states +
-    slot tables + row metadata."""
+QVB8R_SHAPES = {"27b": ("hidden 5120 / FFN 17408 (gate, up, down)", ((17408, 5120), (17408, 5120), (5120, 17408))),
+                "65b": ("hidden 8192 / FFN 28672 (up 8192->28672, down 28672->8192)", ((28672, 8192), (8192, 28672)))}
+
+
+def bench_qvb8r(args, dev, token_counts=None):
+    """Config 5: large-dense shapes as QVB8R at tau = 2e-3, `--tokens` rows (1..48): `--model 65b` (default here) hidden 8192 /
+    FFN 28672, `--model 27b` hidden 5120 / FFN 17408.  A step = the shapes' tensors of `--layers` layers through
+    qvb8r_gemv; bytes = coded words + states + slot tables + row metadata.  With `token_counts` the packs are built once
+    and one result per token count is returned."""
     import ctypes
     import torch
     from qvb8_amd import _lib, ext_qvb8r
@@ -237,21 +249,33 @@ def bench_qvb8r(args, dev):
     from qvb8_amd.formats.qvb8r import pack as RP
     from qvb8_amd.formats.qvb8r.module import QVBandLinearV8R
     lib = _lib.load()
-    M = args.tokens
-    units, step_bytes, n_sym = [], 0, 0
+    shape_name, shapes = QVB8R_SHAPES[args.model if args.model in QVB8R_SHAPES else "65b"]
+    units, coded_bytes, n_sym = [], 0, 0
     for l in range(args.layers):
-        for pi, (Q, P) in enumerate(((17408, 5120), (17408, 5120), (5120, 17408))):
+        for pi, (Q, P) in enumerate(shapes):
             g = torch.Generator(device=dev).manual_seed(5000 + 10 * l + pi)
             W = (0.02 * torch.randn(Q, P, device=dev, generator=g)).to(torch.bfloat16)
             d = RP.transcode(PK.encode_tensor(W, 2e-3, keep_ids=True))
             del W
             lin = QVBandLinearV8R(d, device=dev)
             core, _, _ = ext_qvb8r._core(*lin._core(), P)
-            x = torch.randn(M, P, device=dev, generator=g).to(torch.bfloat16)
-            units.append(dict(lin=lin, core=core, x=x, Y=torch.empty(M, Q, dtype=torch.float32, device=dev),
-                              ws=torch.empty(lib.qvb8r_gemv_workspace_bytes(M, P), dtype=torch.uint8, device=dev)))
-            step_bytes += 4 * len(d["words"]) + 8 * 32 * len(d["tiles"]) + 4 * 4096 * d["K"] + 12 * Q + 8 * Q + 2 * M * (P + Q)
+            units.append(dict(lin=lin, core=core, Q=Q, P=P, seed=5000 + 10 * l + pi))
+            coded_bytes += 4 * len(d["words"]) + 8 * 32 * len(d["tiles"]) + 4 * 4096 * d["K"] + 12 * Q + 8 * Q
             n_sym += Q * P
+            del d
+    results = [_time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name) for M in (token_counts or [args.tokens])]
+    return results if token_counts else results[0]
+
+
+def _time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name):
+    import ctypes
+    import torch
+    step_bytes = coded_bytes + sum(2 * M * (u["P"] + u["Q"]) for u in units)
+    for u in units:
+        g = torch.Generator(device=dev).manual_seed(u["seed"])
+        u["x"] = torch.randn(M, u["P"], device=dev, generator=g).to(torch.bfloat16)
+        u["Y"] = torch.empty(M, u["Q"], dtype=torch.float32, device=dev)
+        u["ws"] = torch.empty(lib.qvb8r_gemv_workspace_bytes(M, u["P"]), dtype=torch.uint8, device=dev)
 
     def step():
         s = torch.cuda.current_stream().cuda_stream
@@ -265,12 +289,12 @@ def bench_qvb8r(args, dev):
     gbs = step_bytes / (ms * 1e-3) / 1e9
     launch_us = ev_ms * 1e3 / len(units)
     kernel = "qvb8::r_gemv_kernel<2>" if M == 1 else "qvb8::r_mma_kernel<%d, false> (+ r_pack_x_kernel)" % ((M + 15) // 16)
-    return {"metric": "QVB8R fused entropy-decode + GEMV GB/s on coded bytes, 27B-class FFN shapes, 1 MI355X",
+    return {"metric": "QVB8R fused entropy-decode + GEMV GB/s on coded bytes, large-dense FFN shapes, 1 MI355X",
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16 activations x fp32 band value (M > 1: exact fp16 operands on the matrix cores), fp32 accumulate",
             "data": "synthetic",
-            "config": {"workload": "QVB8R tau=2e-3, hidden 5120 / FFN 17408 (gate, up, down), M=%d, %d layers" % (M, args.layers),
+            "config": {"workload": "QVB8R tau=2e-3, %s, M=%d, %d layers" % (shape_name, M, args.layers),
                        "bytes_per_step": step_bytes, "bits_per_weight": round(8.0 * step_bytes / n_sym, 3),
                        "symbols_per_s": round(n_sym / (ms * 1e-3), 1)},
             "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -451,13 +475,17 @@ def bench_attn(args, dev):
             "cpu_baseline": None}
 
 
-def bench_smallm(args, dev):
+def bench_smallm(args, dev, prebuilt=None, tokens=None):
     """Config 3: the 9B projections with M = `--tokens` rows (draft-verify / prefill chunk), through QVBandLinearV8's own
     dispatch: M <= 48 the tile kernel (X in registers), 49..256 the workgroup-tiled decode + GEMM kernel (X staged in LDS,
     ids decoded in registers), above that dense restore to fp16 + library GEMM.  Reports GB/s on the packed bytes and TFLOP/s (2 M Q P per projection, decode ops not counted)."""
     import torch
-    layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse)
-    M = args.tokens
+    if prebuilt is None:
+        layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse)
+    else:
+        layers, units = prebuilt
+    n_layers = len(layers)
+    M = args.tokens if tokens is None else tokens
     g = torch.Generator(device=dev).manual_seed(7)
     x_by_p = {P: torch.randn(M, P, device=dev, generator=g).to(torch.bfloat16) for P in (4096, 12288)}
     flat = [enc for lay in layers for enc in lay]
@@ -480,7 +508,7 @@ def bench_smallm(args, dev):
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16 activations, fp32 accumulate, bf16 out", "data": "synthetic", "tflops": round(tflops, 3),
-            "config": {"workload": "9B-shape projections, QVB8 tau=1e-3, M=%d, %d layers, path: %s" % (M, args.layers, path),
+            "config": {"workload": "9B-shape projections, QVB8 tau=1e-3, M=%d, %d layers, path: %s" % (M, n_layers, path),
                        "bytes_per_step": step_bytes, "flops_per_step": flops, "launch_units": len(units)},
             "roofline": ({"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
@@ -488,6 +516,40 @@ def bench_smallm(args, dev):
                          {"bound": "mfma", "achieved": round(tflops, 3), "peak": 2500.0, "unit": "TFLOP/s",
                           "frac": round(tflops / 2500.0, 5), "traffic": None}),
             "cpu_baseline": None}
+
+
+def run_legs(args, dev, layers, units):
+    """Short runs of the other configurations, each on its own synthetic packs, appended to the headline's line under
+    `legs`: the 9B projections with 16 / 64 / 256 rows (the first 8 layers of the headline's packs), the 35B-A3B-shape MoE
+    layer with 1 and 8 tokens, the 65B-shape QVB8R pair with 1 and 16 rows.  Each entry: value, unit, ms_per_step,
+    roofline, config (and tflops for the small-M legs)."""
+    import copy
+    import gc
+    import torch
+    keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "tflops", "dtype", "roofline", "config")
+    legs = {}
+    sub = copy.copy(args)
+    sub.steps, sub.warmup = max(5, min(args.steps, 20)), 3
+    n8 = min(8, len(layers))
+    per_layer = len(units) // len(layers)
+    for M in (16, 64, 256):
+        r = bench_smallm(sub, dev, prebuilt=(layers[:n8], units[:n8 * per_layer]), tokens=M)
+        legs["smallm_M%d" % M] = {k: r[k] for k in keep if k in r}
+    layers.clear()
+    units.clear()
+    gc.collect()
+    torch.cuda.empty_cache()
+    sub.layers = 2
+    for T in (1, 8):
+        sub.tokens = T
+        r = bench_moe(sub, dev)
+        legs["moe_T%d" % T] = {k: r[k] for k in keep if k in r}
+        gc.collect()
+        torch.cuda.empty_cache()
+    sub.layers, sub.model = 1, "65b"
+    for M, r in zip((1, 16), bench_qvb8r(sub, dev, token_counts=[1, 16])):
+        legs["qvb8r_M%d" % M] = {k: r[k] for k in keep if k in r}
+    return legs
 
 
 def main():
@@ -505,8 +567,12 @@ def main():
                     help="attn workload: ids stored (kv heads, keys, channels) instead of the reference's (keys, kv heads, channels)")
     ap.add_argument("--head-dim", type=int, default=256, choices=(128, 256), help="channels per head of the attn workload")
     ap.add_argument("--tokens", type=int, default=1, help="token rows for the moe / qvb8r workloads")
-    ap.add_argument("--model", choices=("9b", "27b"), default="9b",
-                    help="decode9b workload only: layer shapes (9b = the headline configuration; 27b = hidden 5120, FFN 17408)")
+    ap.add_argument("--model", choices=("9b", "27b", "65b"), default="9b",
+                    help="decode9b workload: layer shapes (9b = the headline configuration; 27b = hidden 5120, FFN 17408); "
+                         "qvb8r workload: 65b (default there: hidden 8192, FFN 28672) or 27b")
+    ap.add_argument("--no-legs", action="store_true",
+                    help="decode9b workload: skip the short legs of the other configurations (small-M, MoE, QVB8R) that the "
+                         "default run appends under `legs`")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sort", action="store_true",
                     help="keep the file's row order in memory (row addresses are then read from the row records instead of "
@@ -530,7 +596,7 @@ def main():
     torch.cuda.set_device(dev)
     lib = _lib.load()                                       # raises when the HIP library is missing: no fallback
     if args.layers is None:
-        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 2, "lmhead": 1, "embed": 1, "attn": 16}[args.workload]
+        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 1, "lmhead": 1, "embed": 1, "attn": 16}[args.workload]
     if args.workload != "decode9b":
         fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead, "embed": bench_embed, "attn": bench_attn}[args.workload]
         print(json.dumps(fn(args, dev)))
@@ -538,6 +604,9 @@ def main():
     if args.no_sort:
         from qvb8_amd.formats.qvb8.module import QVBandLinearV8
         QVBandLinearV8.sort_rows = False
+    if args.model == "65b":
+        print("bench.py: --model 65b names QVB8R shapes (--workload qvb8r); the decode step takes 9b or 27b", file=sys.stderr)
+        return 2
     shapes = LAYER_27B if args.model == "27b" else LAYER_9B
     layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse, shapes=shapes)
     g = torch.Generator(device=dev).manual_seed(7)
@@ -614,6 +683,8 @@ def main():
         out["cpu_baseline"] = cpu_baseline(layers, x_by_p)
     else:
         out["cpu_baseline"] = None
+    if not args.no_legs and args.model == "9b" and not args.no_fuse:
+        out["legs"] = run_legs(args, dev, layers, units)
     print(json.dumps(out))
     return 0
 
