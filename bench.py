@@ -475,6 +475,68 @@ def bench_attn(args, dev):
             "cpu_baseline": None}
 
 
+def bench_floor(args, dev):
+    """What a launch costs on this machine.  (1) A graph of 128 launches of a kernel with the tile kernel's launch shape
+    (256 workgroups x 512 threads, 40 KB of LDS, the same scalar arguments) that does nothing: microseconds per graph
+    node.  (2) The tile kernel itself (qvb8_mma, M = 1, bf16 x) on 4096-column weights of 4096, 2048, 1024 and 512 rows,
+    128 launches per graph over distinct packs: time per launch against bytes per launch; the straight line through
+    those points gives the fixed cost per launch (its value at zero bytes) and the rate the bytes stream at beyond it."""
+    import numpy as np
+    import torch
+    from qvb8_amd import _lib
+    from qvb8_amd.formats.qvb8 import pack as PK
+    from qvb8_amd.formats.qvb8.module import QVBandLinearV8
+    lib = _lib.load()
+    n = 128
+
+    def probe_step():
+        s = torch.cuda.current_stream().cuda_stream
+        for _ in range(n):
+            if lib.qvb8_launch_probe(256, 512, 40960, s) != 0:
+                raise RuntimeError(lib.qvb8_last_error().decode())
+    ev, wall = time_graph(probe_step, args.steps, args.warmup)
+    empty_us = max(ev, wall) * 1e3 / n
+    P, points = 4096, []
+    x = torch.randn(1, P, device=dev, generator=torch.Generator(device=dev).manual_seed(1)).to(torch.bfloat16)
+    for Q in (4096, 2048, 1024, 512):
+        n_packs = max(2, min(n, (600 << 20) // (Q * P * 7 // 8)))          # distinct packs: 600 MB, beyond the last-level cache
+        units = []
+        for i in range(n_packs):
+            g = torch.Generator(device=dev).manual_seed(77 * Q + i)
+            W = (0.02 * torch.randn(Q, P, device=dev, generator=g)).to(torch.bfloat16)
+            lin = QVBandLinearV8.from_encoded(PK.encode_tensor(W, TAU, restore="fp16"))
+            perm, rowinfo, layout = lin._mma_order()
+            units.append((lin, perm, rowinfo, layout, torch.empty((1, Q), dtype=torch.float32, device=dev)))
+        nbytes = sum(int(u[0].ids.numel() + 17 * Q + 2 * P + 2 * Q) for u in units) / len(units)
+
+        def step():
+            s = torch.cuda.current_stream().cuda_stream
+            for i in range(n):
+                lin, perm, rowinfo, layout, Y = units[i % len(units)]
+                ne = lin.esc_idx.numel()
+                rc = lib.qvb8_mma(x.data_ptr(), _lib.dtype_code(x.dtype), 1, lin.ids.data_ptr(), lin.ids.numel(), lin.min_s.data_ptr(),
+                                  lin.tau_s.data_ptr(), lin.nbits.data_ptr(), lin.bit_off.data_ptr(), Q, P,
+                                  lin.esc_idx.data_ptr() if ne else None, lin.esc_vals.data_ptr() if ne else None, ne, perm.data_ptr(),
+                                  rowinfo.data_ptr(), ctypes.addressof(layout) if layout is not None else None, MMA_FLAGS,
+                                  Y.data_ptr(), None, 0, s)
+                if rc != 0:
+                    raise RuntimeError(lib.qvb8_last_error().decode())
+        ev, wall = time_graph(step, args.steps, args.warmup)
+        points.append((nbytes, max(ev, wall) * 1e3 / n))
+        del units
+    b = np.array([p[0] for p in points])
+    t = np.array([p[1] for p in points])
+    slope, intercept = np.polyfit(b, t, 1)
+    return {"metric": "cost of a launch: graph node of an empty kernel, and the tile kernel's time per launch against its bytes, 1 MI355X",
+            "value": round(empty_us, 3), "unit": "us per empty launch", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(empty_us * n * 1e-3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+            "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "128-node graphs: an empty kernel of 256 x 512 threads with 40 KB of LDS; qvb8_mma M=1 on Q x 4096 weights, Q = 4096, 2048, 1024, 512",
+                       "tile_kernel_points": [{"bytes_per_launch": int(p[0]), "us_per_launch": round(p[1], 3)} for p in points],
+                       "fixed_us_per_launch": round(float(intercept), 3), "streaming_GBs_beyond_fixed": round(1e-3 / float(slope), 1)},
+            "roofline": None, "cpu_baseline": None}
+
+
 def bench_smallm(args, dev, prebuilt=None, tokens=None):
     """Config 3: the 9B projections with M = `--tokens` rows (draft-verify / prefill chunk), through QVBandLinearV8's own
     dispatch: M <= 48 the tile kernel (X in registers), 49..256 the workgroup-tiled decode + GEMM kernel (X staged in LDS,
@@ -558,10 +620,11 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=None, help="layers of distinct packs (default 32; moe 4; qvb8r 2)")
-    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead", "embed", "attn"), default="decode9b",
+    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead", "embed", "attn", "floor"), default="decode9b",
                     help="decode9b (default, the headline metric): 9B-shape decode step; moe: 35B-A3B-shape expert stack; "
                          "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256); "
-                         "lmhead / embed: the 248320 x 5120 vocabulary table; attn: decode-step attention over a banded KV cache")
+                         "lmhead / embed: the 248320 x 5120 vocabulary table; attn: decode-step attention over a banded KV cache; "
+                         "floor: what a launch costs (empty-kernel graph, tile kernel time against bytes)")
     ap.add_argument("--context", type=int, default=32768, help="keys in the cache of the attn workload")
     ap.add_argument("--head-major", action="store_true",
                     help="attn workload: ids stored (kv heads, keys, channels) instead of the reference's (keys, kv heads, channels)")
@@ -596,9 +659,9 @@ def main():
     torch.cuda.set_device(dev)
     lib = _lib.load()                                       # raises when the HIP library is missing: no fallback
     if args.layers is None:
-        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 1, "lmhead": 1, "embed": 1, "attn": 16}[args.workload]
+        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 1, "lmhead": 1, "embed": 1, "attn": 16, "floor": 1}[args.workload]
     if args.workload != "decode9b":
-        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead, "embed": bench_embed, "attn": bench_attn}[args.workload]
+        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead, "embed": bench_embed, "attn": bench_attn, "floor": bench_floor}[args.workload]
         print(json.dumps(fn(args, dev)))
         return 0
     if args.no_sort:

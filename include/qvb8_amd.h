@@ -167,6 +167,12 @@ int qvb8_mma(const void* X, int x_dtype, int64_t M,
              const int32_t* perm, const uint64_t* rowinfo, const qvb8_mma_layout* layout, int flags, float* Y,
              void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Measurement aid: launches a kernel of the matrix-core path's launch shape (blocks x threads, lds_bytes of dynamic LDS,
+ * the same 56 bytes of scalar arguments) that does nothing.  A graph of such launches gives the cost of a launch on this
+ * machine before any byte moves, the floor under every per-launch figure of the benchmark (bench.py --workload floor).
+ * No counterpart in the reference. */
+int qvb8_launch_probe(int64_t blocks, int64_t threads, int64_t lds_bytes, void* stream);
+
 /* ---- routed MoE expert stack (decode: a few tokens, top-k experts each) ---------------------------------------- */
 
 enum qvb8_moe_act {

@@ -132,10 +132,12 @@ __device__ __forceinline__ uint32_t pair_spread(uint32_t e) {                   
     }
     return r;
 }
-__device__ __forceinline__ uint32_t and_or3(uint32_t t, uint32_t mask, uint32_t bias) {   // (t & mask) | bias
-    uint32_t r;
-    asm("v_bitop3_b32 %0, %1, %2, %3 bitop3:0xea" : "=v"(r) : "v"(t), "v"(mask), "v"(bias));
-    return r;
+// Written in C on purpose: the result is an MFMA operand, and the compiler keeps the wait states between a vector
+// instruction's write and the matrix instruction that reads it only for instructions it can see.  As an inline-asm
+// instruction the same operation was invisible to that check: an operand written two instructions before its MFMA was
+// read stale (measured: the register's previous contents entered the product).
+__device__ __forceinline__ uint32_t and_or3(uint32_t t, uint32_t mask, uint32_t bias) {   // (t & mask) | bias: v_and_or_b32
+    return (t & mask) | bias;
 }
 
 // The lane's NB dwords, 4-byte aligned.

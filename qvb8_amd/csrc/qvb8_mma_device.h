@@ -99,8 +99,12 @@ __device__ __forceinline__ void decode_slice(const uint4& lo, const uint4& hi, v
     constexpr uint32_t mask = ((1u << KEEP) - 1u) * 0x00010001u;
     uint32_t e[16];
     slice_pairs<NB>(lo, hi, e);
+    // the two constants as registers (opaque to constant folding): the last step is then ONE v_and_or_b32 per pair, a
+    // real instruction of the compiler's, so that it keeps the wait states the matrix instruction needs after it
+    uint32_t m = mask, bias = Fmt<BF>::bias_bits;
+    asm("" : "+v"(m), "+v"(bias));
 #pragma unroll
-    for (int p = 0; p < 16; ++p) b[p / 4][p % 4] = and_or3(e[p], mask, Fmt<BF>::bias_bits);
+    for (int p = 0; p < 16; ++p) b[p / 4][p % 4] = and_or3(e[p], m, bias);
 }
 
 }  // namespace qvb8

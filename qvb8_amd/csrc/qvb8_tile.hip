@@ -800,6 +800,30 @@ int launch_gemm(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_
 }
 }  // namespace
 
+// A kernel of the tile kernel's launch shape (grid, workgroup size, dynamic LDS, 56 bytes of scalar arguments) that does
+// nothing: what a launch costs before it moves a byte.
+__global__ void __launch_bounds__(512) launch_probe_kernel(const uint16_t* X, const uint8_t* ids, const uint64_t* loc, float* Y, int64_t ids_bytes,
+                                                           int Q, int P, uint32_t counts, int TW, int first1, int first2, uint32_t widths) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (Q < 0) Y[threadIdx.x] = (float)(smem[threadIdx.x] + X[0] + ids[0] + loc[0] + ids_bytes + P + counts + TW + first1 + first2 + widths);
+}
+
+extern "C" int qvb8_launch_probe(int64_t blocks, int64_t threads, int64_t lds_bytes, void* stream) {
+    if (blocks < 1 || blocks > 65535 || threads < 64 || threads > 512 || (threads & 63) || lds_bytes < 0 || lds_bytes > (int64_t)kLdsPerWorkgroup)
+        return host::fail(QVB8_ERR_ARG, "qvb8_launch_probe: 1..65535 workgroups of 64..512 threads (whole waves), at most 160 KB of LDS");
+    static bool attr[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_launch_probe: no current device");
+    if (!attr[dev]) {
+        if (hipFuncSetAttribute((const void*)launch_probe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup) != hipSuccess)
+            return host::fail(QVB8_ERR_LAUNCH, "qvb8_launch_probe: cannot raise the kernel's LDS limit");
+        attr[dev] = true;
+    }
+    hipLaunchKernelGGL(launch_probe_kernel, dim3((unsigned)blocks), dim3((unsigned)threads), (size_t)lds_bytes, (hipStream_t)stream,
+                       nullptr, nullptr, nullptr, nullptr, (int64_t)0, 1, 1, 0u, 1, 1, 1, 0u);
+    return host::check_launch("qvb8_launch_probe");
+}
+
 extern "C" int64_t qvb8_mma_rowinfo_bytes(int64_t Q) { return Q > 0 ? (int64_t)(rowinfo_loc_words(Q) * 8 + (size_t)Q * 16) : 0; }
 
 extern "C" int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, const float* tau_s, const float* min_s,
@@ -916,7 +940,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     // with four (measured on 27B-class shapes: 16 % faster; more steps per wave did not pay for longer rows)
     const int n_steps_all = (int)(P / kStepCols);
 #define QVB8_TILE_LAUNCH_ROWS16(T_) (mode == 0 ? launch_tile_rows16<T_, false, false>(a, s) : mode == 1 ? launch_tile_rows16<T_, false, true>(a, s) : launch_tile_rows16<T_, true, false>(a, s))
-    if (M <= 16) rc = n_steps_all > 32 && n_steps_all <= 40 ? QVB8_TILE_LAUNCH_ROWS16(5) : QVB8_TILE_LAUNCH_ROWS16(4);
+        if (M <= 16) rc = n_steps_all > 32 && n_steps_all <= 40 ? QVB8_TILE_LAUNCH_ROWS16(5) : QVB8_TILE_LAUNCH_ROWS16(4);
 #undef QVB8_TILE_LAUNCH_ROWS16
     else if (M <= 32) rc = QVB8_TILE_LAUNCH(2, 2);
     else rc = QVB8_TILE_LAUNCH(3, 2);

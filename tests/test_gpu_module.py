@@ -152,7 +152,7 @@ def test_same_input_fusion_is_bit_identical():
     assert blk.self_attn._qvb8_fused._x is None           # every member took its part: nothing is held
 
 
-@pytest.mark.parametrize("widths,sortable", [([7, 6, 9], True), ([5], True), ([7, 6, 9, 3, 8, 5], False)])
+@pytest.mark.parametrize("widths,sortable", [([7, 6, 9], True), ([5], True), ([4], True), ([8, 4], True), ([7, 6, 9, 3, 8, 5], False)])
 def test_rows_copied_into_width_order(widths, sortable):
     """The module copies its rows once into width-sorted order and then lets the kernel compute row addresses (at most
     three widths; other packs keep the row records).  Either way results match the oracle and the dense restore is
