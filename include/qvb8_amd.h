@@ -247,6 +247,15 @@ typedef struct qvb8r_core {
 int qvb8r_decode(const qvb8r_core* core, int64_t max_tile_rows, int out_dtype, int64_t b0, int64_t nb, int64_t row_base,
                  void* out, int64_t out_rows, void* stream);
 
+/* The rows of a LIST of blocks (block numbers of the schedule in `core`, i32 in device memory, any order, repeats
+ * allowed): block j of the list fills rows [j * 8 * max_tile_rows, (j + 1) * 8 * max_tile_rows) of `out`, row r of the
+ * block's tile h at row (j * 8 + h) * max_tile_rows + r; slots of tiles the block does not have, or rows a tile does not
+ * have, are left untouched.  out_dtype as qvb8r_decode; out has out_rows >= n_list * 8 * max_tile_rows rows of P.  A block
+ * number outside the schedule writes nothing.  What a lookup of scattered rows (an embedding read) gathers from.
+ * Replaces the per-row walk of embed_rows  qvb8r_cpu.cpp:13-51 (there on the CPU, one tile prefix per looked-up row). */
+int qvb8r_decode_blocks(const qvb8r_core* core, int64_t max_tile_rows, int out_dtype, const int32_t* block_list,
+                        int64_t n_list, void* out, int64_t out_rows, void* stream);
+
 /* Bytes of workspace qvb8r_gemv needs: 16 for M = 1 (X is read in place); for M = 2..48 the activations packed as
  * fp16 hi + lo planes in matrix-core operand order plus one sum and one scale exponent per row. */
 int64_t qvb8r_gemv_workspace_bytes(int64_t M, int64_t P);

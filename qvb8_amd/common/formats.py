@@ -4,9 +4,9 @@
     spec = get_format(manifest["format"])
     lin  = spec.linear.from_packfile(path, device=dev)
 
-Entries: "qvb8" / "qvband" (the container's file extension) and "qvb8r".  There is no CPU reader in this build and no
-embedding class for "qvb8r" (`cpu_linear`, its `embedding` are None): a caller that needs one gets a clear error from
-`require`, never another format's class.
+Entries: "qvb8" / "qvband" (the container's file extension) and "qvb8r", each with its linear and embedding class and
+its `finalize` hook (same-input fusion).  There is no CPU reader in this build (`cpu_linear` is None): a caller that
+needs one gets a clear error from `require`, never another format's class.
 """
 from __future__ import annotations
 
@@ -42,14 +42,17 @@ def _build_registry() -> None:
     from qvb8_amd.formats.qvb8.embedding import QVBandEmbeddingV8
     from qvb8_amd.formats.qvb8.fuse import fuse_same_input
     from qvb8_amd.formats.qvb8.module import QVBandLinearV8
-    from qvb8_amd.formats.qvb8r.module import QVBandLinearV8R
+    from qvb8_amd.formats.qvb8r.fuse import fuse_same_input as fuse_same_input_r
+    from qvb8_amd.formats.qvb8r.module import QVBandEmbeddingV8R, QVBandLinearV8R
 
     def _decode_v8(lin):
         return ext.decode(lin.ids, lin.min_s, lin.nbits, lin.bit_off, lin.in_features, lin.tau_s, lin.esc_idx, lin.esc_vals)
 
     _REGISTRY["qvb8"] = FormatSpec("qvb8", QVBandLinearV8, QVBandEmbeddingV8, QVBandExpertsV8, decoder=_decode_v8, finalize=fuse_same_input)
     _REGISTRY["qvband"] = dataclasses.replace(_REGISTRY["qvb8"], name="qvband")
-    _REGISTRY["qvb8r"] = FormatSpec("qvb8r", QVBandLinearV8R, None, None, decoder=lambda lin: lin.dense(torch.float32))
+    # no expert reader for qvb8r: expert stacks of such a pack directory stay dense (as in the reference's registry)
+    _REGISTRY["qvb8r"] = FormatSpec("qvb8r", QVBandLinearV8R, QVBandEmbeddingV8R, None, decoder=lambda lin: lin.dense(torch.float32),
+                                    finalize=fuse_same_input_r)
 
 
 def get_format(name: str | None) -> FormatSpec:

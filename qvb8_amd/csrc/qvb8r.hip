@@ -133,12 +133,20 @@ __device__ __forceinline__ TileCtx block_setup(const RCore& c, int block, uint32
 // ---- dense rows -----------------------------------------------------------------------------------------------------
 // DT: 0 fp32, 1 fp16, 2 bf16 values; 3 the ids as int16.  row_base < 0: a row is written at its ORIGINAL index;
 // row_base >= 0: at its sorted position - row_base (a contiguous block range fills a compact chunk of out_rows rows).
+// `list` (or null): workgroup j walks block list[j] instead of block b0 + j and writes row r of the block's tile h at row
+// (j * 8 + h) * T + r of `out` (a fixed slot per tile: what a lookup of scattered rows gathers from).
 template <int DT>
-__global__ void __launch_bounds__(kRThreads) r_decode_kernel(RCore c, int b0, int64_t row_base, int64_t out_rows, void* __restrict__ out, int T) {
+__global__ void __launch_bounds__(kRThreads) r_decode_kernel(RCore c, int b0, int64_t row_base, int64_t out_rows, void* __restrict__ out, int T,
+                                                             const int32_t* __restrict__ list) {
     __shared__ uint32_t st[4096];
     __shared__ uint32_t ring[kRTiles][kRing];
     const int lane = threadIdx.x & 63, l32 = lane & 31, half = lane >> 5, h8 = threadIdx.x >> 5;
-    TileCtx t = block_setup(c, b0 + blockIdx.x, st, h8);
+    int block_no = b0 + (int)blockIdx.x;
+    if (list) {
+        block_no = list[blockIdx.x];
+        if (block_no < 0 || block_no >= c.n_blocks) return;                   // the whole workgroup: a bad entry writes nothing
+    }
+    TileCtx t = block_setup(c, block_no, st, h8);
     uint32_t* rg = ring[h8];
     Walker z;
     walk_init(z, rg, c, t.tile, l32);
@@ -151,7 +159,7 @@ __global__ void __launch_bounds__(kRThreads) r_decode_kernel(RCore c, int b0, in
         const bool row_ok = orow >= 0 && orow < c.Q;
         const float m = row_ok ? c.min_s[orow] : 0.f, ts = row_ok ? c.tau_s[orow] : 0.f;
         const int dr = row_ok ? c.drow[orow] : 0;
-        const int64_t at = row_base < 0 ? (int64_t)orow : (int64_t)(t.r0 + r) - row_base;
+        const int64_t at = list ? ((int64_t)blockIdx.x * kRTiles + h8) * T + r : row_base < 0 ? (int64_t)orow : (int64_t)(t.r0 + r) - row_base;
         const bool store = row_ok && at >= 0 && at < out_rows;
         for (int s0 = 0; s0 < S; s0 += 2) {
             uint32_t s1, s2;
@@ -445,12 +453,35 @@ extern "C" int qvb8r_decode(const qvb8r_core* core, int64_t max_tile_rows, int o
     dim3 grid((unsigned)nb), block(kRThreads);
     const int T = (int)max_tile_rows;
     switch (out_dtype) {
-        case 0: hipLaunchKernelGGL(r_decode_kernel<0>, grid, block, 0, s, c, (int)b0, row_base, out_rows, out, T); break;
-        case 1: hipLaunchKernelGGL(r_decode_kernel<1>, grid, block, 0, s, c, (int)b0, row_base, out_rows, out, T); break;
-        case 2: hipLaunchKernelGGL(r_decode_kernel<2>, grid, block, 0, s, c, (int)b0, row_base, out_rows, out, T); break;
-        default: hipLaunchKernelGGL(r_decode_kernel<3>, grid, block, 0, s, c, (int)b0, row_base, out_rows, out, T); break;
+        case 0: hipLaunchKernelGGL(r_decode_kernel<0>, grid, block, 0, s, c, (int)b0, row_base, out_rows, out, T, (const int32_t*)nullptr); break;
+        case 1: hipLaunchKernelGGL(r_decode_kernel<1>, grid, block, 0, s, c, (int)b0, row_base, out_rows, out, T, (const int32_t*)nullptr); break;
+        case 2: hipLaunchKernelGGL(r_decode_kernel<2>, grid, block, 0, s, c, (int)b0, row_base, out_rows, out, T, (const int32_t*)nullptr); break;
+        default: hipLaunchKernelGGL(r_decode_kernel<3>, grid, block, 0, s, c, (int)b0, row_base, out_rows, out, T, (const int32_t*)nullptr); break;
     }
     return host::check_launch("qvb8r_decode");
+}
+
+extern "C" int qvb8r_decode_blocks(const qvb8r_core* core, int64_t max_tile_rows, int out_dtype, const int32_t* block_list, int64_t n_list,
+                                   void* out, int64_t out_rows, void* stream) {
+    RCore c;
+    if (int rc = check_core("qvb8r_decode_blocks", core, c)) return rc;
+    if (out_dtype < 0 || out_dtype > 3) return host::fail(QVB8_ERR_ARG, "qvb8r_decode_blocks: out_dtype must be 0 (fp32), 1 (fp16), 2 (bf16) or 3 (ids)");
+    if (max_tile_rows < 1 || max_tile_rows > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8r_decode_blocks: bad rows-per-tile bound");
+    if (n_list < 0 || n_list > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8r_decode_blocks: bad list length");
+    if (n_list == 0) return QVB8_OK;
+    if (!block_list || !out) return host::fail(QVB8_ERR_ARG, "qvb8r_decode_blocks: null pointer");
+    if (out_rows < n_list * kRTiles * max_tile_rows)
+        return host::fail(QVB8_ERR_ARG, "qvb8r_decode_blocks: out needs %lld rows (blocks x 8 tiles x rows per tile)", (long long)(n_list * kRTiles * max_tile_rows));
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid((unsigned)n_list), block(kRThreads);
+    const int T = (int)max_tile_rows;
+    switch (out_dtype) {
+        case 0: hipLaunchKernelGGL(r_decode_kernel<0>, grid, block, 0, s, c, 0, (int64_t)0, out_rows, out, T, block_list); break;
+        case 1: hipLaunchKernelGGL(r_decode_kernel<1>, grid, block, 0, s, c, 0, (int64_t)0, out_rows, out, T, block_list); break;
+        case 2: hipLaunchKernelGGL(r_decode_kernel<2>, grid, block, 0, s, c, 0, (int64_t)0, out_rows, out, T, block_list); break;
+        default: hipLaunchKernelGGL(r_decode_kernel<3>, grid, block, 0, s, c, 0, (int64_t)0, out_rows, out, T, block_list); break;
+    }
+    return host::check_launch("qvb8r_decode_blocks");
 }
 
 extern "C" int64_t qvb8r_gemv_workspace_bytes(int64_t M, int64_t P) {

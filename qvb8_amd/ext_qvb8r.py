@@ -97,6 +97,25 @@ def decode(words, off, states, tiles, blocks, tab, perm, mn, ts, drow, P, out_dt
     return W
 
 
+def decode_blocks(block_list, words, off, states, tiles, blocks, tab, perm, mn, ts, drow, P, out_dtype=3, T=None):
+    """Rows of the listed blocks (int32 GPU tensor of block numbers) in fixed slots: row r of tile h of list entry j at
+    row (j * 8 + h) * T + r of the result, (len(list) * 8 * T, P).  out_dtype 0 fp16 / 1 bf16 / 2 fp32 band values (escapes
+    not applied), 3 the ids as int16.  Slots without a row are left as allocated (not initialised)."""
+    lib = _lib.load()
+    _lib.require_cuda(block_list)
+    if block_list.dtype != torch.int32 or not block_list.is_contiguous():
+        raise RuntimeError("qvb8r: block_list must be a contiguous int32 GPU tensor")
+    c, Q, _ = _core(words, off, states, tiles, blocks, tab, perm, mn, ts, drow, P)
+    Tb = _rows_bound(tiles, T)
+    dt = torch.int16 if int(out_dtype) == 3 else _OUT[int(out_dtype)]
+    n = block_list.numel()
+    with torch.cuda.device(mn.device):
+        W = torch.empty((n * 8 * Tb, int(P)), dtype=dt, device=mn.device)
+        _lib._check(lib.qvb8r_decode_blocks(ctypes.byref(c), Tb, _ABI_DT[dt], block_list.data_ptr(), n, W.data_ptr(), W.shape[0],
+                                            _lib.stream_of(mn)), lib)
+    return W
+
+
 def ids(P, words, off, states, tiles, blocks, tab, perm, mn, ts, drow, T=None):
     """The band ids (Q, P) int16 in original row order (qvb8r_cuda.cu:426-444)."""
     lib = _lib.load()

@@ -13,14 +13,9 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
+from qvb8_amd.common.fusion import SAME_INPUT_GROUPS, FusedGroup as _FusedGroup, FusedMember, fuse_groups  # noqa: F401
 from .module import QVBandLinearV8
 
-# (parent attribute, sibling names) whose members are fed the same tensor by the model's forward (fuse.py:17-21)
-SAME_INPUT_GROUPS = (
-    ("self_attn", ("q_proj", "k_proj", "v_proj")),
-    ("linear_attn", ("in_proj_qkv", "in_proj_z")),
-    ("mlp", ("gate_proj", "up_proj")),
-)
 _ALIGN = 16
 
 
@@ -72,69 +67,21 @@ def concat_linears(mods: list[QVBandLinearV8]) -> tuple[QVBandLinearV8, list[int
     return fused, splits
 
 
-class FusedGroup(nn.Module):
-    """One launch for linears that read the same input: the first member called computes every member's output."""
+class FusedGroup(_FusedGroup):
+    """The fused launch of a group of QVBandLinearV8 (members in the order given)."""
 
     def __init__(self, mods: list[QVBandLinearV8]):
-        super().__init__()
-        self.lin, self.splits = concat_linears(mods)
-        self._x = None
-        self._ver = None
-        self._outs = None
-        self._left: set = set()
-
-    def forward(self, x):
-        """All members' outputs for `x`, as views of one result."""
-        return torch.tensor_split(self.lin(x), self.splits, -1)
-
-    def get(self, x, i):
-        # Reuse only for the SAME tensor object, unmodified, and only until every member has taken its part once
-        # (fuse.py:64-77).  Python-side reuse is not valid under graph replay: capture forward() instead.
-        if self._x is not x or x._version != self._ver or i not in self._left:
-            self._outs = self.forward(x)
-            self._x, self._ver = x, x._version
-            self._left = set(range(len(self._outs)))
-        self._left.discard(i)
-        out = self._outs[i]
-        if not self._left:
-            self._x = self._outs = None
-        return out
+        lin, splits = concat_linears(mods)
+        super().__init__(lin, splits)
 
 
-class FusedMember(nn.Module):
-    def __init__(self, group: FusedGroup, i: int, in_features: int, out_features: int):
-        super().__init__()
-        object.__setattr__(self, "group", group)       # shared by the members: kept out of the module tree
-        self.i, self.in_features, self.out_features = i, in_features, out_features
-        self.bias = None                                # the fused linear adds the members' biases itself
-
-    def forward(self, x):
-        return self.group.get(x, self.i)
-
-    def extra_repr(self):
-        return f"in_features={self.in_features}, out_features={self.out_features}, fused member {self.i}"
+def _all_packed(owner, names) -> bool:
+    mods = [getattr(owner, a, None) for a in names]
+    return (all(isinstance(m, QVBandLinearV8) for m in mods) and len({m.in_features for m in mods}) == 1
+            and not any(m.fp16_table_missing for m in mods))
 
 
 def fuse_same_input(model: nn.Module) -> int:
     """Replace every same-input group of QVBandLinearV8 siblings by members of one fused launch; returns the number of
-    groups fused.  The separate modules are dropped before the next group is built, so at most one group exists twice."""
-    n = 0
-    owners = [(owner, names) for parent in model.modules() for sub, names in SAME_INPUT_GROUPS
-              if (owner := getattr(parent, sub, None)) is not None
-              and all(isinstance(getattr(owner, a, None), QVBandLinearV8) for a in names)
-              and len({getattr(owner, a).in_features for a in names}) == 1
-              and not any(getattr(owner, a).fp16_table_missing for a in names)]
-    for owner, names in owners:
-        mods = [getattr(owner, a) for a in names]
-        meta = [(m.in_features, m.out_features) for m in mods]
-        g = FusedGroup(mods)
-        del mods
-        for a in names:
-            setattr(owner, a, None)
-        owner._qvb8_fused = g                           # registered once, under the shared owner
-        for i, (a, (pin, pout)) in enumerate(zip(names, meta)):
-            setattr(owner, a, FusedMember(g, i, pin, pout))
-        n += 1
-    if n and torch.cuda.is_available():
-        torch.cuda.empty_cache()
-    return n
+    groups fused.  The fused linear adds the members' biases itself."""
+    return fuse_groups(model, _all_packed, concat_linears, "_qvb8_fused")

@@ -12,6 +12,7 @@ Slot tables, the block schedule and the read-ahead pad are derived at load (runt
 from __future__ import annotations
 
 import json
+import struct
 import zlib
 
 import numpy as np
@@ -26,27 +27,46 @@ _DTYPES = dict(perm="<i4", freq="<u2", tiles="<i4", tile_off="<u4", states="<u8"
                min_s="<f4", tau_s="<f4", esc_idx="<i8", esc_val="<f4", esc_delta="<f4")
 
 
+_PREFIX = struct.Struct("<4sII")          # magic, version, length of the header text
+
+
+def _up64(n: int) -> int:
+    return (n + 63) & ~63
+
+
+def _place(meta: dict, arrays: list) -> tuple[bytes, dict]:
+    """Where every array goes.  The table of offsets is part of the header text, and the first array starts behind that
+    text: the table is recomputed from the text's length until it no longer changes (the file format's own rule)."""
+    table: dict = {}
+    while True:
+        text = json.dumps(dict(meta, arrays=table)).encode()
+        cursor, proposal = _up64(_PREFIX.size + len(text)), {}
+        for name, a in arrays:
+            proposal[name] = [cursor, a.dtype.str, list(a.shape)]
+            cursor = _up64(cursor + a.nbytes)
+        if proposal == table:
+            return text, table
+        table = proposal
+
+
 def to_bytes(enc: dict, Q: int, P: int, min_s, tau_s, esc_idx, esc_val, esc_delta, cert: dict) -> bytes:
-    """The file's bytes (container.py:30-49): `enc` is what codec.encode_ids returns."""
-    src = dict(enc, min_s=min_s, tau_s=tau_s, esc_idx=esc_idx, esc_val=esc_val, esc_delta=esc_delta)
-    arrs = {k: np.ascontiguousarray(np.asarray(src[k]).astype(_DTYPES[k])) for k in ARRAYS}
-    hdr = dict(Q=int(Q), P=int(P), T=int(enc["T"]), K=int(enc["K"]), N=int(enc["N"]), PB=PB, cert=cert, arrays={})
-    while True:                                            # offsets depend on the header's own length: until stable
-        hj = json.dumps(hdr).encode()
-        pos = (12 + len(hj) + 63) // 64 * 64
-        for k, a in arrs.items():
-            hdr["arrays"][k] = [pos, a.dtype.str, list(a.shape)]
-            pos = (pos + a.nbytes + 63) // 64 * 64
-        if json.dumps(hdr).encode() == hj:
-            break
-    buf = bytearray(MAGIC + np.uint32(VERSION).tobytes() + np.uint32(len(hj)).tobytes() + hj)
-    for k, a in arrs.items():
-        off = hdr["arrays"][k][0]
-        buf += b"\0" * (off - len(buf))
-        buf += a.tobytes()
-    buf += b"\0" * ((len(buf) + 63) // 64 * 64 - len(buf))
-    buf += np.uint32(zlib.crc32(buf)).tobytes()
-    return bytes(buf)
+    """The bytes of a .qvb8r file for the arrays codec.encode_ids returned plus the row metadata and escapes of the QVB8
+    pack (the reference's writer: container.py:30-49; the same bytes for the same input)."""
+    given = dict(enc, min_s=min_s, tau_s=tau_s, esc_idx=esc_idx, esc_val=esc_val, esc_delta=esc_delta)
+    arrays = [(name, np.ascontiguousarray(np.asarray(given[name]).astype(_DTYPES[name]))) for name in ARRAYS]
+    meta = dict(Q=int(Q), P=int(P), T=int(enc["T"]), K=int(enc["K"]), N=int(enc["N"]), PB=PB, cert=cert)
+    text, table = _place(meta, arrays)
+    last_name, last = arrays[-1]
+    body_end = _up64(table[last_name][0] + last.nbytes)
+    out = bytearray(body_end + 4)                                     # zero-filled: every gap is padding already
+    _PREFIX.pack_into(out, 0, MAGIC, VERSION, len(text))
+    out[_PREFIX.size:_PREFIX.size + len(text)] = text
+    view = memoryview(out)
+    for name, a in arrays:
+        at = table[name][0]
+        view[at:at + a.nbytes] = a.reshape(-1).view(np.uint8).data
+    struct.pack_into("<I", out, body_end, zlib.crc32(view[:body_end]))
+    return bytes(out)
 
 
 def write(path: str, enc: dict, Q: int, P: int, min_s, tau_s, esc_idx, esc_val, esc_delta, cert: dict) -> int:
@@ -57,34 +77,45 @@ def write(path: str, enc: dict, Q: int, P: int, min_s, tau_s, esc_idx, esc_val, 
 
 
 def read(path: str | None = None, blob: bytes | None = None) -> dict:
-    """Header fields + arrays (numpy views into the file bytes); QVB8RFormatError on a bad file (container.py:52-71)."""
-    raw = blob if blob is not None else open(path, "rb").read()
-    where = path or "<blob>"
-    if len(raw) < 16 or raw[:4] != MAGIC:
-        raise QVB8RFormatError(f"{where}: not a .qvb8r file")
-    ver = int(np.frombuffer(raw, "<u4", 1, 4)[0])
-    if ver != VERSION:
-        raise QVB8RFormatError(f"{where}: .qvb8r version {ver}, this reader knows {VERSION}"
-                               + (" (re-transcode the pack from its QVB8 form)" if ver < VERSION else ""))
-    if zlib.crc32(memoryview(raw)[:-4]) != int(np.frombuffer(raw, "<u4", 1, len(raw) - 4)[0]):
-        raise QVB8RFormatError(f"{where}: crc32 mismatch (truncated or corrupt file)")
-    hl = int(np.frombuffer(raw, "<u4", 1, 8)[0])
+    """The header's fields and every array (numpy views of the file's bytes) as one dict; QVB8RFormatError names what is
+    wrong with a file that cannot be used (reference reader: container.py:52-71)."""
+    if blob is None:
+        with open(path, "rb") as fh:
+            blob = fh.read()
+    name = path if path else "<bytes>"
+    data = memoryview(blob)
+    if len(data) < _PREFIX.size + 4:
+        raise QVB8RFormatError(f"{name}: {len(data)} bytes is too short for a .qvb8r file")
+    magic, version, text_len = _PREFIX.unpack_from(data, 0)
+    if magic != MAGIC:
+        raise QVB8RFormatError(f"{name}: starts with {bytes(magic)!r}, a .qvb8r file starts with {MAGIC!r}")
+    if version != VERSION:
+        hint = "; older files must be transcoded again from the QVB8 pack" if version < VERSION else ""
+        raise QVB8RFormatError(f"{name}: file format version {version}, supported is {VERSION}{hint}")
+    body = len(data) - 4
+    (stored_crc,) = struct.unpack_from("<I", data, body)
+    if zlib.crc32(data[:body]) != stored_crc:
+        raise QVB8RFormatError(f"{name}: checksum does not match the contents (file damaged or cut short)")
+    if _PREFIX.size + text_len > body:
+        raise QVB8RFormatError(f"{name}: header of {text_len} bytes does not fit the file")
     try:
-        hdr = json.loads(bytes(raw[12:12 + hl]))
-    except ValueError as ex:
-        raise QVB8RFormatError(f"{where}: unreadable header ({ex})") from None
-    if hdr.get("PB") != PB:
-        raise QVB8RFormatError(f"{where}: PB {hdr.get('PB')} != {PB}")
-    out = dict(hdr)
-    for k, (off, dt, shape) in hdr["arrays"].items():
-        n = int(np.prod(shape)) if shape else 1
-        if off < 0 or off + n * np.dtype(dt).itemsize > len(raw) - 4:
-            raise QVB8RFormatError(f"{where}: array {k} lies outside the file")
-        out[k] = np.frombuffer(raw, np.dtype(dt), n, off).reshape(shape)
-    missing = [k for k in ARRAYS if k not in out]
-    if missing:
-        raise QVB8RFormatError(f"{where}: arrays missing: {missing}")
-    return out
+        fields = json.loads(bytes(data[_PREFIX.size:_PREFIX.size + text_len]))
+        table = fields["arrays"]
+    except (ValueError, KeyError, TypeError) as why:
+        raise QVB8RFormatError(f"{name}: header cannot be parsed ({why})") from None
+    if fields.get("PB") != PB:
+        raise QVB8RFormatError(f"{name}: coded with {fields.get('PB')}-bit probabilities, this reader handles {PB}")
+    absent = [k for k in ARRAYS if k not in table]
+    if absent:
+        raise QVB8RFormatError(f"{name}: header lists no {', '.join(absent)}")
+    result = dict(fields)
+    for key, (start, type_str, shape) in table.items():
+        dt = np.dtype(type_str)
+        count = int(np.prod(shape)) if shape else 1
+        if start < 0 or start + count * dt.itemsize > body:
+            raise QVB8RFormatError(f"{name}: '{key}' ({count} x {dt}) at byte {start} runs past the end of the file")
+        result[key] = np.frombuffer(blob, dt, count, start).reshape(shape)
+    return result
 
 
 def blocks_for(tiles: np.ndarray, tiles_per_block: int) -> np.ndarray:

@@ -23,7 +23,23 @@ FP32_METADATA = ("min_s", "tau_s", "esc_val", "esc_val_bf16", "esc_delta")
 
 
 def _t(a, dev):
-    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    a = np.ascontiguousarray(a)
+    return torch.from_numpy(a if a.flags.writeable else a.copy()).to(dev)
+
+
+def _apply_keeping_fp32(module: nn.Module, fn, recurse=True):
+    """nn.Module._apply that moves the fp32 decode metadata with the module but never casts it: `.to(bfloat16)` must not
+    round min_s / tau_s / escape values (module.py:162-175 of the reference)."""
+    keep = {n: module._buffers[n] for n in FP32_METADATA if module._buffers.get(n) is not None}
+    for n in keep:
+        module._buffers[n] = None
+    try:
+        out = nn.Module._apply(module, fn, recurse)
+    finally:
+        dev = module._buffers["words"].device
+        for n, b in keep.items():
+            module._buffers[n] = b.to(dev)
+    return out
 
 
 class QVBandLinearV8R(nn.Module):
@@ -34,6 +50,7 @@ class QVBandLinearV8R(nn.Module):
     def __init__(self, d: dict, bias=None, device="cuda", path: str | None = None):
         super().__init__()
         self.path = path
+        self._arrays = None if path else d               # built from arrays, not from a file: kept for host_arrays()
         tab, tiles, words, off = QF.runtime_tables(d)
         Q, P = int(d["Q"]), int(d["P"])
         self.out_features, self.in_features, self.T = Q, P, int(d["T"])
@@ -97,17 +114,20 @@ class QVBandLinearV8R(nn.Module):
             b = bias.detach() if isinstance(bias, torch.Tensor) else torch.tensor(bias)
         return cls(d, bias=b, device=device, path=path)
 
+    def has_host_arrays(self) -> bool:
+        return bool(self.path) or self._arrays is not None
+
+    def host_arrays(self) -> dict:
+        """The tensor as container.read returns it (host memory): read again from the file the module came from, or the
+        arrays it was built from.  What joining members into one fused tensor starts from."""
+        if self.path:
+            return QF.read(self.path)
+        if self._arrays is None:
+            raise RuntimeError("QVBandLinearV8R: neither a file nor the source arrays are known for this module")
+        return self._arrays
+
     def _apply(self, fn, recurse=True):
-        keep = {n: self._buffers[n] for n in FP32_METADATA if self._buffers.get(n) is not None}
-        for n in keep:
-            self._buffers[n] = None
-        try:
-            out = nn.Module._apply(self, fn, recurse)
-        finally:
-            dev = self._buffers["words"].device
-            for n, b in keep.items():
-                self._buffers[n] = b.to(dev)
-        return out
+        return _apply_keeping_fp32(self, fn, recurse)
 
     def extra_repr(self):
         return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"
@@ -182,3 +202,106 @@ class QVBandLinearV8R(nn.Module):
         if ef.numel():
             W.view(-1)[ef] = ev.to(W.dtype)
         return W.to(dtype)
+
+
+class QVBandEmbeddingV8R(nn.Module):
+    """nn.Embedding over a QVB8R tensor.  A lookup walks only the blocks (up to 8 tiles) that hold looked-up rows, on the GPU,
+    and gathers the rows from them: the table stays coded in memory.  The reference decodes the rows on the CPU, one tile
+    prefix per row, and keeps the table out of VRAM (src/qv_band/formats/qvb8r/module.py:339-395, qvb8r_cpu.cpp:13-51).
+    Value of a row: `min_s + float(id) * tau_s` as an fp32 multiply followed by an fp32 add (two roundings, as that CPU
+    code and the QVB8 embedding compute it), the row's escapes written over it, then rounded once to the output dtype."""
+
+    def __init__(self, d: dict, out_dtype=torch.bfloat16, device="cuda", path: str | None = None):
+        super().__init__()
+        self.path = path
+        tab, tiles, words, off = QF.runtime_tables(d)
+        Q, P = int(d["Q"]), int(d["P"])
+        self.num_embeddings, self.embedding_dim, self._out_dtype, self.T = Q, P, out_dtype, int(d["T"])
+        dev = torch.device(device)
+        buf = lambda name, a: self.register_buffer(name, _t(a, dev), persistent=False)
+        buf("words", words.view(np.int32)); buf("off", off)
+        buf("states", np.asarray(d["states"], np.uint64).view(np.int64)); buf("tiles", tiles)
+        buf("drow", np.asarray(d["drow"]).astype(np.int32))
+        buf("tab", tab.view(np.int32)); buf("perm", np.asarray(d["perm"], np.int32))
+        blocks8 = QF.blocks_for(tiles, WPB)
+        buf("blocks8", blocks8)
+        buf("min_s", np.asarray(d["min_s"], np.float32)); buf("tau_s", np.asarray(d["tau_s"], np.float32))
+        # original row -> slot of its decoded copy inside its block: block number and (tile in block) * T + row in tile
+        perm = np.asarray(d["perm"]).astype(np.int64)
+        sorted_pos = np.empty(Q, np.int64)
+        sorted_pos[perm] = np.arange(Q)
+        tile_of_sorted = np.repeat(np.arange(len(tiles)), tiles[:, 2])
+        block_of_tile = np.repeat(np.arange(len(blocks8)), blocks8[:, 2])
+        tile = tile_of_sorted[sorted_pos]
+        buf("row_block", block_of_tile[tile].astype(np.int32))
+        buf("row_slot", ((tile - blocks8[block_of_tile[tile], 1]) * self.T + (sorted_pos - tiles[tile, 1])).astype(np.int64))
+        # one escape table, chosen by the output dtype (module.py:356-363): the fp16 subset for fp16 output of an fp16+bf16
+        # pack (named by escape_tables.json), the file's full list otherwise; grouped by row
+        ei = np.asarray(d["esc_idx"]).astype(np.int64)
+        ev = np.asarray(d["esc_val"], np.float32)
+        cert = d.get("cert", {}) or {}
+        if out_dtype == torch.float16 and cert.get("restore") == "fp16+bf16":
+            from qvb8_amd.formats.qvb8.escape_split import fp16_list_for, fp16_missing_error, select_fp16
+            lst = fp16_list_for(path)
+            if lst is None:
+                raise fp16_missing_error(str(path))
+            need = select_fp16(ei, lst, str(path))
+            ei, ev = ei[need], ev[need]
+        order = np.argsort(ei, kind="stable")
+        ei, ev = ei[order], ev[order]
+        counts = np.bincount(ei // P, minlength=Q) if len(ei) else np.zeros(Q, np.int64)
+        buf("esc_ptr", np.concatenate([[0], np.cumsum(counts)]).astype(np.int64))
+        buf("esc_col", (ei % P).astype(np.int64)); buf("esc_val", ev)
+
+    @classmethod
+    def from_packfile(cls, path: str, *, out_dtype=torch.bfloat16, tau: float | None = None, device: str = "cuda",
+                      blob: bytes | None = None):
+        del tau
+        return cls(QF.read(path, blob=blob), out_dtype=out_dtype, device=device, path=path)
+
+    def _apply(self, fn, recurse=True):
+        return _apply_keeping_fp32(self, fn, recurse)
+
+    def extra_repr(self):
+        return f"{self.num_embeddings}, {self.embedding_dim}, out_dtype={self._out_dtype}, rows walked on the GPU"
+
+    def _core(self):
+        return (self.words, self.off, self.states, self.tiles, self.blocks8, self.tab, self.perm, self.min_s, self.tau_s,
+                self.drow)
+
+    def _rows(self, rows: torch.Tensor, with_escapes: bool) -> torch.Tensor:
+        """(n, P) fp32 values of the given original rows."""
+        dev = self.words.device
+        rows = rows.reshape(-1).to(device=dev, dtype=torch.int64)
+        n, P = rows.numel(), self.embedding_dim
+        if n == 0:
+            return torch.empty((0, P), dtype=torch.float32, device=dev)
+        if bool(((rows < 0) | (rows >= self.num_embeddings)).any()):
+            raise IndexError("qvb8r embedding: row id out of range")
+        wanted, which = torch.unique(self.row_block[rows], return_inverse=True)
+        ids = ext.decode_blocks(wanted.to(torch.int32).contiguous(), *self._core(), P, 3, T=self.T)
+        picked = ids[which * (WPB * self.T) + self.row_slot[rows]]
+        out = self.min_s[rows, None] + picked.to(torch.float32) * self.tau_s[rows, None]      # multiply, then add: two roundings
+        if with_escapes and self.esc_col.numel():
+            first, count = self.esc_ptr[rows], self.esc_ptr[rows + 1] - self.esc_ptr[rows]
+            total = int(count.sum())
+            if total:
+                owner = torch.repeat_interleave(torch.arange(n, device=dev), count)
+                within = torch.arange(total, device=dev) - torch.repeat_interleave(torch.cumsum(count, 0) - count, count)
+                e = first[owner] + within
+                out[owner, self.esc_col[e]] = self.esc_val[e]
+        return out
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        out = self._rows(input, True).to(self._out_dtype)
+        return out.reshape(*input.shape, self.embedding_dim).to(input.device if input.device.type != "cpu" else self.words.device)
+
+    @property
+    def weight(self):
+        """Dense (Q, P) table in the output dtype, escapes applied, restored in slices of rows."""
+        out = torch.empty(self.num_embeddings, self.embedding_dim, dtype=self._out_dtype, device=self.words.device)
+        step = max(1, (64 << 20) // (4 * self.embedding_dim))
+        for r0 in range(0, self.num_embeddings, step):
+            rows = torch.arange(r0, min(r0 + step, self.num_embeddings), device=self.words.device)
+            out[r0:r0 + rows.numel()] = self._rows(rows, True).to(self._out_dtype)
+        return out

@@ -1,9 +1,11 @@
 """GPU: graph replay of blocks built on the compressed operators is bit-identical to eager execution, replay after
 replay, with the program's own eager work and synchronisations in between."""
+import numpy as np
 import pytest
 import torch
 import torch.nn as nn
 
+from oracle import qvb8_oracle as O
 from qvb8_amd.formats.qvb8 import pack as PK
 from qvb8_amd.formats.qvb8.backends_experts import QVBandExpertsV8
 from qvb8_amd.formats.qvb8.fuse import fuse_same_input
@@ -15,8 +17,26 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+_RESTORED = {}          # module -> the oracle's restore of its pack (float32), for the float64 referee
+
+
 def _lin(Q, P, seed):
-    return QVBandLinearV8.from_encoded(PK.encode_tensor(H.synth_weight(Q, P, seed=seed).to(DEV), 1e-3, restore="fp16"))
+    enc = PK.encode_tensor(H.synth_weight(Q, P, seed=seed).to(DEV), 1e-3, restore="fp16")
+    lin = QVBandLinearV8.from_encoded(enc)
+    d = H.oracle_view(enc)
+    _RESTORED[lin] = O.reconstruct(d["min_s"], d["tau_s"], H.oracle_ids(d), d["esc_idx"], d["esc_vals"])
+    return lin
+
+
+def _mlp_oracle(mlp, x):
+    """gate / up / down through the oracle's restored weights in float64, with the roundings the module chain makes: the
+    activations saturated to fp16 on the way into every product, each product's result rounded to bf16."""
+    bf = lambda a: O.narrow_bf16(a.astype(np.float32)).astype(np.float64)
+    xs = O.sat_half(x.float().cpu().numpy())
+    g = bf(O.linear_f64(xs, _RESTORED[mlp.gate_proj]))
+    u = bf(O.linear_f64(xs, _RESTORED[mlp.up_proj]))
+    h = bf(bf(g / (1.0 + np.exp(-g))) * u)
+    return O.linear_f64(O.sat_half(h.astype(np.float32)), _RESTORED[mlp.down_proj])
 
 
 class _Mlp(nn.Module):
@@ -55,7 +75,13 @@ def test_graph_replay_is_bit_identical(kind):
     torch.manual_seed(0)
     layer = _Layer(_Mlp(512, 256) if kind == "mlp" else _Moe(256, 128, 6, 2))
     if kind == "mlp":
+        unfused = layer.mlp
+        x0 = torch.randn(3, 512, device=DEV).to(torch.bfloat16)
+        ref = _mlp_oracle(unfused, x0)                              # the referee: oracle restore + float64 arithmetic
         assert fuse_same_input(layer) == 1                          # gate+up as one launch, inside the graph as well
+        got = layer.mlp(x0).float().cpu().numpy().astype(np.float64)
+        scale = np.sqrt(np.mean(ref ** 2))
+        assert np.all(np.abs(got - ref) <= 2.0 ** -6 * np.abs(ref) + 2.0 ** -6 * scale), float(np.abs(got - ref).max() / scale)
     eager = layer.mlp
     assert install_block_graphs(layer) == 1 and isinstance(layer.mlp, GraphedBlock)
     assert install_block_graphs(layer) == 0                         # already wrapped

@@ -131,8 +131,12 @@ def test_same_input_fusion_is_bit_identical():
     for M, dtype in ((1, torch.bfloat16), (12, torch.float16), (70, torch.bfloat16), (120, torch.float16)):
         x = torch.randn(M, 512, generator=torch.Generator().manual_seed(M)).to(dtype).to(DEV)
         parts = torch.tensor_split(fused(x), splits, -1)
-        for part, lin in zip(parts, lins):
+        for part, lin, enc in zip(parts, lins, encs):
             assert torch.equal(part, lin(x)), (M, dtype)
+            # and against the oracle, not only against the separate launch
+            ref, Wr, xs = _ref(enc, x, saturate=True, narrow="fp16" if M > 256 else None)
+            b = lin.bias.double().cpu().numpy() if lin.bias is not None else 0.0
+            _close(part, ref + b, Wr, xs, dtype)
 
     class Attn(nn.Module):
         def __init__(self):

@@ -159,3 +159,81 @@ def test_argument_errors():
     short = lin.words[:100].contiguous()
     with pytest.raises(RuntimeError):
         ext.gemv(torch.zeros(256, device=DEV), short, *lin._core()[1:], T=lin.T)   # stream without its pad
+
+
+def test_same_input_fusion_against_the_oracle_and_the_members():
+    """q/k/v-like siblings (different row counts, alphabets and tile heights, one with a bias, escapes in two) joined into
+    one walk: every member's output equals its own launch bit for bit and the oracle's restore + float64 matmul within
+    the product tolerance; the registry's finalize hook does the replacement on a model."""
+    import torch.nn as nn
+    from qvb8_amd.common import formats as F
+    from qvb8_amd.common.fusion import FusedMember
+    from qvb8_amd.formats.qvb8r.fuse import concat_linears
+    P = 512
+    lins, Wrs = [], []
+    for i, (Q, kw, force) in enumerate(((96, dict(rows_per_tile=4, n_classes=2), [7, P * 90 + 500]), (40, dict(rows_per_tile=1), None),
+                                        (33, dict(), [P * 32 + 1]))):
+        W, enc, d = _make(Q, P, 2e-3, seed=70 + i, force=force, **kw)
+        lins.append(QVBandLinearV8R(d, bias=torch.full((Q,), 0.25) if i == 1 else None, device=DEV))
+        Wrs.append(R.reconstruct(d, enc["esc_idx"].cpu().numpy(), enc["esc_vals"].cpu().numpy()))
+    fused, splits = concat_linears(lins)
+    assert splits == [96, 136] and fused.out_features == 169
+    for M, dtype in ((1, torch.bfloat16), (5, torch.float32), (20, torch.float16), (60, torch.bfloat16)):
+        x = torch.randn(M, P, generator=torch.Generator().manual_seed(M)).to(dtype).to(DEV)
+        parts = torch.tensor_split(fused(x), splits, -1)
+        xs = x.float().cpu().numpy()
+        for i, (part, lin, Wr) in enumerate(zip(parts, lins, Wrs)):
+            if M <= 48:
+                assert torch.equal(part, lin(x)), (M, dtype, i)
+            Wm, xm = (O.narrow_fp16(Wr), O.sat_half(xs)) if M > 48 else (Wr, xs)
+            ref = O.linear_f64(xm, Wm) + (lin.bias.double().cpu().numpy() if lin.bias is not None else 0.0)
+            eps = {torch.float32: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+            tol = H.gemv_tolerance(ref, Wm, xm) + eps * np.abs(ref)
+            diff = np.abs(part.float().cpu().numpy().astype(np.float64) - ref)
+            assert np.all(diff <= tol), (M, dtype, i, float((diff / tol).max()))
+
+    class Attn(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj, self.k_proj, self.v_proj = lins
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.self_attn = Attn()
+    blk = Block()
+    x = torch.randn(2, P, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(DEV)
+    want = [lin(x) for lin in lins]
+    assert F.get_format("qvb8r").finalize(blk) == 1 and isinstance(blk.self_attn.k_proj, FusedMember)
+    got = [blk.self_attn.q_proj(x), blk.self_attn.k_proj(x), blk.self_attn.v_proj(x)]
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    assert blk.self_attn._qvb8r_fused._x is None
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_embedding_rows_walked_on_the_gpu(out_dtype, tmp_path):
+    """QVBandEmbeddingV8R: looked-up rows (repeats, any order, 2-D index) equal the oracle's two-rounding lookup value over
+    the oracle's walk of the same stream, escapes written over it, bit for bit; `weight` is every row; an index outside
+    the table raises; the registry hands the class out for the format."""
+    from qvb8_amd.common import formats as F
+    from qvb8_amd.formats.qvb8r.module import QVBandEmbeddingV8R
+    Q, P = 300, 640
+    W, enc, d = _make(Q, P, 2e-3, seed=3, force=[5, P * 17 + 600, P * 299 + 1], rows_per_tile=3, n_classes=2)
+    path = str(tmp_path / "emb.qvb8r")
+    RP.write_pack(path, d)
+    assert F.get_format("qvb8r").embedding is QVBandEmbeddingV8R
+    emb = QVBandEmbeddingV8R.from_packfile(path, out_dtype=out_dtype, device=DEV)
+    tok = torch.tensor([[17, 0, 299, 17], [5, 123, 298, 0]], device=DEV)
+    got = emb(tok)
+    assert got.dtype == out_dtype and got.shape == (2, 4, P)
+    name = {torch.bfloat16: "bf16", torch.float16: "fp16", torch.float32: "fp32"}[out_dtype]
+    ref = O.embedding_rows(tok.cpu().numpy().reshape(-1), d["min_s"], d["tau_s"], R.ids(d), P, d["esc_idx"], d["esc_val"], dtype=name)
+    assert np.array_equal(got.float().cpu().numpy().reshape(-1, P).view(np.uint32), ref.astype(np.float32).view(np.uint32))
+    full = emb.weight
+    ref_all = O.embedding_rows(np.arange(Q), d["min_s"], d["tau_s"], R.ids(d), P, d["esc_idx"], d["esc_val"], dtype=name)
+    assert np.array_equal(full.float().cpu().numpy().view(np.uint32), ref_all.astype(np.float32).view(np.uint32))
+    with pytest.raises(IndexError):
+        emb(torch.tensor([Q], device=DEV))
+    before = emb.tau_s.clone()
+    emb.to(torch.bfloat16)
+    assert emb.tau_s.dtype == torch.float32 and torch.equal(emb.tau_s, before)

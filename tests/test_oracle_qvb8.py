@@ -192,6 +192,23 @@ def test_moe_reference_tiny_brute_force():
     assert np.allclose(out[t], want, rtol=1e-12)
 
 
+def test_moe_reference_relu2_by_hand():
+    """The non-gated ReLU^2 branch on a case small enough to work out by hand: one token, one expert with weight 1/2
+    and one with weight 1/4, integers throughout.  up(x) = (3, -2) -> relu^2 = (9, 0); down rows (1, 5) and (2, 7)."""
+    x = np.array([[1.0, 2.0]], np.float32)
+    W_up = [np.array([[1.0, 1.0], [0.0, -1.0]], np.float32), np.array([[-1.0, 0.0], [2.0, 1.0]], np.float32)]
+    W_dn = [np.array([[1.0, 5.0], [2.0, 7.0]], np.float32), np.array([[3.0, 1.0], [0.0, -2.0]], np.float32)]
+    idx = np.array([[0, 1]], np.int64)
+    w = np.array([[0.5, 0.25]], np.float32)
+    # expert 0: up = (3, -2), h = (9, 0), down = (9, 18); expert 1: up = (-1, 4), h = (0, 16), down = (16, -32)
+    want = 0.5 * np.array([9.0, 18.0]) + 0.25 * np.array([16.0, -32.0])
+    got = O.moe_reference(x, idx, w, W_up, W_dn, act="relu2")
+    assert np.array_equal(got, want[None, :])
+    # and it is not the gated form: the same call as gated SiLU needs an even number of up rows split in halves
+    gated = O.moe_reference(x, idx, w, [np.vstack([u, u]) for u in W_up], W_dn)
+    assert not np.allclose(gated, got)
+
+
 def test_embedding_rows_two_roundings_closed_form():
     """The lookup value is fl(min + fl(id * tau)): checked against float64 arithmetic rounded explicitly at each step
     (id * tau is exact in float64: 14 + 24 bits; min + product of two floats is exact in float64 unless the exponents

@@ -177,3 +177,32 @@ def test_container_against_the_reference_reader_and_writer(golden):
     for got, want in zip(R.runtime_tables(R.read_container(mine)), (g["rt_tab"], g["rt_tiles"], g["rt_words"], g["rt_off"])):
         assert np.array_equal(got, want)
     assert np.array_equal(R.ids(R.read_container(mine)), ids)
+
+
+def test_concat_is_the_members_stacked():
+    """Joining tensors (same row length, different alphabets, classes and rows per tile) gives a tensor whose walk yields
+    the members' ids stacked in order, whose restore is the members' restores stacked, and whose escapes follow their
+    rows; the split points are the members' row counts.  The joined tensor also survives the file round trip."""
+    from qvb8_amd.formats.qvb8r import codec, container, fuse
+    rng = np.random.default_rng(11)
+    P, members = 256, []
+    for Q, spread, kw in ((40, 9, dict(rows_per_tile=3, n_classes=2)), (7, 30, dict(rows_per_tile=1)), (65, 4, dict(n_classes=3))):
+        ids = np.clip(np.rint(rng.normal(60, spread, (Q, P))), 0, 2000).astype(np.int64)
+        enc = codec.encode_ids(ids, **kw)
+        ei = np.sort(rng.choice(Q * P, 5, replace=False)).astype(np.int64)
+        d = dict(enc, Q=Q, P=P, PB=codec.PB, min_s=rng.normal(0, 0.1, Q).astype(np.float32),
+                 tau_s=(np.abs(rng.normal(2e-3, 1e-4, Q)) + 1e-5).astype(np.float32), esc_idx=ei,
+                 esc_val=rng.normal(0, 1, 5).astype(np.float32), esc_delta=rng.normal(0, 1e-3, 5).astype(np.float32), cert={})
+        members.append((ids, d))
+    joined, splits = fuse.concat([d for _, d in members])
+    assert splits == [40, 47] and joined["Q"] == 112 and joined["K"] == 6 and joined["T"] == 16
+    assert joined["N"] == max(d["N"] for _, d in members)
+    assert np.array_equal(R.ids(joined), np.vstack([ids for ids, _ in members]))
+    assert np.array_equal(R.reconstruct(joined).view(np.uint32), np.vstack([R.reconstruct(d) for _, d in members]).view(np.uint32))
+    assert np.array_equal(joined["esc_delta"], np.concatenate([d["esc_delta"] for _, d in members]))
+    blob = container.to_bytes(joined, joined["Q"], P, joined["min_s"], joined["tau_s"], joined["esc_idx"], joined["esc_val"],
+                              joined["esc_delta"], {})
+    back = container.read(blob=blob)
+    assert np.array_equal(R.ids(back), R.ids(joined))
+    with pytest.raises(ValueError):
+        fuse.concat([members[0][1], dict(members[1][1], P=128)])
