@@ -157,7 +157,8 @@ class QVBandLinearV8(nn.Module):
         return mod
 
     def escapes(self, dtype=torch.float16):
-        """(esc_idx, esc_vals) for a decode that rounds the weight to `dtype` (module.py:116-124)."""
+        """The escape table that goes with a weight rounded to `dtype`: the full list for bf16, the fp16 table otherwise
+        (reference: module.py:116-124).  An fp16+bf16 pack whose fp16 table could not be determined refuses fp16."""
         if dtype == torch.bfloat16:
             return self.esc_idx_bf16, self.esc_vals_bf16
         if dtype == torch.float16 and self.fp16_table_missing:
@@ -166,28 +167,31 @@ class QVBandLinearV8(nn.Module):
         return self.esc_idx, self.esc_vals
 
     def row_subset(self, rows: torch.Tensor) -> "QVBandLinearV8":
-        """A linear over output rows `rows` only, sharing this module's `ids` buffer: rows of a pack are independent
-        (own min_s, tau_s, width, offset), so a subset costs no weight memory (module.py:126-160)."""
-        rows = rows.to(self.min_s.device).long()
-        P = self.in_features
-        remap = torch.full((self.out_features,), -1, dtype=torch.long, device=rows.device)
-        remap[rows] = torch.arange(rows.numel(), device=rows.device)
+        """The linear restricted to output rows `rows` (in that order).  A pack's rows are independent -- each has its own
+        min_s, tau_s, width and bit offset -- so the subset only selects row metadata and keeps pointing into THIS
+        module's `ids`: no weight bytes are copied (what the reference does for a restricted vocabulary head,
+        module.py:126-160).  Escapes of other rows are dropped, the kept ones renumbered to the new row order."""
+        rows = rows.to(device=self.min_s.device, dtype=torch.long)
+        P, n = self.in_features, int(rows.numel())
+        new_row_of = torch.full((self.out_features,), -1, dtype=torch.long, device=rows.device)
+        new_row_of[rows] = torch.arange(n, device=rows.device)
 
-        def sub(esc_idx, esc_vals):
-            if not esc_idx.numel():
-                return esc_idx, esc_vals
-            q = esc_idx // P
-            keep = remap[q] >= 0
-            return remap[q[keep]] * P + esc_idx[keep] % P, esc_vals[keep]
-        esc_idx, esc_vals = sub(self.esc_idx, self.esc_vals)
-        same = self.esc_idx_bf16 is self.esc_idx
-        ei_b, ev_b = (None, None) if same else sub(self.esc_idx_bf16, self.esc_vals_bf16)
-        m = type(self)(min_s=self.min_s[rows], nbits=self.nbits[rows], bit_off=self.bit_off[rows], ids=self.ids,
-                       Q=int(rows.numel()), P=P, tau_s=self.tau_s[rows], esc_idx=esc_idx, esc_vals=esc_vals,
-                       bias=None, esc_idx_bf16=ei_b, esc_vals_bf16=ev_b)
-        m.bf16_certified = self.bf16_certified
-        m.fp16_table_missing = self.fp16_table_missing
-        return m
+        def restrict(table):
+            idx, vals = table
+            if idx.numel() == 0:
+                return idx, vals
+            target = new_row_of[torch.div(idx, P, rounding_mode="floor")]
+            kept = target >= 0
+            return target[kept] * P + torch.remainder(idx[kept], P), vals[kept]
+
+        fp16_tab = restrict((self.esc_idx, self.esc_vals))
+        one_table = self.esc_idx_bf16 is self.esc_idx
+        bf16_tab = (None, None) if one_table else restrict((self.esc_idx_bf16, self.esc_vals_bf16))
+        picked = {name: getattr(self, name)[rows] for name in ("min_s", "tau_s", "nbits", "bit_off")}
+        sub = type(self)(ids=self.ids, Q=n, P=P, esc_idx=fp16_tab[0], esc_vals=fp16_tab[1], bias=None,
+                         esc_idx_bf16=bf16_tab[0], esc_vals_bf16=bf16_tab[1], **picked)
+        sub.bf16_certified, sub.fp16_table_missing = self.bf16_certified, self.fp16_table_missing
+        return sub
 
     def _apply(self, fn, recurse=True):
         out = apply_keeping_fp32_metadata(self, fn, recurse)
@@ -200,12 +204,16 @@ class QVBandLinearV8(nn.Module):
         """(perm, rowinfo, layout) for ext.mma_tiles, or None when the tile kernel cannot read this weight.  Rows are sorted by
         width so that a 16-row tile shares one width (one decode pass); the row records hold, in that order, where each
         row's ids start, its width, tau_s, min_s and its output row.  Built once per weight, like the reference's
-        perm / tile_nb (module.py:230-277); never built inside a graph capture (the width check reads the device)."""
+        perm / tile_nb (module.py:230-277).  Inside a graph capture only an earlier result can be used: a first call there
+        raises."""
         cached = self.__dict__.get("_mma_cache", False)
         if cached is not False:
             return cached
         if torch.cuda.is_current_stream_capturing():
-            return None
+            # building them reads the device (width range) and may re-order `ids`: not inside a capture, and falling
+            # back to another kernel here would make a captured graph compute something else than eager calls do
+            raise RuntimeError("QVBandLinearV8: first call inside a graph capture -- call the module once (or prepare()) "
+                               "before capturing")
         order = None
         if self.ids.is_cuda and self.in_features % 128 == 0 and self.ids.data_ptr() % 4 == 0 and self.out_features > 0:
             nb = self.nbits.to(torch.int16)
@@ -222,6 +230,11 @@ class QVBandLinearV8(nn.Module):
                 order = (perm, rowinfo, layout)
         self._mma_cache = order
         return order
+
+    def prepare(self) -> "QVBandLinearV8":
+        """Builds the per-weight launch data now (load time) instead of on the first forward; returns self."""
+        self._mma_order()
+        return self
 
     def _gemm_ok(self, layout, bf16_mode: bool) -> bool:
         """Whether the workgroup-tiled kernel (49..256 rows) can read this weight: rows stored in width order, every
@@ -311,26 +324,28 @@ def enable_bf16_gemm(model: nn.Module) -> tuple[int, int]:
 
 
 def footprint_report(module) -> dict:
-    """Resident bytes of the packed linears under `module`: ids, escapes (12 bytes each), row metadata, and the
-    bytes-per-parameter figure a caller compares with dense fp16's 2.0 (module.py:527-587)."""
-    ids = escapes = meta = 0
-    n_esc = n_params = n_lin = 0
-    for _, m in module.named_modules():
+    """What the packed linears under `module` keep resident, by kind: packed ids, escape tables (each table counted once;
+    an fp16+bf16 pack holds two), per-row metadata; and the bytes per weight that a caller compares with the 2.0 of a
+    dense 16-bit copy (the reference reports the same figures, module.py:527-587)."""
+    def nbytes(*tensors):
+        return sum(t.numel() * t.element_size() for t in tensors)
+
+    report = dict(linears=0, params=0, escape_count=0, ids_bytes=0, escape_bytes=0, meta_bytes=0)
+    for m in module.modules():
         if not isinstance(m, QVBandLinearV8):
             continue
-        n_lin += 1
-        n_params += m.out_features * m.in_features
-        ids += m.ids.numel() * m.ids.element_size()
-        tabs = [m.esc_idx, m.esc_vals]
+        tables = [(m.esc_idx, m.esc_vals)]
         if m.esc_idx_bf16.data_ptr() != m.esc_idx.data_ptr():
-            tabs += [m.esc_idx_bf16, m.esc_vals_bf16]
-        for t in tabs:
-            n_esc += t.numel()
-            escapes += t.numel() * t.element_size()
-        for t in (m.min_s, m.tau_s, m.nbits, m.bit_off):
-            meta += t.numel() * t.element_size()
-    total = ids + escapes + meta
-    return {"linears": n_lin, "params": n_params, "escape_count": n_esc, "ids_bytes": ids, "escape_bytes": escapes,
-            "meta_bytes": meta, "total_bytes": total,
-            "bytes_per_param": (total / n_params) if n_params else 0.0,
-            "escape_ratio": (n_esc / n_params) if n_params else 0.0}
+            tables.append((m.esc_idx_bf16, m.esc_vals_bf16))
+        report["linears"] += 1
+        report["params"] += m.out_features * m.in_features
+        report["ids_bytes"] += nbytes(m.ids)
+        report["meta_bytes"] += nbytes(m.min_s, m.tau_s, m.nbits, m.bit_off)
+        for idx, vals in tables:
+            report["escape_count"] += idx.numel() + vals.numel()
+            report["escape_bytes"] += nbytes(idx, vals)
+    report["total_bytes"] = report["ids_bytes"] + report["escape_bytes"] + report["meta_bytes"]
+    n = report["params"]
+    report["bytes_per_param"] = report["total_bytes"] / n if n else 0.0
+    report["escape_ratio"] = report["escape_count"] / n if n else 0.0
+    return report
