@@ -15,6 +15,7 @@
 // sum, and the two terms joined in double: reproducible, and within rounding of  sum(x * fmaf(id, tau_s, min_s)).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <algorithm>
 #include <mutex>
 #include <type_traits>
 
@@ -29,7 +30,7 @@ constexpr int kMoeMB = 8;              // pairs that share one pass over an expe
 constexpr int kMoeThreads = 256;
 
 // Workspace layout (bytes from the start): plan | H | Yd
-//   plan: i32 n_bad (+3 pad), int4 slot[n_slots] = {expert, first pair, end pair, 0} for the experts that have pairs
+//   plan: i32 n_bad, i32 slots in use (+2 pad), int4 slot[n_slots] = {expert, first pair, end pair, 0} for the experts that have pairs
 //   (end == first for unused slots), i32 order[npairs] (pair numbers grouped by expert)
 struct MoePlan {
     int32_t* n_bad; int4* slot; int32_t* order;
@@ -89,6 +90,7 @@ __global__ void __launch_bounds__(kMoeThreads) moe_plan_kernel(const int64_t* __
         __syncthreads();
     }
     for (int i = run_active + tid; i < n_slots; i += blockDim.x) pl.slot[i] = int4{0, 0, 0, 0};
+    if (tid == 0) pl.n_bad[1] = run_active;                   // slots in use
     __syncthreads();
     for (int p = tid; p < npairs; p += blockDim.x) {
         const int64_t e = idx[p];
@@ -519,6 +521,289 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
     }
 }
 
+// ---- a few tokens (2..16): the tokens that chose an expert share one walk over it, on the matrix cores -------------------
+// The routing plan groups the (token, choice) pairs by expert; a selected expert has at most one pair per token, so its
+// pairs fit the 16 token rows of one MFMA operand, and every id that is read serves all of the expert's tokens: each
+// selected expert's bytes are read once, however many tokens chose it.
+//   work:  the tiles of the experts in use, numbered slot * tiles per expert + tile, are dealt to the workgroups in equal
+//          contiguous shares (the plan holds the number of slots in use, so the shares are equal whatever the routing);
+//          a share is walked in segments: tiles of ONE expert, as many as the LDS holds.
+//   segment: the waves hold the activation rows of the expert's pairs as MFMA operands (row t = pair order[first + t]:
+//          the pair's token for the up projection, the pair's own H row for the down projection; loaded when the expert
+//          changes).  The segment's rows are regrouped BY WIDTH in LDS (a stable counting sort of at most 256 row
+//          records), so that the 16 rows a wave decodes together nearly always share one width and take the
+//          single-width decode; a tile across a boundary takes each width in turn.  Then, per tile: T steps of 128
+//          columns per wave, ids decoded into MFMA operands, the next tile's ids in flight meanwhile, partial sums in LDS.
+//   up:   unit tiles of 16 outputs (gated: the 16 gate rows and the 16 matching up rows); H[pair] as saturated fp16.
+//   down: tiles of 16 rows; Yd[pair] in fp32 for the weighted combine (moe_combine_kernel).
+struct MoeGroupArgs {
+    const uint16_t* X;             // up: (tokens, P) fp16 or bf16 bits; down: H (npairs, P) fp16 bits
+    MoePlan plan;
+    const uint8_t* ids; int64_t ids_bytes;
+    const float* min_s; const float* tau_s; const uint8_t* nbits; const int64_t* bit_off;   // (E, Q)
+    void* out;                     // up: H (npairs, units) fp16 bits; down: Yd (npairs, Q) f32
+    int E, Q, P, topk;
+    int units, gated;              // up: outputs per expert; whether the rows come as (gate, up) halves
+    int tiles_per_seg;             // unit tiles (up) / row tiles (down) per segment
+    int max_tokens;                // most pairs an expert can have in this call (the LDS is laid out for it)
+};
+constexpr int kGroupWaves = 4;         // waves per workgroup: two workgroups share a CU
+constexpr int kGroupMaxRowTiles = 16;  // row tiles per segment: one row record per thread
+
+struct GroupRow { int64_t bit0; int flags; float ts, mn; int pad; };       // flags = width | usable << 8 | sliced << 9
+
+template <int T, bool DOWN, bool XC, bool TWO>
+__device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
+    using F = Fmt<false>;
+    using XI = XIn<false, XC>;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, kg = lane >> 4;
+    const int n_steps = a.P / kStepCols;
+    const int W = (n_steps + T - 1) / T, G = kGroupWaves / W;
+    const int g = wave / W, wc = wave - g * W;
+    const bool walker = g < G;                               // W = 3 leaves one wave without a column range
+    const int step0 = wc * T;
+    const int RT = (!DOWN && a.gated) ? 2 : 1;               // row tiles per unit tile
+    const int UT = DOWN ? a.Q / 16 : a.units / 16;           // tiles per expert
+    const int rt_cap = a.tiles_per_seg * RT;
+    // LDS: partial sums [row tile][column range][row][token], sums of the activations [column range][token], per sorted
+    // row its constants and its record, the counts of the sort, per natural row its sorted place
+    float* s_part = reinterpret_cast<float*>(smem);
+    float* s_sx = s_part + (size_t)rt_cap * W * 16 * a.max_tokens;                        // [W][16]
+    float2* s_fin = reinterpret_cast<float2*>(s_sx + W * 16);                             // [rt_cap * 16]
+    GroupRow* s_row = reinterpret_cast<GroupRow*>(s_fin + (size_t)rt_cap * 16);           // [rt_cap * 16]
+    int* s_cls = reinterpret_cast<int*>(s_row + (size_t)rt_cap * 16);                     // [kGroupWaves][8]
+    uint16_t* s_pos = reinterpret_cast<uint16_t*>(s_cls + kGroupWaves * 8);               // [rt_cap * 16]
+    const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
+    const v4u_t ones = {F::one_bits, F::one_bits, F::one_bits, F::one_bits};
+    // the workgroups are dealt to the experts in use, equally many each; an expert's tiles in equal runs to its workgroups
+    const int n_active = a.plan.n_bad[1];
+    const int per_expert = max(1, (int)gridDim.x / max(1, n_active));
+    const int sl = (int)blockIdx.x / per_expert;
+    if (sl >= n_active) return;                              // the whole workgroup
+    const int run = (UT + per_expert - 1) / per_expert;
+    int t0 = ((int)blockIdx.x - sl * per_expert) * run;
+    const int t_end = min(UT, t0 + run);
+
+    v4u_t xa[T][4];
+    v4f_t sx = {0.f, 0.f, 0.f, 0.f};
+    while (t0 < t_end) {
+        const int ut_first = t0;
+        const int n_rt = min(a.tiles_per_seg, t_end - t0) * RT;
+        t0 += n_rt / RT;
+        auto row0_of = [&](int i) { return DOWN ? (ut_first + i) * 16 : (ut_first + i / RT) * 16 + (i % RT) * a.units; };
+        // ---- the activations of the expert's pairs: operand row t = r (requested for every segment: from the caches after
+        // the first, and never under a branch, so that the waits below are exact) ----
+        const int4 slot = a.plan.slot[sl];
+        const int e = slot.x, first = slot.y, n = max(1, min(slot.z - slot.y, min(16, a.max_tokens)));
+        const bool e_ok = e >= 0 && e < a.E;
+        const int pair = a.plan.order[first + min(r, n - 1)];
+        // ---- the segment's row records, regrouped by width (stable: rows of a width keep their order) ----
+        const int n_rows = n_rt * 16;
+        int key = 7, rank = 0;
+        GroupRow mine{0, 0, 0.f, 0.f, 0};
+        const size_t mi = (size_t)(e_ok ? e : 0) * a.Q + (tid < n_rows ? row0_of(tid >> 4) + (tid & 15) : 0);
+        const int nb = a.nbits[mi];
+        const int64_t bit0 = a.bit_off[mi];
+        const float row_ts = a.tau_s[mi], row_mn = a.min_s[mi];
+        const uint16_t* xrow = a.X + (size_t)(DOWN ? pair : pair / a.topk) * a.P;
+#pragma unroll
+        for (int it = 0; it < T; ++it) {
+            const bool on = (step0 + it) < n_steps;
+            const uint16_t* xp = xrow + (on ? (size_t)(step0 + it) * kStepCols + kg * 32 : (size_t)0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xa[it][j] = *reinterpret_cast<const v4u_t*>(xp + 8 * j);
+        }
+        if (tid < n_rows) {
+            const bool ok = e_ok && nb >= 1 && nb <= 14 && bit0 >= 0 && ((bit0 + (int64_t)nb * a.P + 7) >> 3) + 8 <= a.ids_bytes;
+            const bool sliced = ok && nb >= 4 && nb <= 8 && (bit0 & 31) == 0;
+            mine = GroupRow{ok ? bit0 : 0, nb | (ok ? 256 : 0) | (sliced ? 512 : 0), row_ts, row_mn, tid};
+            key = sliced ? nb - 4 : 5;
+        }
+#pragma unroll
+        for (int c = 0; c < 6; ++c) {
+            const uint64_t m = __builtin_amdgcn_ballot_w64(key == c);
+            if (key == c) rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
+            if (lane == 0) s_cls[wave * 8 + c] = __builtin_popcountll(m);
+        }
+        __syncthreads();
+        if (tid < n_rows) {
+            int base = 0;
+#pragma unroll
+            for (int c = 0; c < 6; ++c)
+#pragma unroll
+                for (int w = 0; w < kGroupWaves; ++w)
+                    if (c < key || (c == key && w < wave)) base += s_cls[w * 8 + c];
+            s_row[base + rank] = mine;
+            s_pos[tid] = (uint16_t)(base + rank);
+        }
+        __syncthreads();
+        const int n_rounds = (n_rt + G - 1) / G;
+        // Requests the lane's slices of the wave's tile of round `rnd` (clamped to the last round: nothing under a branch,
+        // the repeated request at the end reads lines that are in the caches).  Returns the lane's row record.
+        auto issue = [&](int rnd, uint4 (&lo)[T], uint4 (&hi)[T]) __attribute__((always_inline)) -> GroupRow {
+            const int i = min(g + min(rnd, n_rounds - 1) * G, n_rt - 1);
+            const GroupRow rec = s_row[i * 16 + r];
+            const uint32_t nb = (uint32_t)rec.flags & 255u;
+            const bool sliced = (rec.flags & 512) != 0;
+            const uint64_t row_off = (uint64_t)(rec.bit0 >> 3) + (uint64_t)(step0 * 4 + kg) * (4u * nb);
+#pragma unroll
+            for (int it = 0; it < T; ++it) {
+                const bool use = sliced && (step0 + it) < n_steps;
+                const uint64_t off = use ? row_off + (uint64_t)it * (16u * nb) : 0;
+                lo[it] = *reinterpret_cast<const uint4*>(a.ids + off);
+                hi[it] = *reinterpret_cast<const uint4*>(a.ids + off + (use ? 4u * (nb - 4u) : 16u));
+            }
+            return rec;
+        };
+        uint4 lo0[T], hi0[T], lo1[T], hi1[T];
+        GroupRow rec0{0, 0, 0.f, 0.f, 0}, rec1{0, 0, 0.f, 0.f, 0};
+        rec0 = issue(0, lo0, hi0);                           // by every wave: nothing under a branch
+        {
+            // rows past the expert's tokens and steps past the row multiply zeros; bf16 activations are narrowed like
+            // every activation
+#pragma unroll
+            for (int it = 0; it < T; ++it) {
+                const bool on = (step0 + it) < n_steps && r < n;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) xa[it][j][k] = on ? XI::pair(xa[it][j][k]) : 0u;
+            }
+            // sums of the activations over this wave's columns, per token: accumulator layout, lane (row r, token
+            // group kg) register k <-> token 4 kg + k
+            sx = v4f_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int it = 0; it < T; ++it)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) sx = F::mfma(xa[it][j], ones, sx);
+            if (g == 0 && r == 0) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) s_sx[wc * 16 + kg * 4 + k] = sx[k];
+            }
+        }
+        auto compute = [&](int rnd, const GroupRow& rec, const uint4 (&lo_)[T], const uint4 (&hi_)[T]) __attribute__((always_inline)) {
+            v4f_t acc = {0.f, 0.f, 0.f, 0.f};
+            const int nb = rec.flags & 255;
+            const bool sliced = (rec.flags & 512) != 0;
+            const uint32_t info = sliced ? ((uint32_t)nb | 256u) : 0u;
+            const uint32_t info0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
+            const bool uniform = __builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u;
+#pragma unroll
+            for (int it = 0; it < T; ++it) {
+                v4u_t b[4];
+                const uint4 lo = lo_[it], hi = hi_[it];
+                if (uniform) {
+                    switch (info0 & 0xFFu) {
+                        case 7: decode_slice<7, false>(lo, hi, b); break;
+                        case 6: decode_slice<6, false>(lo, hi, b); break;
+                        case 5: decode_slice<5, false>(lo, hi, b); break;
+                        case 4: decode_slice<4, false>(lo, hi, b); break;
+                        default: decode_slice<8, false>(lo, hi, b); break;
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) b[j] = v4u_t{F::bias_bits, F::bias_bits, F::bias_bits, F::bias_bits};
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 7)) { if (sliced && nb == 7) decode_slice<7, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 6)) { if (sliced && nb == 6) decode_slice<6, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 5)) { if (sliced && nb == 5) decode_slice<5, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 4)) { if (sliced && nb == 4) decode_slice<4, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 8)) { if (sliced && nb == 8) decode_slice<8, false>(lo, hi, b); }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc = F::mfma(xa[it][j], b[j], acc);
+            }
+            const int i = g + rnd * G;                            // place of the tile among the sorted rows
+            if (i < n_rt) {                                       // wave-uniform
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int t = kg * 4 + k;
+                    if (t < n) s_part[(((size_t)i * W + wc) * 16 + r) * n + t] = __builtin_fmaf(-F::bias, sx[k], acc[k]);
+                }
+                if (kg == 0 && wc == 0) s_fin[i * 16 + r] = float2{(rec.flags & 256) ? rec.ts : __builtin_nanf(""), rec.mn};
+                // rows the slicing cannot read: element by element over this wave's columns, token by token
+                uint64_t odd = __builtin_amdgcn_ballot_w64(kg == 0 && !sliced);
+                while (odd) {
+                    const int rr = __builtin_ctzll(odd);
+                    odd &= odd - 1;
+                    const GroupRow o = s_row[i * 16 + rr];
+                    const int nb2 = o.flags & 255;
+                    const int c_lo = step0 * kStepCols, c_hi = min(a.P, (step0 + T) * kStepCols);
+                    for (int t = 0; t < n; ++t) {
+                        const int pr = a.plan.order[first + t];
+                        const uint16_t* xr = a.X + (size_t)(DOWN ? pr : pr / a.topk) * a.P;
+                        float sacc = 0.f;
+                        if (o.flags & 256) {
+                            for (int c = c_lo + lane; c < c_hi; c += kWave)
+                                sacc = __builtin_fmaf(XI::scalar(xr[c]), (float)load_field(a.ids, o.bit0 + (int64_t)c * nb2, nb2, clamp_byte), sacc);
+                        }
+                        const float tot = wave_sum(sacc);
+                        if (lane == 0) s_part[(((size_t)i * W + wc) * 16 + rr) * n + t] += tot;
+                    }
+                }
+            }
+        };
+        if (walker) {
+            if constexpr (TWO) {
+                // two register sets: the next tile's ids are in flight while a tile is decoded
+                for (int r0 = 0; r0 < n_rounds; r0 += 2) {
+                    rec1 = issue(r0 + 1, lo1, hi1);
+                    compute(r0, rec0, lo0, hi0);
+                    rec0 = issue(r0 + 2, lo0, hi0);
+                    if (r0 + 1 < n_rounds) compute(r0 + 1, rec1, lo1, hi1);
+                }
+            } else {
+                for (int r0 = 0; r0 < n_rounds; ++r0) {
+                    compute(r0, rec0, lo0, hi0);
+                    if (r0 + 1 < n_rounds) rec0 = issue(r0 + 1, lo0, hi0);
+                }
+            }
+        }
+        __syncthreads();
+
+        // natural row j of the segment, token t: tau_s * sum(x * id) + min_s * sum(x), the column ranges added in order
+        auto row_value = [&](int j, int t) {
+            const int at = s_pos[j];
+            double d = 0.0, xs = 0.0;
+            for (int w = 0; w < W; ++w) { d += (double)s_part[(((size_t)(at >> 4) * W + w) * 16 + (at & 15)) * n + t]; xs += (double)s_sx[w * 16 + t]; }
+            const float2 f = s_fin[at];
+            return (float)((double)f.x * d + (double)f.y * xs);
+        };
+        if constexpr (DOWN) {
+            float* Yd = reinterpret_cast<float*>(a.out);
+            for (int o = tid; o < n_rows * n; o += blockDim.x) {
+                const int t = o % n, j = o / n;
+                Yd[(size_t)a.plan.order[first + t] * a.Q + row0_of(j >> 4) + (j & 15)] = row_value(j, t);
+            }
+        } else {
+            const int n_ut = n_rt / RT;
+            uint16_t* H = reinterpret_cast<uint16_t*>(a.out);
+            for (int o = tid; o < n_ut * 16 * n; o += blockDim.x) {
+                const int t = o % n, u = (o / n) & 15, lut = o / (16 * n), j0 = lut * RT * 16 + u;
+                const float y0 = row_value(j0, t);
+                float h;
+                if (a.gated) h = (y0 / (1.0f + __expf(-y0))) * row_value(j0 + 16, t);
+                else { const float pz = fmaxf(y0, 0.f); h = y0 != y0 ? y0 : pz * pz; }
+                H[(size_t)a.plan.order[first + t] * a.units + (ut_first + lut) * 16 + u] = (uint16_t)sat_half_bits(h);
+            }
+        }
+        __syncthreads();                                     // the next segment reuses the LDS
+    }
+}
+
+// rows of up to 2048 columns: within 256 registers, two workgroups per CU (one starts while the other walks)
+template <int T, bool DOWN, bool XC, bool TWO>
+__global__ void __launch_bounds__(64 * kGroupWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) moe_group_kernel(MoeGroupArgs a) {
+    moe_group_body<T, DOWN, XC, TWO>(a);
+}
+// longer rows: eight steps of activations per wave need more registers, one workgroup per CU
+template <bool DOWN, bool XC>
+__global__ void __launch_bounds__(64 * kGroupWaves) moe_group_wide_kernel(MoeGroupArgs a) {
+    moe_group_body<8, DOWN, XC, false>(a);
+}
+
 template <int DT>
 __global__ void __launch_bounds__(256) moe_combine_kernel(const float* __restrict__ Yd, const float* __restrict__ w, void* __restrict__ out,
                                                           int topk, int D, int tokens, const int32_t* __restrict__ n_bad) {
@@ -588,6 +873,50 @@ int launch_moe_one(const MoeOneArgs& a, unsigned blocks, unsigned tokens, hipStr
     hipLaunchKernelGGL((moe_one_kernel<4, DOWN, XC, DT>), dim3(blocks, tokens), dim3(64 * kOneWaves), 0, s, a);
     return host::check_launch("qvb8_moe_experts");
 }
+
+// The grouped matrix-core path (2..16 tokens): what it needs.
+bool moe_group_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t Q_up, int64_t P_up, int64_t Q_dn, int64_t P_dn, int act) {
+    if (tokens < host::env_int("QVB8_MOE_GROUP_FROM", 2) || tokens > 16 || (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16)) return false;
+    if (P_up % kStepCols != 0 || P_dn % kStepCols != 0 || P_up > 4096 || P_dn > 4096) return false;
+    if (P_dn % 16 != 0 || Q_dn % 16 != 0) return false;
+    (void)Q_up; (void)act; (void)topk;
+    return host::env_int("QVB8_MOE_GROUPED", 1) != 0;
+}
+
+template <bool DOWN, bool XC>
+int launch_moe_group(MoeGroupArgs a, int64_t slots, int64_t max_tokens, hipStream_t s) {
+    const int n_steps = a.P / kStepCols;
+    // steps per wave: four, with the next tile's ids in flight; a short down row (up to 768 columns) is one wave's; rows
+    // beyond 2048 columns take eight steps per wave and one register set
+    const int T = (DOWN && n_steps <= 6) ? 6 : (n_steps <= 4 * kGroupWaves ? 4 : 8);
+    const int W = (n_steps + T - 1) / T;
+    const int RT = (!DOWN && a.gated) ? 2 : 1;
+    const int UT = DOWN ? a.Q / 16 : a.units / 16;
+    a.max_tokens = (int)std::min<int64_t>(16, max_tokens);
+    // tiles per segment: what the LDS of two workgroups per CU holds, one row record per thread
+    auto lds_of = [&](int64_t tiles) {
+        return (size_t)tiles * RT * W * 16 * a.max_tokens * 4 + (size_t)W * 16 * 4 + (size_t)tiles * RT * 16 * (8 + sizeof(GroupRow) + 2)
+               + (size_t)kGroupWaves * 8 * 4 + 16;
+    };
+    int64_t per_seg = std::min<int64_t>(host::env_int("QVB8_MOE_GROUP_SEG_TILES", kGroupMaxRowTiles), kGroupMaxRowTiles / RT);
+    per_seg = std::max<int64_t>(1, std::min<int64_t>(per_seg, UT));
+    while (per_seg > 1 && lds_of(per_seg) > 64 * 1024) --per_seg;
+    a.tiles_per_seg = (int)per_seg;
+    const size_t lds = lds_of(per_seg);
+    if (lds > 64 * 1024) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_moe_experts: rows too long for the grouped kernel's LDS");
+    // two workgroups per CU, at least one per slot (the kernel deals them to the experts in use)
+    const int64_t wgs = std::max<int64_t>(slots, std::min<int64_t>((int64_t)host::env_int("QVB8_MOE_GROUP_WGS_PER_CU", 2) * host::device_cus(), slots * UT));
+    dim3 grid((unsigned)wgs), block(64 * kGroupWaves);
+    if constexpr (DOWN) {
+        if (T == 6) {
+            hipLaunchKernelGGL((moe_group_kernel<6, true, XC, false>), grid, block, lds, s, a);
+            return host::check_launch("qvb8_moe_experts");
+        }
+    }
+    if (T == 4) hipLaunchKernelGGL((moe_group_kernel<4, DOWN, XC, true>), grid, block, lds, s, a);
+    else hipLaunchKernelGGL((moe_group_wide_kernel<DOWN, XC>), grid, block, lds, s, a);
+    return host::check_launch("qvb8_moe_experts");
+}
 }  // namespace
 
 extern "C" int64_t qvb8_moe_workspace_bytes(int64_t tokens, int64_t topk, int64_t n_experts, int64_t Q_up, int64_t P_dn, int64_t Q_dn) {
@@ -627,7 +956,8 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
     float* H = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np));
     float* Yd = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np) + align256((size_t)np * P_dn * 4));
 
-    if (moe_one_token_ok(tokens, topk, x_dtype, Q_up, P_up, Q_dn, P_dn, act)) {
+    const bool grouped = moe_group_ok(tokens, topk, x_dtype, Q_up, P_up, Q_dn, P_dn, act);
+    if (!grouped && moe_one_token_ok(tokens, topk, x_dtype, Q_up, P_up, Q_dn, P_dn, act)) {
         MoeOneArgs o;
         o.X = reinterpret_cast<const uint16_t*>(X); o.idx = idx; o.w = w; o.ids = up_ids; o.ids_bytes = up_ids_bytes;
         o.min_s = up_min; o.tau_s = up_tau; o.nbits = up_nb; o.bit_off = up_off; o.out = H;
@@ -654,6 +984,23 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)(n_experts + 8) * 4, s, idx, (int)np, (int)n_experts, pl);
     if (int rc = host::check_launch("qvb8_moe_experts plan")) return rc;
     const int64_t slots = moe_slots(n_experts, np);
+    if (grouped) {
+        MoeGroupArgs ga;
+        ga.X = reinterpret_cast<const uint16_t*>(X); ga.plan = pl; ga.ids = up_ids; ga.ids_bytes = up_ids_bytes;
+        ga.min_s = up_min; ga.tau_s = up_tau; ga.nbits = up_nb; ga.bit_off = up_off; ga.out = H;        // H as fp16 (pairs, P_dn)
+        ga.E = (int)n_experts; ga.Q = (int)Q_up; ga.P = (int)P_up; ga.topk = (int)topk; ga.units = (int)P_dn; ga.gated = act == 0 ? 1 : 0;
+        ga.tiles_per_seg = 1; ga.max_tokens = 1;
+        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_group<false, true>(ga, slots, tokens, s) : launch_moe_group<false, false>(ga, slots, tokens, s)) return rc;
+        ga.X = reinterpret_cast<const uint16_t*>(H); ga.ids = dn_ids; ga.ids_bytes = dn_ids_bytes;
+        ga.min_s = dn_min; ga.tau_s = dn_tau; ga.nbits = dn_nb; ga.bit_off = dn_off; ga.out = Yd;
+        ga.Q = (int)Q_dn; ga.P = (int)P_dn; ga.units = (int)Q_dn; ga.gated = 0;
+        if (int rc = launch_moe_group<true, false>(ga, slots, tokens, s)) return rc;
+        dim3 cgrid((unsigned)((Q_dn + 255) / 256), (unsigned)tokens);
+        if (out_dtype == QVB8_F32) hipLaunchKernelGGL(moe_combine_kernel<0>, cgrid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
+        else if (out_dtype == QVB8_F16) hipLaunchKernelGGL(moe_combine_kernel<1>, cgrid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
+        else hipLaunchKernelGGL(moe_combine_kernel<2>, cgrid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
+        return host::check_launch("qvb8_moe_experts combine");
+    }
 
     MoeGemvArgs a;
     a.X = X; a.ids = up_ids; a.ids_bytes = up_ids_bytes; a.min_s = up_min; a.tau_s = up_tau; a.nbits = up_nb; a.bit_off = up_off;

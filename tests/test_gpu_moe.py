@@ -180,3 +180,73 @@ def test_moe_refusals():
     with pytest.raises(RuntimeError):                        # gate_up / down shapes disagree
         ext.moe_experts(x, idx, w, s["ids"], s["min_s"], s["tau_s"], s["nbits"], s["bit_off"], s["Q"], s["P"],
                         d["ids"], d["min_s"], d["tau_s"], d["nbits"], d["bit_off"], d["Q"], d["P"] + 32)
+
+
+@pytest.mark.parametrize("T,k,dtype", [(2, 2, torch.bfloat16), (5, 4, torch.float16), (16, 8, torch.bfloat16), (9, 1, torch.float16)])
+def test_moe_few_tokens_share_each_expert(T, k, dtype):
+    """2..16 tokens on the matrix cores: the tokens that chose an expert share one walk over it.  Shapes the grouped
+    kernels take (row lengths that are multiples of 128), more experts than get selected and experts selected by many
+    tokens at once; against the oracle, reproducible, and equal to the per-token result of the same library."""
+    E, hidden, inter = 12, 384, 128
+    gu, dn, Wgu, Wdn = _experts(E, hidden, inter, 2e-3, seed=900)
+    idx, w = _route(T, E, k, seed=50 + T)
+    idx[:, 0] = 3                                              # one expert chosen by every token
+    if k > 1:
+        for t in range(T):                                     # keep a token's choices distinct
+            others = [e for e in range(E) if e != 3]
+            idx[t, 1:] = np.random.default_rng(t).choice(others, k - 1, replace=False)
+    x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(dtype)
+    mod = QVBandExpertsV8(gu, dn, num_experts=E)
+    args = (x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
+    out = mod(*args)
+    _check(out, O.moe_reference(x.float().numpy(), idx, w, Wgu, Wdn), dtype)
+    assert torch.equal(out, mod(*args))
+    # token by token through the one-token kernels: the same products, H and the weighted sums rounded the same way
+    single = torch.cat([mod(args[0][t:t + 1], args[1][t:t + 1], args[2][t:t + 1]) for t in range(T)])
+    _check(single, O.moe_reference(x.float().numpy(), idx, w, Wgu, Wdn), dtype)
+    bad = args[1].clone()
+    bad[T - 1, 0] = E + 5
+    assert torch.isnan(mod(args[0], bad, args[2]).float()).all()
+
+
+def test_moe_few_tokens_relu2_and_rows_the_slicing_cannot_read():
+    """The grouped kernels on hand-made packs: non-gated ReLU^2, every width 1..14 among the up rows (the element-wise
+    path inside the grouped kernel), row lengths of 128 and 256."""
+    E, hidden, inter = 4, 256, 128
+    ups, dns, Wup, Wdn = [], [], [], []
+    for e in range(E):
+        for lst, Wl, (Q, P), widths in ((ups, Wup, (inter, hidden), list(range(1, 15))), (dns, Wdn, (hidden, inter), [4, 5, 6, 7, 8, 11])):
+            d = H.mixed_width_pack(Q, P, widths, seed=17 * e + len(lst))
+            d["tau_s"] = d["tau_s"] * (1.0 / (1 << 7))
+            a = H.to_device_args(d, DEV)
+            lst.append(dict(ids=a[0], min_s=a[1], nbits=a[2], bit_off=a[3], tau_s=a[5]))
+            Wl.append(O.reconstruct(d["min_s"], d["tau_s"], d["ids_dense"], d["esc_idx"], d["esc_vals"]))
+
+    def stack(lst):
+        offs, total = [], 0
+        for t in lst:
+            offs.append(total)
+            total += (t["ids"].numel() + 15) // 16 * 16
+        ids = torch.zeros(total + 64, dtype=torch.uint8, device=DEV)
+        for o, t in zip(offs, lst):
+            ids[o:o + t["ids"].numel()] = t["ids"]
+        return (ids, torch.stack([t["min_s"] for t in lst]), torch.stack([t["tau_s"] for t in lst]),
+                torch.stack([t["nbits"] for t in lst]), torch.stack([t["bit_off"] + 8 * o for t, o in zip(lst, offs)]))
+    for T, k in ((6, 2), (13, 3)):
+        idx, w = _route(T, E, k, seed=T)
+        x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(torch.float16)
+        out = ext.moe_experts_relu2(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV),
+                                    *stack(ups), inter, hidden, *stack(dns), hidden, inter)
+        _check(out, O.moe_reference(x.float().numpy(), idx, w, Wup, Wdn, act="relu2"), torch.float16)
+
+
+def test_moe_config4_all_128_experts():
+    """The 35B-A3B-shape layer with all 128 experts resident (hidden 2048, gate/up 2048->768, top-8): 1 and 8 tokens."""
+    E, hidden, inter = 128, 2048, 768
+    gu, dn, Wgu, Wdn = _experts(E, hidden, inter, 2e-3, seed=7000)
+    mod = QVBandExpertsV8(gu, dn, num_experts=E)
+    for T in (1, 8):
+        idx, w = _route(T, E, 8, seed=30 + T)
+        x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(torch.bfloat16)
+        out = mod(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
+        _check(out, O.moe_reference(x.float().numpy(), idx, w, Wgu, Wdn), torch.bfloat16)
