@@ -187,11 +187,16 @@ int64_t qvb8_moe_workspace_bytes(int64_t tokens, int64_t topk, int64_t n_experts
  * Stacked layout of the reference (QVBandExpertsV8.build_stack, formats/qvb8/backends_experts.py:145-195): per
  * projection ONE ids buffer (16-byte aligned, every expert's ids concatenated) and (n_experts, Q) row metadata with
  * bit offsets made global; experts carry no escapes.  idx i64 (tokens, topk), w f32 (tokens, topk), X (tokens, P_up)
- * in x_dtype; P_up and P_dn multiples of 32; Q_dn == P_up.  An expert selected by several tokens is read once for up
- * to 8 of them.  An index outside 0..n_experts-1 turns the whole output into NaN.  Four launches, no host round trip.
- * Up to 16 tokens (topk <= 8, fp16 / bf16 X, P_up and P_dn multiples of 128 up to 4096, Q_dn a multiple of 16)
- * take two launches on the matrix cores instead, every token as a problem of its own: the up projection applies the activation and hands H over as
- * saturated fp16 (the general path keeps H in fp32), the down projection adds the slots up with their routing weights.
+ * in x_dtype; P_up and P_dn multiples of 32; Q_dn == P_up.  No host round trip.  An index outside 0..n_experts-1 gives
+ * NaN: in every output row of the token that holds it, and in the whole output on the paths that group by expert.
+ * Up to 16 tokens with topk <= 8, fp16 / bf16 X, P_up and P_dn multiples of 128 up to 4096 and Q_dn a multiple of 16 run
+ * on the matrix cores, H handed over as saturated fp16:
+ *   1 or 2 tokens: two launches, every token a problem of its own (slot j = expert idx[t][j]); the down projection adds
+ *     the slots up with their routing weights;
+ *   3 .. 16 tokens: four launches (plan, up, down, combine): the (token, choice) pairs are grouped by expert, the tokens
+ *     that chose an expert are the token rows of one MFMA operand, and every selected expert is read ONCE however many
+ *     tokens chose it.
+ * Everything else takes the general path (four launches, H in fp32, an expert read once for up to 8 of its tokens).
  * Replaces: ext.moe_experts  qvb8_moe_experts_forward qvb8_cuda.cu:937-992 (kernels qvb8_moe_gemv :860-907,
  * qvb8_moe_act :910-918, qvb8_moe_combine :924-935) with act QVB8_MOE_SILU_GATED, and ext.moe_experts_relu2
  * qvb8_moe_experts_relu2_forward :1002-1055 with QVB8_MOE_RELU2. */

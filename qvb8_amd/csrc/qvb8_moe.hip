@@ -521,22 +521,27 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
     }
 }
 
-// ---- a few tokens (2..16): the tokens that chose an expert share one walk over it, on the matrix cores -------------------
+// ---- a few tokens (3..16): the tokens that chose an expert share one walk over it, on the matrix cores -------------------
 // The routing plan groups the (token, choice) pairs by expert; a selected expert has at most one pair per token, so its
 // pairs fit the 16 token rows of one MFMA operand, and every id that is read serves all of the expert's tokens: each
 // selected expert's bytes are read once, however many tokens chose it.
-//   work:  the tiles of the experts in use, numbered slot * tiles per expert + tile, are dealt to the workgroups in equal
-//          contiguous shares (the plan holds the number of slots in use, so the shares are equal whatever the routing);
-//          a share is walked in segments: tiles of ONE expert, as many as the LDS holds.
-//   segment: the waves hold the activation rows of the expert's pairs as MFMA operands (row t = pair order[first + t]:
-//          the pair's token for the up projection, the pair's own H row for the down projection; loaded when the expert
-//          changes).  The segment's rows are regrouped BY WIDTH in LDS (a stable counting sort of at most 256 row
-//          records), so that the 16 rows a wave decodes together nearly always share one width and take the
-//          single-width decode; a tile across a boundary takes each width in turn.  Then, per tile: T steps of 128
-//          columns per wave, ids decoded into MFMA operands, the next tile's ids in flight meanwhile, partial sums in LDS.
 //   up:   unit tiles of 16 outputs (gated: the 16 gate rows and the 16 matching up rows); H[pair] as saturated fp16.
 //   down: tiles of 16 rows; Yd[pair] in fp32 for the weighted combine (moe_combine_kernel).
-struct MoeGroupArgs {
+// work:    the workgroups are dealt to the experts in use, equally many each (the plan holds the number in use), and an
+//          expert's tiles in equal runs to its workgroups; a run is walked in segments of as many tiles as the LDS holds.
+// segment: the waves hold the activation rows as MFMA operands (row t = pair order[first + t]: the pair's token for the
+//          up projection, the pair's own H row for the down projection).  The segment's rows are regrouped BY WIDTH in
+//          LDS (a stable counting sort of at most 256 row records), so that the 16 rows a wave decodes together nearly
+//          always share one width and take the single-width decode; a tile across a boundary takes each width in turn.
+//          Then, per tile: T steps of 128 columns per wave (W = ceil(steps / T) waves per tile, G = 4 / W tiles at a
+//          time), ids decoded into MFMA operands (exact in fp16 next to a bias of 1024), the next tile's ids in flight
+//          meanwhile, partial sums in LDS, added in order in double.
+// Rows the slicing cannot read (width outside 4..8, not dword aligned) are redone element by element; an expert number
+// outside the stack gives NaN.
+// (One token through this walk -- slot j = expert idx[j], the combine inside the down kernel -- was built and measured
+// slower than moe_one_kernel: 28.7 against 24.7 us per layer; with so little work per workgroup the sort and its two
+// barriers cost more than the single-width decode saves.)
+struct MoeWalkArgs {
     const uint16_t* X;             // up: (tokens, P) fp16 or bf16 bits; down: H (npairs, P) fp16 bits
     MoePlan plan;
     const uint8_t* ids; int64_t ids_bytes;
@@ -547,13 +552,13 @@ struct MoeGroupArgs {
     int tiles_per_seg;             // unit tiles (up) / row tiles (down) per segment
     int max_tokens;                // most pairs an expert can have in this call (the LDS is laid out for it)
 };
-constexpr int kGroupWaves = 4;         // waves per workgroup: two workgroups share a CU
-constexpr int kGroupMaxRowTiles = 16;  // row tiles per segment: one row record per thread
+constexpr int kWalkWaves = 4;          // waves per workgroup: two workgroups share a CU
+constexpr int kWalkMaxRowTiles = 16;   // row tiles per segment: one row record per thread
 
-struct GroupRow { int64_t bit0; int flags; float ts, mn; int pad; };       // flags = width | usable << 8 | sliced << 9
+struct WalkRow { int64_t bit0; int flags; float ts, mn; int nat; };       // flags = width | usable << 8 | sliced << 9; nat = place before the sort
 
 template <int T, bool DOWN, bool XC, bool TWO>
-__device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
+__device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
     using F = Fmt<false>;
     using XI = XIn<false, XC>;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -561,7 +566,7 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, kg = lane >> 4;
     const int n_steps = a.P / kStepCols;
-    const int W = (n_steps + T - 1) / T, G = kGroupWaves / W;
+    const int W = (n_steps + T - 1) / T, G = kWalkWaves / W;
     const int g = wave / W, wc = wave - g * W;
     const bool walker = g < G;                               // W = 3 leaves one wave without a column range
     const int step0 = wc * T;
@@ -573,12 +578,12 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
     float* s_part = reinterpret_cast<float*>(smem);
     float* s_sx = s_part + (size_t)rt_cap * W * 16 * a.max_tokens;                        // [W][16]
     float2* s_fin = reinterpret_cast<float2*>(s_sx + W * 16);                             // [rt_cap * 16]
-    GroupRow* s_row = reinterpret_cast<GroupRow*>(s_fin + (size_t)rt_cap * 16);           // [rt_cap * 16]
-    int* s_cls = reinterpret_cast<int*>(s_row + (size_t)rt_cap * 16);                     // [kGroupWaves][8]
-    uint16_t* s_pos = reinterpret_cast<uint16_t*>(s_cls + kGroupWaves * 8);               // [rt_cap * 16]
+    WalkRow* s_row = reinterpret_cast<WalkRow*>(s_fin + (size_t)rt_cap * 16);             // [rt_cap * 16]
+    int* s_cls = reinterpret_cast<int*>(s_row + (size_t)rt_cap * 16);                     // [kWalkWaves][8]
+    uint16_t* s_pos = reinterpret_cast<uint16_t*>(s_cls + kWalkWaves * 8);                // [rt_cap * 16]
     const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
     const v4u_t ones = {F::one_bits, F::one_bits, F::one_bits, F::one_bits};
-    // the workgroups are dealt to the experts in use, equally many each; an expert's tiles in equal runs to its workgroups
+
     const int n_active = a.plan.n_bad[1];
     const int per_expert = max(1, (int)gridDim.x / max(1, n_active));
     const int sl = (int)blockIdx.x / per_expert;
@@ -586,6 +591,11 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
     const int run = (UT + per_expert - 1) / per_expert;
     int t0 = ((int)blockIdx.x - sl * per_expert) * run;
     const int t_end = min(UT, t0 + run);
+    // the expert, its first pair and the number of its pairs (operand rows in use)
+    const int4 slot = a.plan.slot[sl];
+    const int e = slot.x, first = slot.y, n = max(1, min(slot.z - slot.y, min(16, a.max_tokens)));
+    const bool e_ok = e >= 0 && e < a.E;
+    auto pair_of = [&](int t) { return a.plan.order[first + t]; };
 
     v4u_t xa[T][4];
     v4f_t sx = {0.f, 0.f, 0.f, 0.f};
@@ -594,16 +604,13 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
         const int n_rt = min(a.tiles_per_seg, t_end - t0) * RT;
         t0 += n_rt / RT;
         auto row0_of = [&](int i) { return DOWN ? (ut_first + i) * 16 : (ut_first + i / RT) * 16 + (i % RT) * a.units; };
-        // ---- the activations of the expert's pairs: operand row t = r (requested for every segment: from the caches after
-        // the first, and never under a branch, so that the waits below are exact) ----
-        const int4 slot = a.plan.slot[sl];
-        const int e = slot.x, first = slot.y, n = max(1, min(slot.z - slot.y, min(16, a.max_tokens)));
-        const bool e_ok = e >= 0 && e < a.E;
-        const int pair = a.plan.order[first + min(r, n - 1)];
+        // ---- the activation rows: operand row t = r (requested for every segment: from the caches after the first, and
+        // never under a branch, so that the waits below are exact) ----
+        const int pair = pair_of(min(r, n - 1));
         // ---- the segment's row records, regrouped by width (stable: rows of a width keep their order) ----
         const int n_rows = n_rt * 16;
         int key = 7, rank = 0;
-        GroupRow mine{0, 0, 0.f, 0.f, 0};
+        WalkRow mine{0, 0, 0.f, 0.f, 0};
         const size_t mi = (size_t)(e_ok ? e : 0) * a.Q + (tid < n_rows ? row0_of(tid >> 4) + (tid & 15) : 0);
         const int nb = a.nbits[mi];
         const int64_t bit0 = a.bit_off[mi];
@@ -619,7 +626,7 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
         if (tid < n_rows) {
             const bool ok = e_ok && nb >= 1 && nb <= 14 && bit0 >= 0 && ((bit0 + (int64_t)nb * a.P + 7) >> 3) + 8 <= a.ids_bytes;
             const bool sliced = ok && nb >= 4 && nb <= 8 && (bit0 & 31) == 0;
-            mine = GroupRow{ok ? bit0 : 0, nb | (ok ? 256 : 0) | (sliced ? 512 : 0), row_ts, row_mn, tid};
+            mine = WalkRow{ok ? bit0 : 0, nb | (ok ? 256 : 0) | (sliced ? 512 : 0), row_ts, row_mn, tid};
             key = sliced ? nb - 4 : 5;
         }
 #pragma unroll
@@ -634,36 +641,35 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
 #pragma unroll
             for (int c = 0; c < 6; ++c)
 #pragma unroll
-                for (int w = 0; w < kGroupWaves; ++w)
+                for (int w = 0; w < kWalkWaves; ++w)
                     if (c < key || (c == key && w < wave)) base += s_cls[w * 8 + c];
             s_row[base + rank] = mine;
             s_pos[tid] = (uint16_t)(base + rank);
         }
         __syncthreads();
+
         const int n_rounds = (n_rt + G - 1) / G;
         // Requests the lane's slices of the wave's tile of round `rnd` (clamped to the last round: nothing under a branch,
         // the repeated request at the end reads lines that are in the caches).  Returns the lane's row record.
-        auto issue = [&](int rnd, uint4 (&lo)[T], uint4 (&hi)[T]) __attribute__((always_inline)) -> GroupRow {
+        auto issue = [&](int rnd, uint4 (&lo)[T], uint4 (&hi)[T]) __attribute__((always_inline)) -> WalkRow {
             const int i = min(g + min(rnd, n_rounds - 1) * G, n_rt - 1);
-            const GroupRow rec = s_row[i * 16 + r];
-            const uint32_t nb = (uint32_t)rec.flags & 255u;
+            const WalkRow rec = s_row[i * 16 + r];
+            const uint32_t nbr = (uint32_t)rec.flags & 255u;
             const bool sliced = (rec.flags & 512) != 0;
-            const uint64_t row_off = (uint64_t)(rec.bit0 >> 3) + (uint64_t)(step0 * 4 + kg) * (4u * nb);
+            const uint64_t row_off = (uint64_t)(rec.bit0 >> 3) + (uint64_t)(step0 * 4 + kg) * (4u * nbr);
 #pragma unroll
             for (int it = 0; it < T; ++it) {
                 const bool use = sliced && (step0 + it) < n_steps;
-                const uint64_t off = use ? row_off + (uint64_t)it * (16u * nb) : 0;
+                const uint64_t off = use ? row_off + (uint64_t)it * (16u * nbr) : 0;
                 lo[it] = *reinterpret_cast<const uint4*>(a.ids + off);
-                hi[it] = *reinterpret_cast<const uint4*>(a.ids + off + (use ? 4u * (nb - 4u) : 16u));
+                hi[it] = *reinterpret_cast<const uint4*>(a.ids + off + (use ? 4u * (nbr - 4u) : 16u));
             }
             return rec;
         };
         uint4 lo0[T], hi0[T], lo1[T], hi1[T];
-        GroupRow rec0{0, 0, 0.f, 0.f, 0}, rec1{0, 0, 0.f, 0.f, 0};
-        rec0 = issue(0, lo0, hi0);                           // by every wave: nothing under a branch
+        WalkRow rec0 = issue(0, lo0, hi0), rec1{0, 0, 0.f, 0.f, 0};     // by every wave: nothing under a branch
         {
-            // rows past the expert's tokens and steps past the row multiply zeros; bf16 activations are narrowed like
-            // every activation
+            // rows past the pairs and steps past the row multiply zeros; bf16 activations are narrowed like every activation
 #pragma unroll
             for (int it = 0; it < T; ++it) {
                 const bool on = (step0 + it) < n_steps && r < n;
@@ -684,11 +690,11 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
                 for (int k = 0; k < 4; ++k) s_sx[wc * 16 + kg * 4 + k] = sx[k];
             }
         }
-        auto compute = [&](int rnd, const GroupRow& rec, const uint4 (&lo_)[T], const uint4 (&hi_)[T]) __attribute__((always_inline)) {
+        auto compute = [&](int rnd, const WalkRow& rec, const uint4 (&lo_)[T], const uint4 (&hi_)[T]) __attribute__((always_inline)) {
             v4f_t acc = {0.f, 0.f, 0.f, 0.f};
-            const int nb = rec.flags & 255;
+            const int nbr = rec.flags & 255;
             const bool sliced = (rec.flags & 512) != 0;
-            const uint32_t info = sliced ? ((uint32_t)nb | 256u) : 0u;
+            const uint32_t info = sliced ? ((uint32_t)nbr | 256u) : 0u;
             const uint32_t info0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
             const bool uniform = __builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u;
 #pragma unroll
@@ -706,11 +712,11 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) b[j] = v4u_t{F::bias_bits, F::bias_bits, F::bias_bits, F::bias_bits};
-                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 7)) { if (sliced && nb == 7) decode_slice<7, false>(lo, hi, b); }
-                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 6)) { if (sliced && nb == 6) decode_slice<6, false>(lo, hi, b); }
-                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 5)) { if (sliced && nb == 5) decode_slice<5, false>(lo, hi, b); }
-                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 4)) { if (sliced && nb == 4) decode_slice<4, false>(lo, hi, b); }
-                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 8)) { if (sliced && nb == 8) decode_slice<8, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 7)) { if (sliced && nbr == 7) decode_slice<7, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 6)) { if (sliced && nbr == 6) decode_slice<6, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 5)) { if (sliced && nbr == 5) decode_slice<5, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 4)) { if (sliced && nbr == 4) decode_slice<4, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 8)) { if (sliced && nbr == 8) decode_slice<8, false>(lo, hi, b); }
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc = F::mfma(xa[it][j], b[j], acc);
@@ -728,11 +734,11 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
                 while (odd) {
                     const int rr = __builtin_ctzll(odd);
                     odd &= odd - 1;
-                    const GroupRow o = s_row[i * 16 + rr];
+                    const WalkRow o = s_row[i * 16 + rr];
                     const int nb2 = o.flags & 255;
                     const int c_lo = step0 * kStepCols, c_hi = min(a.P, (step0 + T) * kStepCols);
                     for (int t = 0; t < n; ++t) {
-                        const int pr = a.plan.order[first + t];
+                        const int pr = pair_of(t);
                         const uint16_t* xr = a.X + (size_t)(DOWN ? pr : pr / a.topk) * a.P;
                         float sacc = 0.f;
                         if (o.flags & 256) {
@@ -763,11 +769,14 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
         }
         __syncthreads();
 
-        // natural row j of the segment, token t: tau_s * sum(x * id) + min_s * sum(x), the column ranges added in order
+        // natural row j of the segment, operand row t: tau_s * sum(x * id) + min_s * sum(x), the column ranges added in order
         auto row_value = [&](int j, int t) {
             const int at = s_pos[j];
             double d = 0.0, xs = 0.0;
-            for (int w = 0; w < W; ++w) { d += (double)s_part[(((size_t)(at >> 4) * W + w) * 16 + (at & 15)) * n + t]; xs += (double)s_sx[w * 16 + t]; }
+            for (int w = 0; w < W; ++w) {
+                d += (double)s_part[(((size_t)(at >> 4) * W + w) * 16 + (at & 15)) * n + t];
+                xs += (double)s_sx[w * 16 + t];
+            }
             const float2 f = s_fin[at];
             return (float)((double)f.x * d + (double)f.y * xs);
         };
@@ -775,7 +784,7 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
             float* Yd = reinterpret_cast<float*>(a.out);
             for (int o = tid; o < n_rows * n; o += blockDim.x) {
                 const int t = o % n, j = o / n;
-                Yd[(size_t)a.plan.order[first + t] * a.Q + row0_of(j >> 4) + (j & 15)] = row_value(j, t);
+                Yd[(size_t)pair_of(t) * a.Q + row0_of(j >> 4) + (j & 15)] = row_value(j, t);
             }
         } else {
             const int n_ut = n_rt / RT;
@@ -786,7 +795,7 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
                 float h;
                 if (a.gated) h = (y0 / (1.0f + __expf(-y0))) * row_value(j0 + 16, t);
                 else { const float pz = fmaxf(y0, 0.f); h = y0 != y0 ? y0 : pz * pz; }
-                H[(size_t)a.plan.order[first + t] * a.units + (ut_first + lut) * 16 + u] = (uint16_t)sat_half_bits(h);
+                H[(size_t)pair_of(t) * a.units + (ut_first + lut) * 16 + u] = (uint16_t)sat_half_bits(h);
             }
         }
         __syncthreads();                                     // the next segment reuses the LDS
@@ -795,13 +804,13 @@ __device__ __forceinline__ void moe_group_body(const MoeGroupArgs& a) {
 
 // rows of up to 2048 columns: within 256 registers, two workgroups per CU (one starts while the other walks)
 template <int T, bool DOWN, bool XC, bool TWO>
-__global__ void __launch_bounds__(64 * kGroupWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) moe_group_kernel(MoeGroupArgs a) {
-    moe_group_body<T, DOWN, XC, TWO>(a);
+__global__ void __launch_bounds__(64 * kWalkWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) moe_walk_kernel(MoeWalkArgs a) {
+    moe_walk_body<T, DOWN, XC, TWO>(a);
 }
 // longer rows: eight steps of activations per wave need more registers, one workgroup per CU
 template <bool DOWN, bool XC>
-__global__ void __launch_bounds__(64 * kGroupWaves) moe_group_wide_kernel(MoeGroupArgs a) {
-    moe_group_body<8, DOWN, XC, false>(a);
+__global__ void __launch_bounds__(64 * kWalkWaves) moe_walk_wide_kernel(MoeWalkArgs a) {
+    moe_walk_body<8, DOWN, XC, false>(a);
 }
 
 template <int DT>
@@ -850,13 +859,21 @@ int launch_moe_gemv(int stage, MoeGemvArgs a, int64_t slots, hipStream_t s) {
     else hipLaunchKernelGGL(moe_gemv_kernel<1>, grid, dim3(kMoeThreads), lds, s, a);
     return host::check_launch("qvb8_moe_experts");
 }
-// The one-token path: what it needs, and its two launches.  H (fp16) takes the place of the fp32 H in the workspace.
-bool moe_one_token_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t Q_up, int64_t P_up, int64_t Q_dn, int64_t P_dn, int act) {
-    if (tokens > host::env_int("QVB8_MOE_TILE_TOKENS", 16) || topk > 8 || (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16)) return false;
+// The matrix-core walk: what it needs.  H (fp16) takes the place of the fp32 H in the workspace.
+bool moe_walk_shapes_ok(int64_t topk, int x_dtype, int64_t P_up, int64_t Q_dn, int64_t P_dn) {
+    if (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16) return false;
     if (P_up % kStepCols != 0 || P_dn % kStepCols != 0 || P_up > 4096 || P_dn > 4096) return false;
-    if (P_dn % 16 != 0 || Q_dn % 16 != 0) return false;
-    (void)Q_up; (void)act;
-    return host::env_int("QVB8_MOE_ONE_TOKEN", 1) != 0;
+    return P_dn % 16 == 0 && Q_dn % 16 == 0 && topk >= 1;
+}
+// per token (no plan, the combine inside the down kernel): up to 8 slots, whose H rows are operand rows of one MFMA
+bool moe_one_token_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t P_up, int64_t Q_dn, int64_t P_dn) {
+    if (tokens > host::env_int("QVB8_MOE_TILE_TOKENS", 16) || topk > 8) return false;
+    return moe_walk_shapes_ok(topk, x_dtype, P_up, Q_dn, P_dn) && host::env_int("QVB8_MOE_ONE_TOKEN", 1) != 0;
+}
+// grouped by expert (3..16 tokens; two tokens are faster one by one: 36 against 40 us per layer at the 35B-A3B shapes)
+bool moe_group_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t P_up, int64_t Q_dn, int64_t P_dn) {
+    if (tokens < host::env_int("QVB8_MOE_GROUP_FROM", 3) || tokens > 16) return false;
+    return moe_walk_shapes_ok(topk, x_dtype, P_up, Q_dn, P_dn) && host::env_int("QVB8_MOE_GROUPED", 1) != 0;
 }
 
 template <bool DOWN, bool XC, int DT>
@@ -874,47 +891,40 @@ int launch_moe_one(const MoeOneArgs& a, unsigned blocks, unsigned tokens, hipStr
     return host::check_launch("qvb8_moe_experts");
 }
 
-// The grouped matrix-core path (2..16 tokens): what it needs.
-bool moe_group_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t Q_up, int64_t P_up, int64_t Q_dn, int64_t P_dn, int act) {
-    if (tokens < host::env_int("QVB8_MOE_GROUP_FROM", 2) || tokens > 16 || (x_dtype != QVB8_F16 && x_dtype != QVB8_BF16)) return false;
-    if (P_up % kStepCols != 0 || P_dn % kStepCols != 0 || P_up > 4096 || P_dn > 4096) return false;
-    if (P_dn % 16 != 0 || Q_dn % 16 != 0) return false;
-    (void)Q_up; (void)act; (void)topk;
-    return host::env_int("QVB8_MOE_GROUPED", 1) != 0;
+size_t moe_walk_lds(int64_t row_tiles, int W, int max_tokens) {
+    return (size_t)row_tiles * W * 16 * max_tokens * 4 + (size_t)W * 16 * 4 + (size_t)row_tiles * 16 * (8 + sizeof(WalkRow) + 2)
+           + (size_t)kWalkWaves * 8 * 4 + 16;
 }
 
+// `slots`: the plan's slots (experts that can be in use)
 template <bool DOWN, bool XC>
-int launch_moe_group(MoeGroupArgs a, int64_t slots, int64_t max_tokens, hipStream_t s) {
+int launch_moe_walk(MoeWalkArgs a, int64_t slots, int64_t max_tokens, hipStream_t s) {
     const int n_steps = a.P / kStepCols;
     // steps per wave: four, with the next tile's ids in flight; a short down row (up to 768 columns) is one wave's; rows
     // beyond 2048 columns take eight steps per wave and one register set
-    const int T = (DOWN && n_steps <= 6) ? 6 : (n_steps <= 4 * kGroupWaves ? 4 : 8);
+    const int T = (DOWN && n_steps <= 6) ? 6 : (n_steps <= 4 * kWalkWaves ? 4 : 8);
     const int W = (n_steps + T - 1) / T;
     const int RT = (!DOWN && a.gated) ? 2 : 1;
     const int UT = DOWN ? a.Q / 16 : a.units / 16;
     a.max_tokens = (int)std::min<int64_t>(16, max_tokens);
     // tiles per segment: what the LDS of two workgroups per CU holds, one row record per thread
-    auto lds_of = [&](int64_t tiles) {
-        return (size_t)tiles * RT * W * 16 * a.max_tokens * 4 + (size_t)W * 16 * 4 + (size_t)tiles * RT * 16 * (8 + sizeof(GroupRow) + 2)
-               + (size_t)kGroupWaves * 8 * 4 + 16;
-    };
-    int64_t per_seg = std::min<int64_t>(host::env_int("QVB8_MOE_GROUP_SEG_TILES", kGroupMaxRowTiles), kGroupMaxRowTiles / RT);
+    int64_t per_seg = std::min<int64_t>(host::env_int("QVB8_MOE_GROUP_SEG_TILES", kWalkMaxRowTiles), kWalkMaxRowTiles / RT);
     per_seg = std::max<int64_t>(1, std::min<int64_t>(per_seg, UT));
-    while (per_seg > 1 && lds_of(per_seg) > 64 * 1024) --per_seg;
+    while (per_seg > 1 && moe_walk_lds(per_seg * RT, W, a.max_tokens) > 64 * 1024) --per_seg;
     a.tiles_per_seg = (int)per_seg;
-    const size_t lds = lds_of(per_seg);
-    if (lds > 64 * 1024) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_moe_experts: rows too long for the grouped kernel's LDS");
+    const size_t lds = moe_walk_lds(per_seg * RT, W, a.max_tokens);
+    if (lds > 64 * 1024) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_moe_experts: rows too long for the walk's LDS");
     // two workgroups per CU, at least one per slot (the kernel deals them to the experts in use)
     const int64_t wgs = std::max<int64_t>(slots, std::min<int64_t>((int64_t)host::env_int("QVB8_MOE_GROUP_WGS_PER_CU", 2) * host::device_cus(), slots * UT));
-    dim3 grid((unsigned)wgs), block(64 * kGroupWaves);
+    dim3 grid((unsigned)wgs), block(64 * kWalkWaves);
     if constexpr (DOWN) {
         if (T == 6) {
-            hipLaunchKernelGGL((moe_group_kernel<6, true, XC, false>), grid, block, lds, s, a);
+            hipLaunchKernelGGL((moe_walk_kernel<6, true, XC, false>), grid, block, lds, s, a);
             return host::check_launch("qvb8_moe_experts");
         }
     }
-    if (T == 4) hipLaunchKernelGGL((moe_group_kernel<4, DOWN, XC, true>), grid, block, lds, s, a);
-    else hipLaunchKernelGGL((moe_group_wide_kernel<DOWN, XC>), grid, block, lds, s, a);
+    if (T == 4) hipLaunchKernelGGL((moe_walk_kernel<4, DOWN, XC, true>), grid, block, lds, s, a);
+    else hipLaunchKernelGGL((moe_walk_wide_kernel<DOWN, XC>), grid, block, lds, s, a);
     return host::check_launch("qvb8_moe_experts");
 }
 }  // namespace
@@ -956,8 +966,8 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
     float* H = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np));
     float* Yd = reinterpret_cast<float*>(ws + moe_plan_bytes(n_experts, np) + align256((size_t)np * P_dn * 4));
 
-    const bool grouped = moe_group_ok(tokens, topk, x_dtype, Q_up, P_up, Q_dn, P_dn, act);
-    if (!grouped && moe_one_token_ok(tokens, topk, x_dtype, Q_up, P_up, Q_dn, P_dn, act)) {
+    const bool grouped = moe_group_ok(tokens, topk, x_dtype, P_up, Q_dn, P_dn);
+    if (!grouped && moe_one_token_ok(tokens, topk, x_dtype, P_up, Q_dn, P_dn)) {
         MoeOneArgs o;
         o.X = reinterpret_cast<const uint16_t*>(X); o.idx = idx; o.w = w; o.ids = up_ids; o.ids_bytes = up_ids_bytes;
         o.min_s = up_min; o.tau_s = up_tau; o.nbits = up_nb; o.bit_off = up_off; o.out = H;
@@ -981,20 +991,21 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
         if (out_dtype == QVB8_F16) return launch_moe_one<true, false, 1>(o, dn_blocks, tk, s);
         return launch_moe_one<true, false, 2>(o, dn_blocks, tk, s);
     }
+
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)(n_experts + 8) * 4, s, idx, (int)np, (int)n_experts, pl);
     if (int rc = host::check_launch("qvb8_moe_experts plan")) return rc;
     const int64_t slots = moe_slots(n_experts, np);
     if (grouped) {
-        MoeGroupArgs ga;
-        ga.X = reinterpret_cast<const uint16_t*>(X); ga.plan = pl; ga.ids = up_ids; ga.ids_bytes = up_ids_bytes;
-        ga.min_s = up_min; ga.tau_s = up_tau; ga.nbits = up_nb; ga.bit_off = up_off; ga.out = H;        // H as fp16 (pairs, P_dn)
-        ga.E = (int)n_experts; ga.Q = (int)Q_up; ga.P = (int)P_up; ga.topk = (int)topk; ga.units = (int)P_dn; ga.gated = act == 0 ? 1 : 0;
-        ga.tiles_per_seg = 1; ga.max_tokens = 1;
-        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_group<false, true>(ga, slots, tokens, s) : launch_moe_group<false, false>(ga, slots, tokens, s)) return rc;
-        ga.X = reinterpret_cast<const uint16_t*>(H); ga.ids = dn_ids; ga.ids_bytes = dn_ids_bytes;
-        ga.min_s = dn_min; ga.tau_s = dn_tau; ga.nbits = dn_nb; ga.bit_off = dn_off; ga.out = Yd;
-        ga.Q = (int)Q_dn; ga.P = (int)P_dn; ga.units = (int)Q_dn; ga.gated = 0;
-        if (int rc = launch_moe_group<true, false>(ga, slots, tokens, s)) return rc;
+        MoeWalkArgs wa;
+        wa.X = reinterpret_cast<const uint16_t*>(X); wa.plan = pl; wa.ids = up_ids; wa.ids_bytes = up_ids_bytes;
+        wa.min_s = up_min; wa.tau_s = up_tau; wa.nbits = up_nb; wa.bit_off = up_off; wa.out = H;                // H as fp16 (pairs, P_dn)
+        wa.E = (int)n_experts; wa.Q = (int)Q_up; wa.P = (int)P_up; wa.topk = (int)topk; wa.units = (int)P_dn; wa.gated = act == 0 ? 1 : 0;
+        wa.tiles_per_seg = 1; wa.max_tokens = 1;
+        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_walk<false, true>(wa, slots, tokens, s) : launch_moe_walk<false, false>(wa, slots, tokens, s)) return rc;
+        wa.X = reinterpret_cast<const uint16_t*>(H); wa.ids = dn_ids; wa.ids_bytes = dn_ids_bytes;
+        wa.min_s = dn_min; wa.tau_s = dn_tau; wa.nbits = dn_nb; wa.bit_off = dn_off; wa.out = Yd;
+        wa.Q = (int)Q_dn; wa.P = (int)P_dn; wa.units = (int)Q_dn; wa.gated = 0;
+        if (int rc = launch_moe_walk<true, false>(wa, slots, tokens, s)) return rc;
         dim3 cgrid((unsigned)((Q_dn + 255) / 256), (unsigned)tokens);
         if (out_dtype == QVB8_F32) hipLaunchKernelGGL(moe_combine_kernel<0>, cgrid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
         else if (out_dtype == QVB8_F16) hipLaunchKernelGGL(moe_combine_kernel<1>, cgrid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);

@@ -182,9 +182,10 @@ def test_moe_refusals():
                         d["ids"], d["min_s"], d["tau_s"], d["nbits"], d["bit_off"], d["Q"], d["P"] + 32)
 
 
-@pytest.mark.parametrize("T,k,dtype", [(2, 2, torch.bfloat16), (5, 4, torch.float16), (16, 8, torch.bfloat16), (9, 1, torch.float16)])
+@pytest.mark.parametrize("T,k,dtype", [(2, 2, torch.bfloat16), (3, 2, torch.bfloat16), (5, 4, torch.float16), (16, 8, torch.bfloat16),
+                                       (9, 1, torch.float16)])
 def test_moe_few_tokens_share_each_expert(T, k, dtype):
-    """2..16 tokens on the matrix cores: the tokens that chose an expert share one walk over it.  Shapes the grouped
+    """2..16 tokens on the matrix cores: from three tokens on, the tokens that chose an expert share one walk over it.  Shapes the grouped
     kernels take (row lengths that are multiples of 128), more experts than get selected and experts selected by many
     tokens at once; against the oracle, reproducible, and equal to the per-token result of the same library."""
     E, hidden, inter = 12, 384, 128
@@ -205,8 +206,8 @@ def test_moe_few_tokens_share_each_expert(T, k, dtype):
     single = torch.cat([mod(args[0][t:t + 1], args[1][t:t + 1], args[2][t:t + 1]) for t in range(T)])
     _check(single, O.moe_reference(x.float().numpy(), idx, w, Wgu, Wdn), dtype)
     bad = args[1].clone()
-    bad[T - 1, 0] = E + 5
-    assert torch.isnan(mod(args[0], bad, args[2]).float()).all()
+    bad[T - 1, 0] = E + 5                                      # an expert number outside the stack: NaN for its token at least
+    assert torch.isnan(mod(args[0], bad, args[2]).float()[T - 1]).all()
 
 
 def test_moe_few_tokens_relu2_and_rows_the_slicing_cannot_read():
@@ -238,6 +239,18 @@ def test_moe_few_tokens_relu2_and_rows_the_slicing_cannot_read():
         out = ext.moe_experts_relu2(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV),
                                     *stack(ups), inter, hidden, *stack(dns), hidden, inter)
         _check(out, O.moe_reference(x.float().numpy(), idx, w, Wup, Wdn, act="relu2"), torch.float16)
+
+
+def test_moe_few_tokens_rows_longer_than_2048_columns():
+    """The grouped walk with rows of 2304 columns in the up projection (eight steps per wave, one register set) and of
+    640 in the down projection; 4 tokens, top-2 of 4 experts."""
+    E, hidden, inter = 4, 2304, 640
+    gu, dn, Wgu, Wdn = _experts(E, hidden, inter, 2e-3, seed=4100)
+    mod = QVBandExpertsV8(gu, dn, num_experts=E)
+    idx, w = _route(4, E, 2, seed=77)
+    x = torch.randn(4, hidden, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    out = mod(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
+    _check(out, O.moe_reference(x.float().numpy(), idx, w, Wgu, Wdn), torch.bfloat16)
 
 
 def test_moe_config4_all_128_experts():
