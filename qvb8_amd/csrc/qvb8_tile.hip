@@ -474,9 +474,12 @@ struct GemmArgs {
 };
 
 // grid (M, splits): sx[z][m] = sum of row m of X over column range z, as the operands see it; XC: X16[m] = the row narrowed
+// tile_rows > 0: X16 is written for every operand format, stage by stage -- [block of tile_rows rows][P / 64][tile_rows][64 columns] -- so that
+// the 64 columns of all rows that a workgroup stages together are one contiguous run (rows of a row-major X are a
+// multiple of 4 KB apart: the same few L2 channels for every row of a stage, asked by every workgroup at once)
 template <bool BF, bool XC>
 __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t* __restrict__ X, int M, int P, int cols_per_split,
-                                                        uint16_t* __restrict__ X16, float* __restrict__ sx) {
+                                                        uint16_t* __restrict__ X16, float* __restrict__ sx, int tile_rows) {
     __shared__ float red[4];
     const int m = blockIdx.x, z = blockIdx.y, tid = threadIdx.x;
     const int c_begin = z * cols_per_split, c_end = min(P, c_begin + cols_per_split);
@@ -489,7 +492,8 @@ __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t* __restri
             w[k] = XIn<BF, XC>::pair(w[k]);
             part += Fmt<BF>::to_f32(w[k] & 0xFFFFu) + Fmt<BF>::to_f32(w[k] >> 16);
         }
-        if constexpr (XC) *reinterpret_cast<uint4*>(X16 + (size_t)m * P + c) = uint4{w[0], w[1], w[2], w[3]};
+        if (tile_rows > 0) *reinterpret_cast<uint4*>(X16 + (((size_t)(m / tile_rows) * (P >> 6) + (c >> 6)) * tile_rows + m % tile_rows) * 64 + (c & 63)) = uint4{w[0], w[1], w[2], w[3]};
+        else if constexpr (XC) *reinterpret_cast<uint4*>(X16 + (size_t)m * P + c) = uint4{w[0], w[1], w[2], w[3]};
     }
     part = wave_sum(part);
     if ((tid & 63) == 0) red[tid >> 6] = part;
@@ -644,6 +648,220 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     }
 }
 
+// ---- fused decode + GEMM through LDS, M = 65..256 ----------------------------------------------------------------------
+// With this many rows of X every weight must serve many of them once it has been read and decoded: a workgroup takes 128
+// weight rows of ONE width x BM rows of X (256: all of X, or 128) x one range of columns, and every id it fetches is
+// decoded once, into LDS.  Its 16 waves have two jobs:
+//   waves 8..15 fill LDS.  X (stored stage by stage by gemm_prep_kernel): per 64-column stage, 16-byte pieces into the
+//         stage's A buffer ([row of X][64 columns], two buffers), requested four stages before they are stored.  ids:
+//         per 128-column block, a thread fetches the 32-id slice g of a row (two 16-byte loads; four neighbouring lanes
+//         read 16 NB contiguous bytes), decodes it into 32 `bias + id` halves and writes them to the block's B buffer
+//         ([weight row][128 columns], two buffers); requested two blocks before they are decoded.
+//   waves 0..7 multiply.  Wave (wm, wn) owns 64 rows of X x 32 NT weight rows (NT = 2 for BM = 256, 1 for BM = 128): per
+//         16 columns two A operands and NT B operands from LDS (rows padded by 16 bytes: conflict-free 16-byte reads)
+//         feed 2 NT v_mfma_f32_32x32x16.  A wave issues in order and both the LDS requests (about 30 cycles each,
+//         measured) and the matrix instructions (32 cycles) hold its issue, so two multiplying waves share a SIMD: one
+//         requests operands while the other one's products run.
+// One barrier per stage, met by all 16 waves.  The end is the end of gemm_run: bias and min_s through the row sums of X
+// (gemm_prep_kernel), partial results per column range, added in order by gemm_reduce_kernel.
+constexpr int kG2Rows = 128, kG2Cols = 64, kG2Mul = 8, kG2Waves = 16, kG2Fill = 512;   // multiplying waves, all waves, filling threads
+constexpr int kG2AStride = kG2Cols * 2 + 16;                       // bytes per row of X of one stage
+constexpr int kG2BStride = 2 * kG2Cols * 2 + 16;                   // bytes per weight row of one 128-column block
+
+template <int WM, bool BF, int NB>
+__device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_end, int run_first, uint64_t run_byte0, unsigned char* smem) {
+    using F = Fmt<BF>;
+    constexpr int BM = 64 * WM, WN = kG2Mul / WM, NT = kG2Rows / (32 * WN);   // WM = 4: 256 rows of X, 64 x 64 sums per wave; WM = 2: 128 rows, 64 x 32
+    constexpr int MT = 2;
+    constexpr int XL = BM * 8 / kG2Fill;                           // 16-byte pieces of a stage per filling thread
+    unsigned char* As = smem;                                      // [2][BM][kG2AStride]
+    unsigned char* Bs = smem + (size_t)2 * BM * kG2AStride;        // [2][kG2Rows][kG2BStride]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tok0 = (int)blockIdx.y * BM;
+    const int s_begin = (int)blockIdx.z * a.stages_per_split * 2;  // stages_per_split counts 128-column stages
+    const int s_end = min(a.P / kG2Cols, s_begin + a.stages_per_split * 2);
+    const int n_st = s_end - s_begin;                              // a multiple of 4
+    if (n_st <= 0) return;
+    const int n_blk = n_st / 2;
+    const int wm = wave / WN, wn = wave - wm * WN;                 // of the multiplying waves
+    const int n = lane & 31, kh = lane >> 5;
+    v16f_t acc[MT][NT];
+
+    if (wave >= kG2Mul) {
+        // ================= filling =================
+        // Requests run far ahead of their use (X from L2, ids from HBM: one to two microseconds under load): four
+        // register sets of X pieces (stage s in set s % 4, requested four stages before it is stored), two of id slices
+        // (block b in set b % 2, requested two blocks before it is decoded).  Four stages per turn of the loop.
+        const int p = tid - 64 * kG2Mul;
+        // ids: slice g = p % 4 of row p / 4; a position past the run reads the run's last row (never stored)
+        const int dg = p & 3, drow = p >> 2;
+        const int dpos = min(pos0 + drow, pos_end - 1);
+        const uint8_t* const idp = a.ids + run_byte0 + (uint64_t)(dpos - run_first) * ((uint64_t)a.P * NB / 8)
+                                   + (uint64_t)(s_begin / 2) * (16u * NB) + (uint32_t)dg * (4u * NB);
+        uint4 raw[2][2];
+        auto request_ids = [&](int blk, uint4 (&w)[2]) __attribute__((always_inline)) {
+            const uint32_t off = (uint32_t)min(blk, n_blk - 1) * (16u * NB);
+            w[0] = *reinterpret_cast<const uint4*>(idp + off);
+            w[1] = *reinterpret_cast<const uint4*>(idp + off + 4u * (NB - 4u));
+        };
+        auto store_ids = [&](int buf, const uint4 (&w)[2]) __attribute__((always_inline)) {
+            v4u_t b[4];
+            decode_slice<NB, BF>(w[0], w[1], b);
+            unsigned char* dst = Bs + ((size_t)buf * kG2Rows + drow) * kG2BStride + 64 * dg;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) *reinterpret_cast<v4u_t*>(dst + 16 * j) = b[j];
+        };
+        // X, stored stage by stage ([block of BM rows][stage][BM rows][64 columns], gemm_prep_kernel): piece p % 8 (8
+        // columns) of rows p / 8 + 64 i of the block; rows past M read row M - 1 (not stored at the end)
+        const int xch = p & 7, xrow = p >> 3;
+        const int M = a.M;
+        const uint16_t* x_piece[XL];
+#pragma unroll
+        for (int i = 0; i < XL; ++i)
+            x_piece[i] = a.X + (((size_t)blockIdx.y * (a.P / kG2Cols) + s_begin) * BM + min(xrow + 64 * i, M - 1 - tok0)) * kG2Cols + 8 * xch;
+        v4u_t xg[4][XL];
+        auto request_x = [&](int st, v4u_t (&g)[XL]) __attribute__((always_inline)) {
+            const size_t c = (size_t)min(st, n_st - 1) * (BM * kG2Cols);
+#pragma unroll
+            for (int i = 0; i < XL; ++i) g[i] = *reinterpret_cast<const v4u_t*>(x_piece[i] + c);
+        };
+        auto store_x = [&](int buf, const v4u_t (&g)[XL]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < XL; ++i)
+                *reinterpret_cast<v4u_t*>(As + ((size_t)buf * BM + xrow + 64 * i) * kG2AStride + 16 * xch) = g[i];
+        };
+        request_x(0, xg[0]);
+        request_ids(0, raw[0]);
+        request_x(1, xg[1]);
+        request_ids(1, raw[1]);
+        request_x(2, xg[2]);
+        request_x(3, xg[3]);
+        store_x(0, xg[0]);
+        request_x(4, xg[0]);
+        store_ids(0, raw[0]);
+        request_ids(2, raw[0]);
+        __syncthreads();
+        for (int ls = 0; ls < n_st; ls += 4) {
+            const int blk = ls >> 1;                               // even
+            // stage ls is multiplied: X of stage ls + 1, ids of block blk + 1 (set 1) into B buffer 1
+            store_x(1, xg[1]);
+            request_x(ls + 5, xg[1]);
+            store_ids(1, raw[1]);
+            request_ids(blk + 3, raw[1]);
+            __syncthreads();
+            store_x(0, xg[2]);                                     // stage ls + 2
+            request_x(ls + 6, xg[2]);
+            __syncthreads();
+            store_x(1, xg[3]);                                     // stage ls + 3; ids of block blk + 2 (set 0) into B buffer 0
+            request_x(ls + 7, xg[3]);
+            store_ids(0, raw[0]);
+            request_ids(blk + 4, raw[0]);
+            __syncthreads();
+            store_x(0, xg[0]);                                     // stage ls + 4
+            request_x(ls + 8, xg[0]);
+            __syncthreads();
+        }
+    } else {
+        // ================= multiplying =================
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.f;
+        // Operands of 16 columns ahead of their products, in two register sets: the requests for the next 16 columns go to
+        // LDS before the matrix instructions of the current ones are issued (a wave issues in order, and the matrix
+        // pipe holds the issue for 32 cycles per instruction), and the last 16 columns of a stage are multiplied after
+        // the barrier, behind the first requests of the next stage.
+        auto operands = [&](int ls, int q, v4u_t (&av)[MT], v4u_t (&bv)[NT]) __attribute__((always_inline)) {
+            const unsigned char* Ab = As + ((size_t)(ls & 1) * BM + wm * (32 * MT) + n) * kG2AStride + 16 * kh + 32 * q;
+            const unsigned char* Bb = Bs + ((size_t)((ls >> 1) & 1) * kG2Rows + wn * (32 * NT) + n) * kG2BStride + (ls & 1) * (2 * kG2Cols) + 16 * kh + 32 * q;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) av[mt] = *reinterpret_cast<const v4u_t*>(Ab + (size_t)(32 * mt) * kG2AStride);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) bv[nt] = *reinterpret_cast<const v4u_t*>(Bb + (size_t)(32 * nt) * kG2BStride);
+        };
+        auto products = [&](const v4u_t (&av)[MT], const v4u_t (&bv)[NT]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = F::mfma32(av[mt], bv[nt], acc[mt][nt]);
+        };
+        v4u_t av0[MT], bv0[NT], av1[MT], bv1[NT];
+        __syncthreads();
+        operands(0, 0, av0, bv0);
+        for (int ls = 0; ls < n_st; ++ls) {
+            operands(ls, 1, av1, bv1);
+            __builtin_amdgcn_sched_barrier(0);
+            products(av0, bv0);
+            __builtin_amdgcn_sched_barrier(0);
+            operands(ls, 2, av0, bv0);
+            __builtin_amdgcn_sched_barrier(0);
+            products(av1, bv1);
+            __builtin_amdgcn_sched_barrier(0);
+            operands(ls, 3, av1, bv1);
+            __builtin_amdgcn_sched_barrier(0);
+            products(av0, bv0);
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            operands(ls + 1, 0, av0, bv0);                     // past the last stage: a buffer nobody writes any more, never used
+            __builtin_amdgcn_sched_barrier(0);
+            products(av1, bv1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // ---- the end: a multiplying lane holds, for weight row n of each row tile, rows of X 32 mt + 8 (i / 4) + 4 kh + i % 4 ----
+    float* sxs = reinterpret_cast<float*>(smem);                   // the buffers are no longer read (barrier above)
+    if (tid < BM) sxs[tid] = tok0 + tid < a.M ? a.sx[(size_t)blockIdx.z * a.M + tok0 + tid] : 0.f;
+    __syncthreads();
+    if (wave >= kG2Mul) return;
+    float* out = a.out + (size_t)blockIdx.z * (size_t)a.M * (size_t)a.Q;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int pos = pos0 + wn * (32 * NT) + 32 * nt + n;
+        if (pos >= pos_end) continue;
+        const uint4 f = a.fin[pos];
+        if (f.z >= (uint32_t)a.Q) continue;
+        const double ts = (double)__uint_as_float(f.x), mn = (double)__uint_as_float(f.y);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int tl = wm * (32 * MT) + 32 * mt + 8 * (i >> 2) + 4 * kh + (i & 3);
+                const int t = tok0 + tl;
+                if (t < a.M) {
+                    const float sx = sxs[tl];
+                    const float d = __builtin_fmaf(-F::bias, sx, acc[mt][nt][i]);
+                    out[(size_t)t * a.Q + f.z] = (float)(ts * (double)d + mn * (double)sx);
+                }
+            }
+    }
+}
+
+template <int WM, bool BF>
+__global__ void __launch_bounds__(64 * kG2Waves) gemm2_kernel(GemmArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    // which run of equal widths this workgroup's 128 positions belong to
+    const int bx = (int)blockIdx.x;
+    const int c = (bx >= a.blocks1 ? 1 : 0) + (bx >= a.blocks2 ? 1 : 0);
+    const uint32_t nb0 = a.widths & 255u, nb1 = (a.widths >> 8) & 255u, nb2 = (a.widths >> 16) & 255u;
+    const uint64_t row0 = (uint64_t)a.P * nb0 / 8, row1 = (uint64_t)a.P * nb1 / 8;
+    const int run_first = c == 0 ? 0 : c == 1 ? a.first1 : a.first2;
+    const int run_end = c == 0 ? a.first1 : c == 1 ? a.first2 : a.Q;
+    const uint64_t byte0 = c == 0 ? 0 : c == 1 ? (uint64_t)a.first1 * row0 : (uint64_t)a.first1 * row0 + (uint64_t)(a.first2 - a.first1) * row1;
+    const int pos0 = run_first + (bx - (c == 0 ? 0 : c == 1 ? a.blocks1 : a.blocks2)) * kG2Rows;
+    if (pos0 >= run_end) return;
+    switch (c == 0 ? nb0 : c == 1 ? nb1 : nb2) {
+        case 4: gemm2_run<WM, BF, 4>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 5: gemm2_run<WM, BF, 5>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 6: gemm2_run<WM, BF, 6>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 7: gemm2_run<WM, BF, 7>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 8: if constexpr (!BF) gemm2_run<WM, BF, 8>(a, pos0, run_end, run_first, byte0, smem); break;
+        default: break;
+    }
+}
+
 // Y = sum of the column ranges' partial results, in ascending order
 __global__ void __launch_bounds__(256) gemm_reduce_kernel(const float* __restrict__ part, float* __restrict__ Y, int64_t n, int splits) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -781,6 +999,37 @@ GemmPlan plan_gemm(int64_t M, int64_t Q, int64_t P) {
     return g;
 }
 
+// The kernel that stages decoded weights in LDS: one block of rows of X (M <= 256), 128 weight rows per workgroup, column
+// ranges for about one workgroup per CU (it holds most of a CU's LDS).
+int gemm2_from() { const int v = host::env_int("QVB8_GEMM_LDS_FROM", 65); return v < 33 ? 33 : v; }
+GemmPlan plan_gemm2(int64_t M, int64_t Q, int64_t P) {
+    GemmPlan g;
+    g.row_blocks = (int)((Q + kG2Rows - 1) / kG2Rows);
+    // All of X in one block of 256 rows when the weight alone has row blocks for most of the chip; otherwise blocks of 128
+    // rows of X: twice the workgroups before any column range is split off, and half the partial results to add up.
+    const int mt_env = host::env_int("QVB8_GEMM_MT", 0);
+    g.MT = mt_env == 2 || mt_env == 4 ? mt_env : ((M > 128 && 2 * g.row_blocks >= (int)host::device_cus()) ? 4 : 2);
+    const int BM = 64 * g.MT;
+    g.tok_blocks = (int)((M + BM - 1) / BM);
+    const int64_t groups = P / (2 * kGemmStageCols);
+    const int64_t base = (int64_t)g.row_blocks * g.tok_blocks;
+    const int64_t target = host::env_int("QVB8_GEMM_TARGET_WGS", 0) > 0 ? host::env_int("QVB8_GEMM_TARGET_WGS", 0) : (int64_t)host::device_cus();
+    int64_t splits = (target + base / 2) / base;
+    if (splits > groups) splits = groups;
+    if (splits > 16) splits = 16;
+    if (splits < 1) splits = 1;
+    const int64_t groups_per_split = (groups + splits - 1) / splits;
+    g.stages_per_split = (int)(2 * groups_per_split);
+    g.splits = (int)((groups + groups_per_split - 1) / groups_per_split);
+    g.lds = (size_t)2 * BM * kG2AStride + (size_t)2 * kG2Rows * kG2BStride;
+    g.x16_at = align256i(qvb8_mma_rowinfo_bytes(Q));
+    g.sx_at = g.x16_at + align256i((int64_t)g.tok_blocks * BM * P * 2);    // X stage by stage, in blocks of BM rows
+    g.part_at = g.sx_at + align256i((int64_t)g.splits * M * 4);
+    g.bytes = g.part_at + (g.splits > 1 ? (int64_t)g.splits * M * Q * 4 : 0);
+    return g;
+}
+GemmPlan plan_gemm_for(int64_t M, int64_t Q, int64_t P) { return M >= gemm2_from() ? plan_gemm2(M, Q, P) : plan_gemm(M, Q, P); }
+
 // Fewest rows of X that go to the workgroup-tiled kernel when it can read the weight (49..: always; below that the tile
 // kernel is the alternative).
 int gemm_from() { const int v = host::env_int("QVB8_MMA_GEMM_FROM", 33); return v < 17 ? 17 : (v > 49 ? 49 : v); }
@@ -796,6 +1045,20 @@ int launch_gemm(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_
         attr[dev] = true;
     }
     hipLaunchKernelGGL((gemm_kernel<MT, BF>), dim3((unsigned)row_blocks, (unsigned)g.tok_blocks, (unsigned)g.splits), dim3(256), g.lds, s, a);
+    return host::check_launch("qvb8_mma");
+}
+
+template <int WM, bool BF>
+int launch_gemm2(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_t s) {
+    static bool attr[64] = {false};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: no current device");
+    if (!attr[dev]) {
+        if (hipFuncSetAttribute((const void*)gemm2_kernel<WM, BF>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds) != hipSuccess)
+            return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: cannot raise the kernel's LDS limit");
+        attr[dev] = true;
+    }
+    hipLaunchKernelGGL((gemm2_kernel<WM, BF>), dim3((unsigned)row_blocks, (unsigned)g.tok_blocks, (unsigned)g.splits), dim3(64 * kG2Waves), g.lds, s, a);
     return host::check_launch("qvb8_mma");
 }
 }  // namespace
@@ -838,7 +1101,7 @@ extern "C" int qvb8_mma_prepare(const uint8_t* nbits, const int64_t* bit_off, co
 }
 
 extern "C" int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P) {
-    if (M >= gemm_from() && M <= 256 && Q > 0 && P > 0 && (P % (2 * kGemmStageCols)) == 0) return plan_gemm(M, Q, P).bytes;
+    if (M >= gemm_from() && M <= 256 && Q > 0 && P > 0 && (P % (2 * kGemmStageCols)) == 0) return plan_gemm_for(M, Q, P).bytes;
     return qvb8_mma_rowinfo_bytes(Q);
 }
 
@@ -894,7 +1157,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     // can read the weight and the caller brought its workspace.
     bool tiled = M > 48;
     if (!tiled && M >= gemm_from() && layout && (P % (2 * kGemmStageCols)) == 0 && workspace
-        && workspace_bytes >= plan_gemm(M, Q, P).bytes && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
+        && workspace_bytes >= plan_gemm_for(M, Q, P).bytes && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
         tiled = true;
         for (int c = 0; c < a.n_classes; ++c) tiled = tiled && a.nb[c] >= 4 && a.nb[c] <= (mode == 2 ? 7 : 8);
     }
@@ -904,7 +1167,8 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         for (int c = 0; c < a.n_classes; ++c)
             if (a.nb[c] < 4 || a.nb[c] > (mode == 2 ? 7 : 8))
                 return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: M > 48 needs widths 4..8 (4..7 on bf16 operands), found %d", a.nb[c]);
-        const GemmPlan g = plan_gemm(M, Q, P);
+        const bool staged = M >= gemm2_from();
+        const GemmPlan g = plan_gemm_for(M, Q, P);
         if (!workspace || workspace_bytes < g.bytes || (reinterpret_cast<uintptr_t>(workspace) & 15u))
             return host::fail(QVB8_ERR_WORKSPACE, "qvb8_mma: M=%lld needs %lld bytes of 16-byte aligned workspace", (long long)M, (long long)g.bytes);
         unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
@@ -913,20 +1177,25 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         float* out = g.splits > 1 ? reinterpret_cast<float*>(ws + g.part_at) : Y;
         const int cols_per_split = g.stages_per_split * kGemmStageCols;
         const dim3 pgrid((unsigned)M, (unsigned)g.splits);
-        if (mode == 0) hipLaunchKernelGGL((gemm_prep_kernel<false, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx);
-        else if (mode == 1) hipLaunchKernelGGL((gemm_prep_kernel<false, true>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx);
-        else hipLaunchKernelGGL((gemm_prep_kernel<true, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx);
+        const int tile_rows = staged ? 64 * g.MT : 0;                 // the staged kernel reads X stage by stage
+        if (mode == 0) hipLaunchKernelGGL((gemm_prep_kernel<false, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx, tile_rows);
+        else if (mode == 1) hipLaunchKernelGGL((gemm_prep_kernel<false, true>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx, tile_rows);
+        else hipLaunchKernelGGL((gemm_prep_kernel<true, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx, tile_rows);
         if (int rc2 = host::check_launch("qvb8_mma activations")) return rc2;
         GemmArgs ga;
-        ga.X = mode == 1 ? x16 : a.X; ga.ids = ids; ga.fin = a.fin; ga.sx = sx; ga.out = out;
+        ga.X = (mode == 1 || staged) ? x16 : a.X; ga.ids = ids; ga.fin = a.fin; ga.sx = sx; ga.out = out;
         ga.M = (int)M; ga.Q = (int)Q; ga.P = (int)P; ga.stages_per_split = g.stages_per_split;
         ga.first1 = a.first1; ga.first2 = a.first2;
         const int rows0 = a.first1, rows1 = a.first2 - a.first1, rows2 = (int)Q - a.first2;
-        ga.blocks1 = (rows0 + kGemmRows - 1) / kGemmRows;
-        ga.blocks2 = ga.blocks1 + (rows1 + kGemmRows - 1) / kGemmRows;
-        const int row_blocks = ga.blocks2 + (rows2 + kGemmRows - 1) / kGemmRows;
+        const int br = staged ? kG2Rows : kGemmRows;                  // weight rows per workgroup
+        ga.blocks1 = (rows0 + br - 1) / br;
+        ga.blocks2 = ga.blocks1 + (rows1 + br - 1) / br;
+        const int row_blocks = ga.blocks2 + (rows2 + br - 1) / br;
         ga.widths = (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16);
-        if (g.MT == 4) rc = mode == 2 ? launch_gemm<4, true>(ga, g, row_blocks, s) : launch_gemm<4, false>(ga, g, row_blocks, s);
+        if (staged) {
+            if (g.MT == 4) rc = mode == 2 ? launch_gemm2<4, true>(ga, g, row_blocks, s) : launch_gemm2<4, false>(ga, g, row_blocks, s);
+            else rc = mode == 2 ? launch_gemm2<2, true>(ga, g, row_blocks, s) : launch_gemm2<2, false>(ga, g, row_blocks, s);
+        } else if (g.MT == 4) rc = mode == 2 ? launch_gemm<4, true>(ga, g, row_blocks, s) : launch_gemm<4, false>(ga, g, row_blocks, s);
         else rc = mode == 2 ? launch_gemm<2, true>(ga, g, row_blocks, s) : launch_gemm<2, false>(ga, g, row_blocks, s);
         if (rc) return rc;
         if (g.splits > 1) {
