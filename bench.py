@@ -37,6 +37,9 @@ TAU = 1e-3
 # plus WRITE_SIZE), as recorded in profiles/tile_kernel_9b_decode_step_hbm_traffic.md, by launch class
 MEASURED_TRAFFIC = {"q+k+v": (2 * 10999.9 + 33.2) * 1024, "fused-other": (2 * 24196.5 + 59.7) * 1024,      # default
                     256: (2 * 16078.3 + 39.8) * 1024, 64: (2 * 2014.4 + 4.9) * 1024}                        # --no-fuse
+# symbols per second of the QVB8R walk with the activations and the multiply-adds taken out (same launch shape, the 65B
+# shapes, one row of X), measured once on this hardware: the ceiling the fused kernel is compared with
+WALK_CEILING_TSYM = 1.814
 MMA_FLAGS = int(os.environ.get("QVB8_BENCH_MMA_FLAGS", "1"))     # 1 = QVB8_MMA_SATURATE_X: the operator's default for bf16 x
 
 
@@ -301,7 +304,10 @@ def _time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name):
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                          "kernel": kernel,
                          "bytes_per_launch": step_bytes // len(units), "launch_us": round(launch_us, 3),
-                         "note": "the walk is bound by dependent LDS lookups and a 64-bit multiply per symbol, not by HBM"},
+                         "note": "the walk is bound by its instruction count (vector ALU 91 % busy), not by HBM"},
+            "roofline_walk": {"bound": "rANS walk alone (slot lookup, 64-bit state update, ballot / popcount, ring read) at this launch shape",
+                              "achieved": round(n_sym / (ms * 1e-3) / 1e12, 4), "peak": WALK_CEILING_TSYM, "unit": "T symbols/s",
+                              "frac": round(n_sym / (ms * 1e-3) / 1e12 / WALK_CEILING_TSYM, 4)},
             "cpu_baseline": None}
 
 

@@ -21,6 +21,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/qvb8_amd.h"
 #include "qvb8_device.h"
 #include "qvb8_host.h"
@@ -193,10 +195,10 @@ __global__ void __launch_bounds__(kRThreads) r_gemv_kernel(RCore c, const void* 
     __syncthreads();
     const int S = c.P >> 5;
     float sx = 0.f;                  // sum of x over this lane's columns (the same for every row): taken while the first row is walked
-    for (int r = 0; r < T; ++r) {
-        if (!(t.has && r < t.nr)) continue;                                // per half-wave
-        const int orow = c.perm[t.r0 + r];
-        const bool row_ok = orow >= 0 && orow < c.Q;
+    // one row: the walk with two multiply-adds per pair; FIRST also adds the activations up (a second copy of the loop
+    // instead of a test per pair: the loop is bound by its instruction count)
+    auto walk_row = [&](auto first) __attribute__((always_inline)) {
+        constexpr bool FIRST = decltype(first)::value;
         float acc = 0.f;
         float x1 = load_as_f32<DT>(X, l32), x2 = load_as_f32<DT>(X, 32 + l32);
         for (int s0 = 0; s0 < S; s0 += 2) {
@@ -206,10 +208,17 @@ __global__ void __launch_bounds__(kRThreads) r_gemv_kernel(RCore c, const void* 
             walk_pair(z, st, rg, l32, half, t.room, s1, s2);
             acc = __builtin_fmaf(x1, (float)s1, acc);
             acc = __builtin_fmaf(x2, (float)s2, acc);
-            if (r == 0) sx += x1 + x2;
+            if constexpr (FIRST) sx += x1 + x2;
             x1 = n1; x2 = n2;
         }
-        if (r == 0) sx = half_sum(sx);
+        if constexpr (FIRST) sx = half_sum(sx);
+        return acc;
+    };
+    for (int r = 0; r < T; ++r) {
+        if (!(t.has && r < t.nr)) continue;                                // per half-wave
+        const int orow = c.perm[t.r0 + r];
+        const bool row_ok = orow >= 0 && orow < c.Q;
+        const float acc = r == 0 ? walk_row(std::true_type{}) : walk_row(std::false_type{});
         const double m = row_ok ? (double)c.min_s[orow] : 0.0, ts = row_ok ? (double)c.tau_s[orow] : 0.0;
         const double dr = row_ok ? (double)c.drow[orow] : 0.0;
         const float a = half_sum(acc);
