@@ -33,14 +33,35 @@ LAYER_9B = (("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096,
 LAYER_27B = (("q", 5120, 5120), ("k", 1024, 5120), ("v", 1024, 5120), ("o", 5120, 5120),
              ("gate", 17408, 5120), ("up", 17408, 5120), ("down", 5120, 17408))
 TAU = 1e-3
-# HBM bytes per launch of the tile kernel from hardware counters (FETCH_SIZE scaled by 2.0 against a plain 1 GiB pass,
-# plus WRITE_SIZE), as recorded in profiles/tile_kernel_9b_decode_step_hbm_traffic.md, by launch class
-MEASURED_TRAFFIC = {"q+k+v": (2 * 10999.9 + 33.2) * 1024, "fused-other": (2 * 24196.5 + 59.7) * 1024,      # default
-                    256: (2 * 16078.3 + 39.8) * 1024, 64: (2 * 2014.4 + 4.9) * 1024}                        # --no-fuse
+def measured_traffic(profile, kernel):
+    """HBM bytes per launch by launch class, from the `traffic_bytes_per_launch <kernel> <class> <bytes>` lines of a
+    summary under profiles/ (hardware counters, recorded there with the commands that took them); {} without the file."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", profile)
+    out = {}
+    try:
+        with open(path) as fh:
+            for line in fh:
+                f = line.split()
+                if len(f) == 4 and f[0] == "traffic_bytes_per_launch" and f[1] == kernel:
+                    out[f[2]] = int(f[3])
+    except OSError:
+        pass
+    return out
+
+
 # symbols per second of the QVB8R walk with the activations and the multiply-adds taken out (same launch shape, the 65B
 # shapes, one row of X), measured once on this hardware: the ceiling the fused kernel is compared with
 WALK_CEILING_TSYM = 1.814
 MMA_FLAGS = int(os.environ.get("QVB8_BENCH_MMA_FLAGS", "1"))     # 1 = QVB8_MMA_SATURATE_X: the operator's default for bf16 x
+
+
+def tile_traffic(units, n_launch):
+    """Mean measured HBM bytes per launch of the step's launch mix (None when the counters' summary is not there)."""
+    t = measured_traffic("tile_kernel_9b_decode_step_hbm_traffic.md", "tile_kernel")
+    cls = {"q+k+v": "q+k+v", "o": "o,gate+up", "gate+up": "o,gate+up", "down": "down"}
+    if any(cls.get(u["name"]) not in t for u in units):
+        return None
+    return round(sum(t[cls[u["name"]]] for u in units) / n_launch)
 
 
 def algorithmic_bytes(enc, M):
@@ -228,8 +249,12 @@ def bench_moe(args, dev):
                                    "tau=2e-3, %d token(s), %d layers x %d routings per step" % (T, args.layers, rounds),
                        "bytes_per_step": step_bytes, "us_per_layer": round(per_layer_us, 2)},
             "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                         "kernel": ("qvb8::moe_one_kernel<4,false,..> + moe_one_kernel<6,true,..> (one layer = 2 launches)" if T <= 16 else
+                         "frac": round(gbs / HBM_PEAK_GBS, 4),
+                         # HBM bytes of one layer's launches from hardware counters, where the summary holds this token count
+                         "traffic": measured_traffic("moe_kernels_35b_a3b_layer_kernel_trace.md", "moe_layer").get("tokens=%d" % T),
+                         "kernel": ("qvb8::moe_one_kernel<4,false,..> + moe_one_kernel<6,true,..> (one layer = 2 launches)" if T <= 2 else
+                                    "qvb8::moe_plan_kernel + moe_walk_kernel<4,false,..> + moe_walk_kernel<6,true,..> + "
+                                    "moe_combine_kernel (one layer = 4 launches)" if T <= 16 else
                                     "qvb8::moe_plan_kernel + moe_gemv_kernel<0> + moe_gemv_kernel<1> + moe_combine_kernel "
                                     "(one layer = 4 launches)"),
                          "bytes_per_launch": step_bytes // n_calls, "launch_us": round(per_layer_us, 3)},
@@ -594,7 +619,7 @@ def run_legs(args, dev, layers, units):
     import copy
     import gc
     import torch
-    keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "tflops", "dtype", "roofline", "config")
+    keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "tflops", "dtype", "roofline", "roofline_walk", "config")
     legs = {}
     sub = copy.copy(args)
     sub.steps, sub.warmup = max(5, min(args.steps, 20)), 3
@@ -732,9 +757,7 @@ def main():
                    "bits_per_weight": round(8.0 * sum(u["lin"].ids.numel() for u in units) / sum(e["Q"] * e["P"] for e in flat), 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": (None if MMA_FLAGS != 1 or args.model != "9b" else
-                                 round(sum(MEASURED_TRAFFIC[256 if e["Q"] >= 4096 else 64] for e in flat) / n_launch) if args.no_fuse
-                                 else round(sum(MEASURED_TRAFFIC["q+k+v" if u["name"] == "q+k+v" else "fused-other"] for u in units) / n_launch)),
+                     "traffic": tile_traffic(units, n_launch) if (MMA_FLAGS == 1 and args.model == "9b" and not args.no_fuse) else None,
                      "kernel": "qvb8::tile_kernel<1,4,false,true,XP> (XP = 1 or 4 pieces of X per thread through LDS)" + (" / <1,5,false,true,XP> for 5120-column rows" if args.model == "27b" else ""),
                      "bytes_per_launch": step_bytes // n_launch,
                      "launch_us": round(launch_us, 3)},
