@@ -111,10 +111,14 @@ int qvb8_gemv(const void* X, int x_dtype, int64_t M,
 /* ---- fused decode + small-M GEMM on the matrix cores, M = 1..48 (and 49..256, see qvb8_mma) ---------------- */
 
 enum qvb8_mma_flags {
-    QVB8_MMA_SATURATE_X = 1   /* bf16 X is narrowed as saturating_half does (clamp to +-65504, round to fp16, NaN kept) while
+    QVB8_MMA_SATURATE_X = 1,  /* bf16 X is narrowed as saturating_half does (clamp to +-65504, round to fp16, NaN kept) while
                                  it is loaded, and the product runs on fp16 operands: what the fp16 paths of the reference
                                  multiply.  Without it bf16 X is used as it is, on bf16 operands (the reference's bf16
                                  mode).  No effect on fp16 X. */
+    QVB8_MMA_Y_F16 = 2,       /* Y is (M, Q) fp16: each result rounded to nearest even from the fp32 value the call would */
+    QVB8_MMA_Y_BF16 = 4       /* otherwise store; likewise bf16.  Only for a weight without escapes (n_esc == 0): the escape
+                                 correction adds to fp32 results.  Saves the caller's cast pass over Y (the reference's
+                                 operator casts the extension's fp32 result, formats/qvb8/module.py:430-441). */
 };
 
 /* Row records of the matrix-core path: qvb8_mma_rowinfo_bytes(Q) bytes (24 per row, 8-byte aligned), in tile order

@@ -33,6 +33,13 @@ namespace qvb8 {
 constexpr uint64_t kRowOffMask = (1ull << 48) - 1;
 __host__ __device__ inline size_t rowinfo_loc_words(int64_t Q) { return (size_t)((Q + 1) & ~(int64_t)1); }
 
+// a result into Y in the caller's format (wave-uniform choice)
+__device__ __forceinline__ void store_y(float* Y, int out_dt, int64_t i, float v) {
+    if (out_dt == 0) Y[i] = v;
+    else if (out_dt == 1) store_from_f32<1>(Y, i, v);
+    else store_from_f32<2>(Y, i, v);
+}
+
 struct TileArgs {
     const uint16_t* X;            // (M, P) fp16 or bf16 bits
     const uint8_t* ids;
@@ -41,6 +48,7 @@ struct TileArgs {
     float* Y;                     // (M, Q) fp32
     int64_t ids_bytes;
     int M, Q, P;
+    int out_dt;                   // what Y holds: 0 fp32, 1 fp16, 2 bf16
     int n_steps;                  // P / 128
     int W, G, panels;             // waves per tile, tile groups per workgroup, column panels
     int TW;                       // tiles per workgroup (multiple of G)
@@ -101,7 +109,7 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
     TileArgs a;
     a.X = X; a.ids = ids; a.loc = loc; a.fin = reinterpret_cast<const uint4*>(loc + rowinfo_loc_words(Q)); a.Y = Y;
     a.ids_bytes = ids_bytes; a.Q = Q; a.P = P; a.n_steps = P / kStepCols; a.TW = TW;
-    a.M = (int)(counts & 63u); a.W = (int)((counts >> 8) & 15u); a.G = (int)((counts >> 12) & 15u); a.panels = (int)(counts >> 16);
+    a.M = (int)(counts & 63u); a.out_dt = (int)((counts >> 6) & 3u); a.W = (int)((counts >> 8) & 15u); a.G = (int)((counts >> 12) & 15u); a.panels = (int)(counts >> 16);
     a.first1 = first1; a.first2 = first2; a.n_classes = (int)(widths >> 24);
     a.nb[0] = (int)(widths & 255u); a.nb[1] = (int)((widths >> 8) & 255u); a.nb[2] = (int)((widths >> 16) & 255u);
     using F = Fmt<BF>;
@@ -415,7 +423,7 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
             dsum += (double)part[((size_t)rl * ranges + w) * MS + t];
             xsum += (double)sxs[w * TM + t];
         }
-        a.Y[(size_t)t * a.Q + f.z] = (float)((double)__uint_as_float(f.x) * dsum + (double)__uint_as_float(f.y) * xsum);
+        store_y(a.Y, a.out_dt, (int64_t)t * a.Q + f.z, (float)((double)__uint_as_float(f.x) * dsum + (double)__uint_as_float(f.y) * xsum));
     }
 }
 
@@ -467,6 +475,7 @@ struct GemmArgs {
     const float* sx;               // [splits][M] sums of X over each column range
     float* out;                    // Y (one column range) or the partial results [splits][M][Q]
     int M, Q, P;
+    int out_dt;                    // what `out` holds when there is one column range: 0 fp32, 1 fp16, 2 bf16 (partial results are fp32)
     int stages_per_split;          // even
     int first1, first2;            // positions where the second and the third width start (Q when there is none)
     int blocks1, blocks2;          // row blocks before the second / the third width (blocks of 256 positions from a width's first)
@@ -619,7 +628,7 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
                 if (t < a.M) {
                     const float sx = sxs[tl];
                     const float d = __builtin_fmaf(-F::bias, sx, acc[rt][mt][i]);
-                    out[(size_t)t * a.Q + f.z] = (float)(ts * (double)d + mn * (double)sx);
+                    store_y(out, a.out_dt, (int64_t)t * a.Q + f.z, (float)(ts * (double)d + mn * (double)sx));
                 }
             }
     }
@@ -833,7 +842,7 @@ __device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_e
                 if (t < a.M) {
                     const float sx = sxs[tl];
                     const float d = __builtin_fmaf(-F::bias, sx, acc[mt][nt][i]);
-                    out[(size_t)t * a.Q + f.z] = (float)(ts * (double)d + mn * (double)sx);
+                    store_y(out, a.out_dt, (int64_t)t * a.Q + f.z, (float)(ts * (double)d + mn * (double)sx));
                 }
             }
     }
@@ -863,12 +872,12 @@ __global__ void __launch_bounds__(64 * kG2Waves) gemm2_kernel(GemmArgs a) {
 }
 
 // Y = sum of the column ranges' partial results, in ascending order
-__global__ void __launch_bounds__(256) gemm_reduce_kernel(const float* __restrict__ part, float* __restrict__ Y, int64_t n, int splits) {
+__global__ void __launch_bounds__(256) gemm_reduce_kernel(const float* __restrict__ part, float* __restrict__ Y, int64_t n, int splits, int out_dt) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float v = part[i];
     for (int s = 1; s < splits; ++s) v += part[(int64_t)s * n + i];
-    Y[i] = v;
+    store_y(Y, out_dt, i, v);
 }
 
 }  // namespace qvb8
@@ -939,7 +948,7 @@ int launch_tile(TileArgs& a, hipStream_t s) {
         attr[dev] = true;
     }
     if (pl.panels > 0xffff) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: rows too long");
-    const uint32_t counts = (uint32_t)a.M | ((uint32_t)a.W << 8) | ((uint32_t)a.G << 12) | ((uint32_t)a.panels << 16);
+    const uint32_t counts = (uint32_t)a.M | ((uint32_t)a.out_dt << 6) | ((uint32_t)a.W << 8) | ((uint32_t)a.G << 12) | ((uint32_t)a.panels << 16);
     hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC, XP>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s,
                        a.X, a.ids, a.loc, a.Y, a.ids_bytes, a.Q, a.P, counts, a.TW, a.first1, a.first2,
                        (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16) | ((uint32_t)a.n_classes << 24));
@@ -1148,7 +1157,9 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         a.first2 = n > 2 ? layout->first_pos[2] : (int)Q;
         a.n_classes = n;
     }
-    a.Y = Y; a.ids_bytes = ids_bytes; a.M = (int)M; a.Q = (int)Q; a.P = (int)P; a.n_steps = (int)(P / kStepCols);
+    const int out_dt = (flags & QVB8_MMA_Y_F16) ? 1 : (flags & QVB8_MMA_Y_BF16) ? 2 : 0;
+    if (out_dt != 0 && n_esc > 0) return host::fail(QVB8_ERR_ARG, "qvb8_mma: fp16 / bf16 results need a weight without escapes (the correction adds to fp32 results)");
+    a.Y = Y; a.out_dt = out_dt; a.ids_bytes = ids_bytes; a.M = (int)M; a.Q = (int)Q; a.P = (int)P; a.n_steps = (int)(P / kStepCols);
     // mode 0: fp16 X, fp16 operands; 1: bf16 X narrowed to saturated fp16 on the way in, fp16 operands; 2: bf16 operands
     const int mode = x_dtype == QVB8_F16 ? 0 : (flags & QVB8_MMA_SATURATE_X) ? 1 : 2;
     int rc;
@@ -1185,6 +1196,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         GemmArgs ga;
         ga.X = (mode == 1 || staged) ? x16 : a.X; ga.ids = ids; ga.fin = a.fin; ga.sx = sx; ga.out = out;
         ga.M = (int)M; ga.Q = (int)Q; ga.P = (int)P; ga.stages_per_split = g.stages_per_split;
+        ga.out_dt = g.splits > 1 ? 0 : out_dt;
         ga.first1 = a.first1; ga.first2 = a.first2;
         const int rows0 = a.first1, rows1 = a.first2 - a.first1, rows2 = (int)Q - a.first2;
         const int br = staged ? kG2Rows : kGemmRows;                  // weight rows per workgroup
@@ -1200,7 +1212,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         if (rc) return rc;
         if (g.splits > 1) {
             const int64_t n = M * Q;
-            hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, out, Y, n, g.splits);
+            hipLaunchKernelGGL(gemm_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, out, Y, n, g.splits, out_dt);
             if (int rc2 = host::check_launch("qvb8_mma reduce")) return rc2;
         }
     } else {

@@ -172,6 +172,7 @@ def gemv(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals):
 MMA_MAX_M = 48
 MMA_GEMM_MAX_M = 256          # with a row layout (rows stored in width order, widths 4..8): the workgroup-tiled kernel
 MMA_SATURATE_X = 1
+MMA_Y_F16, MMA_Y_BF16 = 2, 4                      # qvb8_mma_flags: results stored as fp16 / bf16
 
 
 def mma_prepare(row_nbits, row_bit_off, tau_s, min_s, P, ids_bytes, perm=None):
@@ -238,14 +239,15 @@ def sort_rows_by_width(ids, row_nbits, row_bit_off, P, perm):
 
 
 def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm=None, saturate=True,
-              rowinfo=None, layout=None):
+              rowinfo=None, layout=None, out_dtype=None):
     """Matrix-core path for P % 128 == 0: X (fp16 or bf16) times the fp32 band value, fp32 (M, Q).  1 <= M <= 48 always;
     49 <= M <= 256 (the workgroup-tiled decode + GEMM kernel) when `layout` is given and its widths are 4..8.
     `perm` (int32, position -> row) groups rows of equal width into tiles; `rowinfo` = mma_prepare(...) for the
     same perm (built on the fly when absent); `layout` = the third result of sort_rows_by_width for a pack whose rows were
     copied into that order (needs `rowinfo`).  `saturate` (bf16 X only): X is narrowed like saturating_half while it
     is loaded and the product runs on fp16 operands, as every fp16 path of the reference does; without it bf16 X is
-    multiplied as it is on bf16 operands."""
+    multiplied as it is on bf16 operands.  `out_dtype` torch.float16 / torch.bfloat16: the kernels store the results
+    rounded to that type (the same values as casting the fp32 result; only for a weight without escapes)."""
     lib = _lib.load()
     Q = _check_pack(ids, min_s, row_nbits, row_bit_off, tau_s)
     n_esc = _check_escapes(esc_idx, esc_vals)
@@ -272,7 +274,15 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
     ids, min_s, tau_s = ids.contiguous(), min_s.contiguous(), tau_s.contiguous()
     row_nbits, row_bit_off = row_nbits.contiguous(), row_bit_off.contiguous()
     with torch.cuda.device(Xc.device):
-        Y = torch.empty((M, Q), dtype=torch.float32, device=Xc.device)
+        if out_dtype in (torch.float16, torch.bfloat16):
+            if n_esc:
+                raise RuntimeError("qvb8 mma-multi: fp16 / bf16 results need a weight without escapes")
+            y_flag = MMA_Y_F16 if out_dtype == torch.float16 else MMA_Y_BF16
+        elif out_dtype in (None, torch.float32):
+            out_dtype, y_flag = torch.float32, 0
+        else:
+            raise RuntimeError("qvb8 mma-multi: results are fp32, fp16 or bf16")
+        Y = torch.empty((M, Q), dtype=out_dtype, device=Xc.device)
         ei = esc_idx.contiguous() if n_esc else None
         ev = esc_vals.contiguous() if n_esc else None
         need = lib.qvb8_mma_workspace_bytes(M, Q, int(P))          # row records when none are passed; more for the tiled kernel
@@ -283,7 +293,7 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
                                  Q, int(P), _lib.ptr(ei), _lib.ptr(ev), n_esc, _lib.ptr(perm),
                                  None if rowinfo is None else rowinfo.contiguous().data_ptr(),
                                  None if layout is None else ctypes.addressof(layout),
-                                 MMA_SATURATE_X if saturate else 0, _lib.ptr(Y),
+                                 (MMA_SATURATE_X if saturate else 0) | y_flag, _lib.ptr(Y),
                                  None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel() * 8,
                                  _lib.stream_of(Xc)), lib)
     return Y

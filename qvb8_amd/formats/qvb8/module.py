@@ -288,8 +288,10 @@ class QVBandLinearV8(nn.Module):
         if order is not None:
             perm, rowinfo, layout = order
             xm = xk if xk.dtype in (torch.float16, torch.bfloat16) else ext.saturating_half(xk)
+            # without escapes and bias the kernels round the results to the caller's type themselves: no cast pass over Y
+            direct = out_dtype if (ei.numel() == 0 and self.bias is None and out_dtype in (torch.float16, torch.bfloat16)) else None
             y = ext.mma_tiles(xm, self.ids, self.min_s, self.nbits, self.bit_off, self.in_features, self.tau_s,
-                              ei, ev, perm=perm, saturate=not bf16_mode, rowinfo=rowinfo, layout=layout)
+                              ei, ev, perm=perm, saturate=not bf16_mode, rowinfo=rowinfo, layout=layout, out_dtype=direct)
             return self._finish(y, orig, out_dtype)
         if M <= 8:
             y = ext.gemv_multi(xk, self.ids, self.min_s, self.nbits, self.bit_off, self.in_features, self.tau_s,

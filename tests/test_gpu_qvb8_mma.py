@@ -184,6 +184,27 @@ def test_gemm_many_rows(M, mode):
     assert torch.equal(y, ext.mma_tiles(x, *args, perm=perm, saturate=mode != "bf16_operands", rowinfo=rowinfo, layout=layout))
 
 
+@pytest.mark.parametrize("M", [1, 16, 40, 64, 100, 256])
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16])
+def test_results_stored_as_16_bit_are_the_rounded_fp32_results(M, out_dtype):
+    """QVB8_MMA_Y_F16 / _BF16 on every kernel behind qvb8_mma (tile kernel, both GEMM kernels, one and several column
+    ranges): bit for bit what casting the fp32 result gives; refused for a weight with escapes."""
+    for Q, P in ((300, 768), (136, 2048)):
+        d = H.mixed_width_pack(Q, P, [7, 6, 5], seed=3 * M + Q)
+        d["tau_s"] = d["tau_s"] * (1.0 / 64)
+        args, perm, rowinfo, layout = _sorted_pack(d)
+        x = _x(M, P, torch.bfloat16, M)
+        kw = dict(perm=perm, saturate=True, rowinfo=rowinfo, layout=layout)
+        y32 = ext.mma_tiles(x, *args, **kw)
+        y16 = ext.mma_tiles(x, *args, out_dtype=out_dtype, **kw)
+        assert y16.dtype == out_dtype and torch.equal(y16, y32.to(out_dtype))
+    with_esc = list(args)
+    with_esc[6] = torch.tensor([5], dtype=torch.int64, device=DEV)
+    with_esc[7] = torch.tensor([0.25], dtype=torch.float32, device=DEV)
+    with pytest.raises(RuntimeError):
+        ext.mma_tiles(x, *with_esc, out_dtype=out_dtype, **kw)
+
+
 def test_gemm_needs_layout_and_sliceable_widths():
     d = H.mixed_width_pack(64, 256, [9, 6], seed=1)
     args, perm, rowinfo, layout = _sorted_pack(d)
