@@ -17,6 +17,18 @@
  *   nbits    u8[Q]          row width, 1..14    bit_off i64[Q]  absolute bit of the row's first id
  *   esc_idx  i64[n_esc]     flat positions q*P+c, ascending     esc_vals f32[n_esc]  exact values
  * value(q, c) = fmaf((float)id, tau_s[q], min_s[q]) in fp32, escapes overwrite.
+ *
+ * Rows stored in planes (optional, made by a loader; no counterpart in the reference, whose rows are always back to
+ * back).  16 rows of ONE width nb in 4..8 (P a multiple of 128) may share a TILE of 16 * P * nb / 8 bytes -- the bytes
+ * of the 16 rows, permuted -- laid out so that each 16-byte and each 4 (nb - 4)-byte request of a 64-lane wave of the
+ * matrix-core kernels is one contiguous run.  Call the nb dwords that hold ids 32 g .. 32 g + 31 of a row its slice g.
+ * The tile is a sequence of P / 128 steps of 256 nb bytes; step s holds slices 4 s .. 4 s + 3 of the 16 rows as
+ *   plane A, 64 x 16 bytes:          entry l = r + 16 (g mod 4) holds dwords 0..3 of slice g of row r;
+ *   plane B, 64 x 4 (nb - 4) bytes:  entry l holds dwords 4..nb-1 of that slice (empty for nb = 4).
+ * Row r of such a tile is marked in its bit_off word: bit 62 set, bits 0..47 = bit offset of the TILE's first byte (a
+ * multiple of 32), bits 48..51 = r.  Every entry point that takes a pack reads such rows (qvb8_gemv and the escape
+ * corrections id by id); qvb8_mma is told of them with QVB8_MMA_PLANES.  The expert stacks of qvb8_moe_experts do not
+ * take them (a marked row there comes out as NaN, like any row whose metadata points outside its buffer).
  */
 #ifndef QVB8_AMD_H
 #define QVB8_AMD_H
@@ -48,7 +60,8 @@ const char* qvb8_last_error(void);
 
 /* ---- dense restore ------------------------------------------------------------------------------------- */
 
-/* Dense (Q, P) restore, each value rounded ONCE to out_dtype: out[q*P+c] = (T)fmaf(id, tau_s[q], min_s[q]).
+/* Dense (Q, P) restore: out[q*P+c] = (T)fmaf(id, tau_s[q], min_s[q]) -- the fp32 result of the fused multiply-add,
+ * then that fp32 value rounded to out_dtype (two roundings for fp16 / bf16, as a cast of the reference's fp32 value gives).
  * Bit-exact with the reference restore.  Escapes are NOT applied (see qvb8_scatter_escapes).
  * Replaces: qvb8_decode_launch / qvb8_decode_all(_v3)  qvb8_cuda.cu:535-649; out_dtype QVB8_F16 = ext.decode
  * (:651-699), QVB8_BF16 = ext.decode_bf16 (:1711-1727), QVB8_F32 = the fp32 band value of decode.py:196-209. */
@@ -116,9 +129,13 @@ enum qvb8_mma_flags {
                                  multiply.  Without it bf16 X is used as it is, on bf16 operands (the reference's bf16
                                  mode).  No effect on fp16 X. */
     QVB8_MMA_Y_F16 = 2,       /* Y is (M, Q) fp16: each result rounded to nearest even from the fp32 value the call would */
-    QVB8_MMA_Y_BF16 = 4       /* otherwise store; likewise bf16.  Only for a weight without escapes (n_esc == 0): the escape
+    QVB8_MMA_Y_BF16 = 4,      /* otherwise store; likewise bf16.  Only for a weight without escapes (n_esc == 0): the escape
                                  correction adds to fp32 results.  Saves the caller's cast pass over Y (the reference's
                                  operator casts the extension's fp32 result, formats/qvb8/module.py:430-441). */
+    QVB8_MMA_PLANES = 8       /* the pack has rows stored in planes (bit 62 of their bit_off, see "rows stored in planes"
+                                 above): with a row layout these are the rows of every whole 16-row tile that lies inside
+                                 one run of a width 4..8; without one, whatever rows the records mark.  The call then asks
+                                 for ids in operand order with non-temporal loads. */
 };
 
 /* Row records of the matrix-core path: qvb8_mma_rowinfo_bytes(Q) bytes (24 per row, 8-byte aligned), in tile order

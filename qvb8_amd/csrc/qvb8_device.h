@@ -22,6 +22,10 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {      // round to
 }
 
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    // The fp32 value is rounded to fp16 as a step of its own: without the empty statement the compiler folds a preceding
+    // fused multiply-add into v_fma_mixlo_f16, which rounds the exact sum ONCE to fp16 and differs from
+    // fp16(fp32 result) where the fp32 rounding lands on an fp16 tie (about one value in 10^5).
+    asm("" : "+v"(f));
     _Float16 h = (_Float16)f;                                         // v_cvt_f16_f32, round to nearest even
     return (uint32_t)__builtin_bit_cast(uint16_t, h);
 }
@@ -68,6 +72,53 @@ __device__ __forceinline__ uint32_t load_field(const uint8_t* __restrict__ ids, 
     const uint64_t v = (uint64_t)p[0] | ((uint64_t)p[1] << 32);
     const uint32_t sh = (uint32_t)(bit - a * 8) & 63u;
     return (uint32_t)(v >> sh) & ((1u << nb) - 1u);
+}
+
+// ---- rows stored in planes ------------------------------------------------------------------------------------
+// A loader may store a 16-row tile of ONE width nb (4..8, P a multiple of 128) so that every request instruction of a
+// wave reads one contiguous run: per 128-column step first plane A -- the first four dwords of every lane's slice, lane
+// l = row + 16 * (column group of 32 within the step), 64 x 16 bytes -- then plane B, the remaining nb - 4 dwords of every
+// lane, 64 x 4 (nb - 4) bytes.  A step takes 256 nb bytes and a tile n_steps x 256 nb = 16 rows' worth: the same bytes
+// as 16 rows stored back to back, permuted inside the tile.  Such a row is marked in its bit offset:
+//   bit 62 set, bits 0..47 = bit offset of the TILE's first byte, bits 48..51 = the row's number inside the tile.
+constexpr int64_t kPlaneFlag = (int64_t)1 << 62;
+constexpr int64_t kOffBitsMask = ((int64_t)1 << 48) - 1;
+__host__ __device__ __forceinline__ bool off_is_plane(int64_t off) { return (off & kPlaneFlag) != 0; }
+__host__ __device__ __forceinline__ int off_plane_row(int64_t off) { return (int)((off >> 48) & 15); }
+// byte offset (from the tile's first byte) of dword d of the 32-id slice `cg` (column group of 32) of row r
+__host__ __device__ __forceinline__ uint64_t plane_dword_at(int r, uint32_t nb, int cg, int d) {
+    const uint64_t sb = (uint64_t)(cg >> 2) * (256u * nb);
+    const uint32_t lane = (uint32_t)r + 16u * (uint32_t)(cg & 3);
+    return d < 4 ? sb + lane * 16u + 4u * (uint32_t)d : sb + 1024u + lane * (4u * (nb - 4u)) + 4u * (uint32_t)(d - 4);
+}
+// One id of a row stored in planes (any column): at most two dwords.
+__device__ __forceinline__ uint32_t plane_field(const uint8_t* __restrict__ ids, uint64_t tile_byte, int r, int nb, int col) {
+    const int cg = col >> 5, bit = (col & 31) * nb, d = bit >> 5, sh = bit & 31;
+    uint32_t v = *reinterpret_cast<const uint32_t*>(ids + tile_byte + plane_dword_at(r, (uint32_t)nb, cg, d)) >> sh;
+    if (sh + nb > 32) v |= *reinterpret_cast<const uint32_t*>(ids + tile_byte + plane_dword_at(r, (uint32_t)nb, cg, d + 1)) << (32 - sh);
+    return v & ((1u << nb) - 1u);
+}
+// One id of a row, however it is stored.  `off` = the row's bit offset word; in bounds by the caller's check.
+__device__ __forceinline__ uint32_t row_field(const uint8_t* __restrict__ ids, int64_t off, int nb, int col, int64_t clamp_byte) {
+    if (off_is_plane(off)) return plane_field(ids, (uint64_t)((off & kOffBitsMask) >> 3), off_plane_row(off), nb, col);
+    return load_field(ids, off + (int64_t)col * nb, nb, clamp_byte);
+}
+// Whether the bytes a row's metadata points at lie inside the buffer (with the 8 pad bytes behind the payload).
+__host__ __device__ __forceinline__ bool row_in_bounds(int64_t off, int nb, int64_t P, int64_t ids_bytes) {
+    if (nb < 1 || nb > 14 || off < 0) return false;
+    if (off_is_plane(off)) {
+        const int64_t t0 = (off & kOffBitsMask) >> 3;
+        return nb >= 4 && nb <= 8 && (P & 127) == 0 && (t0 & 3) == 0 && t0 + 2 * P * nb + 8 <= ids_bytes;     // 16 rows
+    }
+    return off < kOffBitsMask && ((off + (int64_t)nb * P + 7) >> 3) + 8 <= ids_bytes;
+}
+// The lane's NB dwords of slice `cg` of a row stored in planes.
+template <int NB>
+__device__ __forceinline__ void load_slice_planes(const uint8_t* __restrict__ ids, uint64_t tile_byte, int r, int cg, uint32_t (&w)[kMaxFastNb]) {
+    const uint4 a = *reinterpret_cast<const uint4*>(ids + tile_byte + plane_dword_at(r, NB, cg, 0));
+    w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w;
+#pragma unroll
+    for (int k = 4; k < NB; ++k) w[k] = *reinterpret_cast<const uint32_t*>(ids + tile_byte + plane_dword_at(r, NB, cg, k));
 }
 
 // Field J (NB bits) of a lane's NB-dword slice, every shift a compile-time constant.

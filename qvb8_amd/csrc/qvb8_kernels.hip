@@ -111,12 +111,29 @@ __global__ void __launch_bounds__(256) decode_kernel(DecodeArgs a) {
     const float ts = a.tau_s[q], m = a.min_s[q];
     const int col0 = c * kChunk;
     const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
-    const int64_t row_bits = (int64_t)nb * a.P;
-    const bool in_bounds = row_ok && nb >= 1 && nb <= 14 && bit0 >= 0 && ((bit0 + row_bits + 7) >> 3) + 8 <= a.ids_bytes;
+    const bool in_bounds = row_ok && row_in_bounds(bit0, nb, a.P, a.ids_bytes);
     // the lane's 32 values go out as 16-byte stores: the output row must start on 16 bytes as well
-    const bool fast = in_bounds && (a.P % kFieldsPerLane) == 0 && (bit0 & 31) == 0 && nb >= 4 && nb <= kMaxFastNb;
+    const bool planes = off_is_plane(bit0);
+    const bool fast = in_bounds && !planes && (a.P % kFieldsPerLane) == 0 && (bit0 & 31) == 0 && nb >= 4 && nb <= kMaxFastNb;
     const int col_end = min(a.P, col0 + kChunk);
-    if (fast) {
+    if (in_bounds && planes) {
+        // a row stored in planes: the lane's slice comes from two places of its tile
+        const int col = col0 + lane * kFieldsPerLane;
+        if (col < a.P) {
+            const uint64_t tile_byte = (uint64_t)((bit0 & kOffBitsMask) >> 3);
+            const int r = off_plane_row(bit0), cg = col / kFieldsPerLane;
+            uint32_t w[kMaxFastNb];
+            float v[32];
+            switch (nb) {
+                case 4: load_slice_planes<4>(a.ids, tile_byte, r, cg, w); restore_fields<4, FMA, 0, 32>(w, ts, m, v); break;
+                case 5: load_slice_planes<5>(a.ids, tile_byte, r, cg, w); restore_fields<5, FMA, 0, 32>(w, ts, m, v); break;
+                case 6: load_slice_planes<6>(a.ids, tile_byte, r, cg, w); restore_fields<6, FMA, 0, 32>(w, ts, m, v); break;
+                case 7: load_slice_planes<7>(a.ids, tile_byte, r, cg, w); restore_fields<7, FMA, 0, 32>(w, ts, m, v); break;
+                default: load_slice_planes<8>(a.ids, tile_byte, r, cg, w); restore_fields<8, FMA, 0, 32>(w, ts, m, v); break;
+            }
+            OutPack<DT>::store(a.out, orow * a.P + col, v);
+        }
+    } else if (fast) {
         const int col = col0 + lane * kFieldsPerLane;
         if (col < a.P) {
             const int64_t oi = orow * a.P + col;
@@ -306,9 +323,9 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
         const int q = row0 + g + a.G * lane;
         const int nb = a.nbits[q];
         my_bit0 = a.bit_off[q];
-        const int64_t row_bits = (int64_t)nb * a.P;
-        const bool ok = nb >= 1 && nb <= 14 && my_bit0 >= 0 && ((my_bit0 + row_bits + 7) >> 3) + 8 <= a.ids_bytes;
-        const int kind = !ok ? 0 : (FAST && (my_bit0 & 31) == 0 && nb >= 4 && nb <= kMaxFastNb) ? 1 : 2;
+        const bool ok = row_in_bounds(my_bit0, nb, a.P, a.ids_bytes);
+        // a row stored in planes is read element by element here (this kernel serves the shapes the matrix-core path does not)
+        const int kind = !ok ? 0 : (FAST && !off_is_plane(my_bit0) && (my_bit0 & 31) == 0 && nb >= 4 && nb <= kMaxFastNb) ? 1 : 2;
         my_info = (uint32_t)nb | ((uint32_t)kind << 8);
     }
     uint32_t my_b_lo = (uint32_t)my_bit0, my_b_hi = (uint32_t)((uint64_t)my_bit0 >> 32);
@@ -445,7 +462,7 @@ __global__ void __launch_bounds__(512) gemv_kernel(GemvArgs a) {
             } else if (s.kind == 2) {
                 const int col_end = min(a.P, (c + 1) * kChunk);
                 for (int cc = c * kChunk + lane; cc < col_end; cc += kWave) {
-                    const float idf = (float)load_field(a.ids, s.bit0 + (int64_t)cc * s.nb, s.nb, clamp_byte);
+                    const float idf = (float)row_field(a.ids, s.bit0, s.nb, cc, clamp_byte);
 #pragma unroll
                     for (int m = 0; m < MB; ++m) d[m] = __builtin_fmaf(f16_bits_to_f32(xh[(size_t)m * a.P + cc]), idf, d[m]);
                 }
@@ -508,7 +525,7 @@ __global__ void __launch_bounds__(256) gemv_fix_escapes_kernel(const void* __res
     for (int m = 0; m < 8; ++m) acc[m] = 0.f;
     for (int64_t e = i; e < n_esc && esc_idx[e] / P == q; ++e) {
         const int c = (int)(esc_idx[e] - q * P);
-        const float banded = __builtin_fmaf((float)load_field(ids, bit0 + (int64_t)c * nb, nb, clamp_byte), ts, mn);
+        const float banded = __builtin_fmaf((float)row_field(ids, bit0, nb, c, clamp_byte), ts, mn);
         const float delta = esc_vals[e] - banded;
 #pragma unroll
         for (int m = 0; m < 8; ++m)

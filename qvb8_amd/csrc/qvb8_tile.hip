@@ -28,6 +28,8 @@ namespace qvb8 {
 //   loc[pos]  u64   bits 0..47 absolute bit offset of the row's first id | bits 48..55 width | bits 56..57 kind
 //             kind 0: the metadata points outside the buffer (the row yields NaN), 1: dword-aligned row of width
 //             4..8 (sliced path), 2: anything else that is in bounds (read element by element), 3: no such row
+//             bit 58: the row is stored in planes (then bits 0..47 = bit offset of its 16-row tile, bits 59..62 = its
+//             number inside the tile; kind 1)
 //   fin[pos]  4 x u32   tau_s bits, min_s bits, output row q (or 0xffffffff), 0 -- what the end of a tile needs
 // loc has Q rounded up to even entries, so that fin is 16-byte aligned.
 constexpr uint64_t kRowOffMask = (1ull << 48) - 1;
@@ -56,6 +58,7 @@ struct TileArgs {
     // nb[0], [first1, first2) nb[1], [first2, Q) nb[2].  n_classes == 0: addresses come from `loc`.
     int n_classes, first1, first2;
     int nb[3];
+    int planes;                   // rows of whole 16-row tiles of one sliceable width are stored in planes (see qvb8_device.h)
 };
 
 __global__ void __launch_bounds__(256) rowinfo_kernel(const uint8_t* __restrict__ nbits, const int64_t* __restrict__ bit_off,
@@ -71,10 +74,13 @@ __global__ void __launch_bounds__(256) rowinfo_kernel(const uint8_t* __restrict_
         f = uint4{__float_as_uint(tau_s[q]), __float_as_uint(min_s[q]), (uint32_t)q, 0u};
         const int nb = nbits[q];
         const int64_t bit0 = bit_off[q];
-        const int64_t row_bits = (int64_t)nb * P;
-        const bool ok = nb >= 1 && nb <= 14 && bit0 >= 0 && bit0 < (int64_t)kRowOffMask && ((bit0 + row_bits + 7) >> 3) + 8 <= ids_bytes;
-        const uint64_t kind = !ok ? 0 : ((bit0 & 31) == 0 && nb >= 4 && nb <= 8) ? 1 : 2;
-        rec = (ok ? (uint64_t)bit0 : 0) | ((uint64_t)nb << 48) | (kind << 56);
+        const bool ok = row_in_bounds(bit0, nb, P, ids_bytes);
+        if (ok && off_is_plane(bit0)) {
+            rec = (uint64_t)(bit0 & kOffBitsMask) | ((uint64_t)nb << 48) | (1ull << 56) | (1ull << 58) | ((uint64_t)off_plane_row(bit0) << 59);
+        } else {
+            const uint64_t kind = !ok ? 0 : ((bit0 & 31) == 0 && nb >= 4 && nb <= 8) ? 1 : 2;
+            rec = (ok ? (uint64_t)bit0 : 0) | ((uint64_t)nb << 48) | (kind << 56);
+        }
     }
     loc[i] = rec;
     fin[i] = f;
@@ -100,7 +106,7 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
 // slots.  After one barrier the whole workgroup combines the column ranges of each row in a fixed order.
 // The kernel's arguments are 56 bytes of scalars (measured: every further 64 bytes of kernel arguments cost about a
 // microsecond per launch): fin follows loc, n_steps follows P, the small counts share one word.
-template <int NT, int T, bool BF, bool XC, int XP = 0>
+template <int NT, int T, bool BF, bool XC, int XP = 0, bool PL = false>
 __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ ids,
                                                    const uint64_t* __restrict__ loc, float* __restrict__ Y, int64_t ids_bytes,
                                                    int Q, int P, uint32_t counts, int TW, int first1, int first2, uint32_t widths) {
@@ -110,7 +116,7 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
     a.X = X; a.ids = ids; a.loc = loc; a.fin = reinterpret_cast<const uint4*>(loc + rowinfo_loc_words(Q)); a.Y = Y;
     a.ids_bytes = ids_bytes; a.Q = Q; a.P = P; a.n_steps = P / kStepCols; a.TW = TW;
     a.M = (int)(counts & 63u); a.out_dt = (int)((counts >> 6) & 3u); a.W = (int)((counts >> 8) & 15u); a.G = (int)((counts >> 12) & 15u); a.panels = (int)(counts >> 16);
-    a.first1 = first1; a.first2 = first2; a.n_classes = (int)(widths >> 24);
+    a.first1 = first1; a.first2 = first2; a.n_classes = (int)((widths >> 24) & 0x7Fu); a.planes = PL ? 1 : 0;
     a.nb[0] = (int)(widths & 255u); a.nb[1] = (int)((widths >> 8) & 255u); a.nb[2] = (int)((widths >> 16) & 255u);
     using F = Fmt<BF>;
     using XI = XIn<BF, XC>;
@@ -167,6 +173,14 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
                 const uint64_t bit0 = (c == 0 ? 0 : c == 1 ? base1 : base2)
                                       + (uint64_t)(pos - (c == 0 ? 0 : c == 1 ? a.first1 : a.first2)) * P64 * nbc;
                 rec = bit0 | (nbc << 48) | ((uint64_t)((nbc >= 4 && nbc <= 8) ? 1 : 2) << 56);
+                if constexpr (PL) {
+                    // a tile that lies inside one run of a sliceable width is stored in planes: the record then names the tile
+                    const int first_c = c == 0 ? 0 : c == 1 ? a.first1 : a.first2;
+                    const int end_c = c == 0 ? a.first1 : c == 1 ? a.first2 : a.Q;
+                    const int t0 = pos & ~15;
+                    if (nbc >= 4 && nbc <= 8 && t0 >= first_c && t0 + 16 <= end_c)
+                        rec = (bit0 - (uint64_t)(pos & 15) * P64 * nbc) | (nbc << 48) | (1ull << 56) | (1ull << 58) | ((uint64_t)(pos & 15) << 59);
+                }
             } else {
                 rec = a.loc[pos];
             }
@@ -195,9 +209,14 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
     // neighbouring lanes read 4 x 4*nb consecutive bytes of one row (in operand order -- lane = row + 16 * chunk --
     // every lane is a row of its own: measured 61 L1 accesses per request instruction against 25 this way, and about
     // 1.3 % of the decode step).  to_operand then moves a register from request order to operand order across the wave.
-    const int lr = lane >> 2, lk = lane & 3;
+    // PL (the weight has rows stored in planes): every lane asks for its own operand's slice -- for a row in planes the two
+    // requests of a wave are then one contiguous run each (plane A: 1024 bytes, plane B: 256 (nb - 4)), nothing is read
+    // twice, and the loads can be non-temporal; the few rows that are not in planes (tiles across two widths, the last
+    // rows) are asked for row by row in the same lane order.  No move across the wave afterwards.
+    const int lr = PL ? r : lane >> 2, lk = PL ? kg : lane & 3;
     const int pull = 4 * (4 * r + kg);                         // byte address of the lane whose request holds this lane's operand
     auto to_operand = [&](const uint4& v) -> uint4 {
+        if constexpr (PL) return v;
         return uint4{(uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y),
                      (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w)};
     };
@@ -206,15 +225,34 @@ __global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ 
         const uint64_t rec = has_tile ? rec_read : 3ull << 56;  // a wave without tiles: no row, every request reads the buffer's start
         const uint32_t nb = (uint32_t)(rec >> 48) & 0xFFu, kind = (uint32_t)(rec >> 56) & 3u;
         const bool row_sliced = kind == 1u;
-        const uint64_t row_off = ((rec & kRowOffMask) >> 3) + (uint64_t)(step0 * 4 + lk) * (4u * nb);
-        const uint32_t step_bytes = 16u * nb;
-        const uint32_t tail = row_sliced ? 4u * (nb - 4u) : 16u;
+        if constexpr (PL) {
+            const bool in_planes = ((rec >> 58) & 1ull) != 0;
+            const uint32_t slot = (uint32_t)((rec >> 59) & 15ull) + 16u * (uint32_t)lk;      // the lane's place in a plane
+            const uint64_t base = (rec & kRowOffMask) >> 3;
+            // first / last four dwords of the slice: in planes the last four end with the lane's share of plane B
+            const uint64_t lo0 = in_planes ? base + slot * 16u : base + (uint64_t)lk * (4u * nb);
+            const uint64_t hi0 = in_planes ? base + 1024u + (uint64_t)slot * (4u * (nb - 4u)) + 4u * (nb - 4u) - 16u : lo0 + 4u * (nb - 4u);
+            const uint32_t step_bytes = in_planes ? 256u * nb : 16u * nb;
 #pragma unroll
-        for (int it = 0; it < T; ++it) {
-            const bool use = row_sliced && (step0 + it) < a.n_steps;
-            const uint64_t off = use ? row_off + (uint64_t)it * step_bytes : 0;
-            wlo[it] = *reinterpret_cast<const uint4*>(a.ids + off);
-            whi[it] = *reinterpret_cast<const uint4*>(a.ids + off + tail);
+            for (int it = 0; it < T; ++it) {
+                const bool use = row_sliced && (step0 + it) < a.n_steps;
+                const uint64_t at = (uint64_t)(step0 + it) * step_bytes;
+                const v4u_t va = __builtin_nontemporal_load(reinterpret_cast<const v4u_t*>(a.ids + (use ? lo0 + at : 0)));
+                const v4u_t vb = __builtin_nontemporal_load(reinterpret_cast<const v4u_t*>(a.ids + (use ? hi0 + at : 16)));
+                wlo[it] = uint4{va.x, va.y, va.z, va.w};
+                whi[it] = uint4{vb.x, vb.y, vb.z, vb.w};
+            }
+        } else {
+            const uint64_t row_off = ((rec & kRowOffMask) >> 3) + (uint64_t)(step0 * 4 + lk) * (4u * nb);
+            const uint32_t step_bytes = 16u * nb;
+            const uint32_t tail = row_sliced ? 4u * (nb - 4u) : 16u;
+#pragma unroll
+            for (int it = 0; it < T; ++it) {
+                const bool use = row_sliced && (step0 + it) < a.n_steps;
+                const uint64_t off = use ? row_off + (uint64_t)it * step_bytes : 0;
+                wlo[it] = *reinterpret_cast<const uint4*>(a.ids + off);
+                whi[it] = *reinterpret_cast<const uint4*>(a.ids + off + tail);
+            }
         }
         const uint64_t rec2 = my_loc[tk * kTileRows + r];       // what the lane will decode: its operand row's width
         return has_tile && ((uint32_t)(rec2 >> 56) & 3u) == 1u ? (((uint32_t)(rec2 >> 48) & 0xFFu) | (1u << 8)) : 0u;
@@ -446,7 +484,7 @@ __global__ void __launch_bounds__(256) tile_fix_escapes_kernel(const uint16_t* _
     float acc = 0.f;
     for (int64_t e = i; e < n_esc && esc_idx[e] / P == q; ++e) {
         const int c = (int)(esc_idx[e] - q * P);
-        const float banded = __builtin_fmaf((float)load_field(ids, bit0 + (int64_t)c * nb, nb, clamp_byte), ts, mn);
+        const float banded = __builtin_fmaf((float)row_field(ids, bit0, nb, c, clamp_byte), ts, mn);
         acc = __builtin_fmaf(XIn<BF, XC>::scalar(X[(size_t)t * P + c]), esc_vals[e] - banded, acc);
     }
     Y[(size_t)t * Q + q] += acc;
@@ -480,6 +518,7 @@ struct GemmArgs {
     int first1, first2;            // positions where the second and the third width start (Q when there is none)
     int blocks1, blocks2;          // row blocks before the second / the third width (blocks of 256 positions from a width's first)
     uint32_t widths;               // nb0 | nb1 << 8 | nb2 << 16
+    int planes;                    // whole 16-row tiles inside a run are stored in planes (see qvb8_device.h)
 };
 
 // grid (M, splits): sx[z][m] = sum of row m of X over column range z, as the operands see it; XC: X16[m] = the row narrowed
@@ -527,7 +566,7 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
     if (u_begin >= u_end) return;
 
     // ---- this lane's two rows; a position past the run reads the run's last row (finite operands, result not stored) ----
-    const uint8_t* row_ptr[2]; int row_pos[2]; bool row_ok[2];
+    const uint8_t* row_ptr[2]; const uint8_t* row_hi[2]; int row_pos[2]; bool row_ok[2], row_pl[2];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
         const int pos = pos0 + wave * kGemmWaveRows + rt * 32 + n;
@@ -536,7 +575,20 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
         // requests go out in the order lane = 2 * row + half, so that neighbouring lanes read neighbouring bytes
         // (fewer L1 accesses per request); to_operand moves the registers into operand order (lane = row + 32 * half)
         const int rpos = min(pos0 + wave * kGemmWaveRows + rt * 32 + (lane >> 1), pos_end - 1);
-        row_ptr[rt] = a.ids + run_byte0 + (uint64_t)(rpos - run_first) * ((uint64_t)a.P * NB / 8) + (uint32_t)(lane & 1) * (4u * NB);
+        const uint64_t row_bytes = (uint64_t)a.P * NB / 8;
+        // a row of a whole tile inside the run may be stored in planes: first / last four dwords of its slice then come
+        // from the tile's two planes (the slice of 64-column step u, half h is column group 2 u + h of the row)
+        const int t0 = rpos & ~15;
+        row_pl[rt] = a.planes != 0 && t0 >= run_first && t0 + 16 <= pos_end;
+        if (row_pl[rt]) {
+            const uint8_t* tile = a.ids + run_byte0 + (uint64_t)(t0 - run_first) * row_bytes;
+            const uint32_t slot = (uint32_t)(rpos & 15) + 16u * (uint32_t)(lane & 1);
+            row_ptr[rt] = tile + slot * 16u;
+            row_hi[rt] = tile + 1024u + slot * (4u * (NB - 4u)) + 4u * (NB - 4u) - 16u;
+        } else {
+            row_ptr[rt] = a.ids + run_byte0 + (uint64_t)(rpos - run_first) * row_bytes + (uint32_t)(lane & 1) * (4u * NB);
+            row_hi[rt] = row_ptr[rt] + 4u * (NB - 4u);
+        }
     }
     const int pull = 4 * (2 * n + kh);
     auto to_operand = [pull](const uint4& v) -> uint4 {
@@ -546,12 +598,18 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
     uint4 raw[4][2][2];                            // [step % 4][row tile][first / last four dwords]
     const uint8_t* const rp0 = row_ptr[0];
     const uint8_t* const rp1 = row_ptr[1];
-    auto request_ids = [u_end, rp0, rp1](int u, uint4 (&w)[2][2]) {
-        const uint32_t off = (uint32_t)min(u, u_end - 1) * (8u * NB);      // a step is 64 columns = 8 NB bytes of a row
-        w[0][0] = *reinterpret_cast<const uint4*>(rp0 + off);
-        w[0][1] = *reinterpret_cast<const uint4*>(rp0 + off + 4u * (NB - 4u));
-        w[1][0] = *reinterpret_cast<const uint4*>(rp1 + off);
-        w[1][1] = *reinterpret_cast<const uint4*>(rp1 + off + 4u * (NB - 4u));
+    const uint8_t* const rh0 = row_hi[0];
+    const uint8_t* const rh1 = row_hi[1];
+    const bool pl0 = row_pl[0], pl1 = row_pl[1];
+    auto request_ids = [u_end, rp0, rp1, rh0, rh1, pl0, pl1](int u, uint4 (&w)[2][2]) {
+        const uint32_t uc = (uint32_t)min(u, u_end - 1);
+        const uint32_t off = uc * (8u * NB);                               // a step is 64 columns = 8 NB bytes of a row
+        const uint32_t pa = (uc >> 1) * (256u * NB) + (uc & 1u) * 512u;    // in planes: step u / 2, column groups 2 (u % 2) + half
+        const uint32_t pb = (uc >> 1) * (256u * NB) + (uc & 1u) * (128u * (NB - 4u));
+        w[0][0] = *reinterpret_cast<const uint4*>(rp0 + (pl0 ? pa : off));
+        w[0][1] = *reinterpret_cast<const uint4*>(rh0 + (pl0 ? pb : off));
+        w[1][0] = *reinterpret_cast<const uint4*>(rp1 + (pl1 ? pa : off));
+        w[1][1] = *reinterpret_cast<const uint4*>(rh1 + (pl1 ? pb : off));
     };
     // ---- X: thread tid stages piece tid % 16 (8 columns) of rows tid / 16 + 16 * i; rows past M read row M - 1 (not stored at the end) ----
     const int xch = tid & 15, xrow = tid >> 4;
@@ -706,13 +764,24 @@ __device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_e
         // ids: slice g = p % 4 of row p / 4; a position past the run reads the run's last row (never stored)
         const int dg = p & 3, drow = p >> 2;
         const int dpos = min(pos0 + drow, pos_end - 1);
-        const uint8_t* const idp = a.ids + run_byte0 + (uint64_t)(dpos - run_first) * ((uint64_t)a.P * NB / 8)
-                                   + (uint64_t)(s_begin / 2) * (16u * NB) + (uint32_t)dg * (4u * NB);
+        const uint64_t row_bytes = (uint64_t)a.P * NB / 8;
+        // a row of a whole tile inside the run may be stored in planes (a wave's 16 rows x 4 slices are then the tile's two
+        // planes, one contiguous run per request)
+        const int t0 = dpos & ~15;
+        const bool in_planes = a.planes != 0 && t0 >= run_first && t0 + 16 <= pos_end;
+        const uint32_t slot = (uint32_t)(dpos & 15) + 16u * (uint32_t)dg;
+        const uint8_t* const tile = a.ids + run_byte0 + (uint64_t)(t0 - run_first) * row_bytes;
+        const uint32_t blk_bytes = in_planes ? 256u * NB : 16u * NB;
+        const uint8_t* const idp = (in_planes ? tile + slot * 16u
+                                              : a.ids + run_byte0 + (uint64_t)(dpos - run_first) * row_bytes + (uint32_t)dg * (4u * NB))
+                                   + (uint64_t)(s_begin / 2) * blk_bytes;
+        const uint8_t* const idh = in_planes ? tile + 1024u + slot * (4u * (NB - 4u)) + 4u * (NB - 4u) - 16u + (uint64_t)(s_begin / 2) * blk_bytes
+                                             : idp + 4u * (NB - 4u);
         uint4 raw[2][2];
         auto request_ids = [&](int blk, uint4 (&w)[2]) __attribute__((always_inline)) {
-            const uint32_t off = (uint32_t)min(blk, n_blk - 1) * (16u * NB);
+            const uint32_t off = (uint32_t)min(blk, n_blk - 1) * blk_bytes;
             w[0] = *reinterpret_cast<const uint4*>(idp + off);
-            w[1] = *reinterpret_cast<const uint4*>(idp + off + 4u * (NB - 4u));
+            w[1] = *reinterpret_cast<const uint4*>(idh + off);
         };
         auto store_ids = [&](int buf, const uint4 (&w)[2]) __attribute__((always_inline)) {
             v4u_t b[4];
@@ -933,7 +1002,7 @@ bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl) {
     return true;
 }
 
-template <int NT, int T, bool BF, bool XC, int XP = 0>
+template <int NT, int T, bool BF, bool XC, int XP = 0, bool PL = false>
 int launch_tile(TileArgs& a, hipStream_t s) {
     TilePlan pl;
     if (!plan_tile(NT, T, a.M, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
@@ -943,13 +1012,13 @@ int launch_tile(TileArgs& a, hipStream_t s) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: no current device");
     if (!attr[dev]) {
-        if (hipFuncSetAttribute((const void*)tile_kernel<NT, T, BF, XC, XP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)tile_kernel<NT, T, BF, XC, XP, PL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup) != hipSuccess)
             return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: cannot raise the kernel's LDS limit");
         attr[dev] = true;
     }
     if (pl.panels > 0xffff) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: rows too long");
     const uint32_t counts = (uint32_t)a.M | ((uint32_t)a.out_dt << 6) | ((uint32_t)a.W << 8) | ((uint32_t)a.G << 12) | ((uint32_t)a.panels << 16);
-    hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC, XP>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s,
+    hipLaunchKernelGGL((tile_kernel<NT, T, BF, XC, XP, PL>), dim3(pl.blocks), dim3(pl.threads), pl.lds, s,
                        a.X, a.ids, a.loc, a.Y, a.ids_bytes, a.Q, a.P, counts, a.TW, a.first1, a.first2,
                        (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16) | ((uint32_t)a.n_classes << 24));
     return host::check_launch("qvb8_mma");
@@ -957,17 +1026,17 @@ int launch_tile(TileArgs& a, hipStream_t s) {
 // One to sixteen rows of X on the NT = 1 kernel: X goes through LDS when all of it fits (64 KB, and the workgroup's LDS),
 // with 1, 4 or 8 pieces of 16 bytes per thread (a request past the end of X would be a wasted one: the count is exact to
 // within those three variants).
-template <int T, bool BF, bool XC>
+template <int T, bool BF, bool XC, bool PL = false>
 int launch_tile_rows16(TileArgs& a, hipStream_t s) {
     TilePlan pl;
     if (!plan_tile(1, T, a.M, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
     const size_t x_bytes = (size_t)a.M * (size_t)a.P * 2;
     const size_t per_thread = (x_bytes / 16 + pl.threads - 1) / pl.threads;
     const bool fits = x_bytes <= kTileXLdsLimit && pl.lds + x_bytes <= kLdsPerWorkgroup && host::env_int("QVB8_TILE_X_LDS", 1) != 0;
-    if (fits && per_thread <= 1) return launch_tile<1, T, BF, XC, 1>(a, s);
-    if (fits && per_thread <= 4) return launch_tile<1, T, BF, XC, 4>(a, s);
-    if (fits && per_thread <= 8) return launch_tile<1, T, BF, XC, 8>(a, s);
-    return launch_tile<1, T, BF, XC, 0>(a, s);
+    if (fits && per_thread <= 1) return launch_tile<1, T, BF, XC, 1, PL>(a, s);
+    if (fits && per_thread <= 4) return launch_tile<1, T, BF, XC, 4, PL>(a, s);
+    if (fits && per_thread <= 8) return launch_tile<1, T, BF, XC, 8, PL>(a, s);
+    return launch_tile<1, T, BF, XC, 0, PL>(a, s);
 }
 
 struct GemmPlan {
@@ -1139,7 +1208,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     }
     TileArgs a;
     a.X = (const uint16_t*)X; a.ids = ids; a.loc = rowinfo; a.fin = reinterpret_cast<const uint4*>(rowinfo + rowinfo_loc_words(Q));
-    a.n_classes = 0; a.first1 = a.first2 = (int)Q; a.nb[0] = a.nb[1] = a.nb[2] = 0;
+    a.n_classes = 0; a.first1 = a.first2 = (int)Q; a.nb[0] = a.nb[1] = a.nb[2] = 0; a.planes = 0;
     if (layout) {
         if (!rowinfo) return host::fail(QVB8_ERR_ARG, "qvb8_mma: a row layout goes with the row records of the same order");
         const int n = layout->n_classes;
@@ -1158,6 +1227,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         a.n_classes = n;
     }
     const int out_dt = (flags & QVB8_MMA_Y_F16) ? 1 : (flags & QVB8_MMA_Y_BF16) ? 2 : 0;
+    a.planes = (flags & QVB8_MMA_PLANES) ? 1 : 0;
     if (out_dt != 0 && n_esc > 0) return host::fail(QVB8_ERR_ARG, "qvb8_mma: fp16 / bf16 results need a weight without escapes (the correction adds to fp32 results)");
     a.Y = Y; a.out_dt = out_dt; a.ids_bytes = ids_bytes; a.M = (int)M; a.Q = (int)Q; a.P = (int)P; a.n_steps = (int)(P / kStepCols);
     // mode 0: fp16 X, fp16 operands; 1: bf16 X narrowed to saturated fp16 on the way in, fp16 operands; 2: bf16 operands
@@ -1197,6 +1267,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         ga.X = (mode == 1 || staged) ? x16 : a.X; ga.ids = ids; ga.fin = a.fin; ga.sx = sx; ga.out = out;
         ga.M = (int)M; ga.Q = (int)Q; ga.P = (int)P; ga.stages_per_split = g.stages_per_split;
         ga.out_dt = g.splits > 1 ? 0 : out_dt;
+        ga.planes = a.planes;
         ga.first1 = a.first1; ga.first2 = a.first2;
         const int rows0 = a.first1, rows1 = a.first2 - a.first1, rows2 = (int)Q - a.first2;
         const int br = staged ? kG2Rows : kGemmRows;                  // weight rows per workgroup
@@ -1216,16 +1287,20 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
             if (int rc2 = host::check_launch("qvb8_mma reduce")) return rc2;
         }
     } else {
-#define QVB8_TILE_LAUNCH(NT_, T_) (mode == 0 ? launch_tile<NT_, T_, false, false>(a, s) : mode == 1 ? launch_tile<NT_, T_, false, true>(a, s) : launch_tile<NT_, T_, true, false>(a, s))
+#define QVB8_TILE_LAUNCH_P(NT_, T_, PL_) (mode == 0 ? launch_tile<NT_, T_, false, false, 0, PL_>(a, s) : mode == 1 ? launch_tile<NT_, T_, false, true, 0, PL_>(a, s) : launch_tile<NT_, T_, true, false, 0, PL_>(a, s))
+#define QVB8_TILE_LAUNCH(NT_, T_) (a.planes ? QVB8_TILE_LAUNCH_P(NT_, T_, true) : QVB8_TILE_LAUNCH_P(NT_, T_, false))
     // rows of 33..40 steps (P = 5120): one panel of eight waves with five steps each instead of two panels of five waves
     // with four (measured on 27B-class shapes: 16 % faster; more steps per wave did not pay for longer rows)
     const int n_steps_all = (int)(P / kStepCols);
-#define QVB8_TILE_LAUNCH_ROWS16(T_) (mode == 0 ? launch_tile_rows16<T_, false, false>(a, s) : mode == 1 ? launch_tile_rows16<T_, false, true>(a, s) : launch_tile_rows16<T_, true, false>(a, s))
+#define QVB8_TILE_LAUNCH_ROWS16_P(T_, PL_) (mode == 0 ? launch_tile_rows16<T_, false, false, PL_>(a, s) : mode == 1 ? launch_tile_rows16<T_, false, true, PL_>(a, s) : launch_tile_rows16<T_, true, false, PL_>(a, s))
+#define QVB8_TILE_LAUNCH_ROWS16(T_) (a.planes ? QVB8_TILE_LAUNCH_ROWS16_P(T_, true) : QVB8_TILE_LAUNCH_ROWS16_P(T_, false))
         if (M <= 16) rc = n_steps_all > 32 && n_steps_all <= 40 ? QVB8_TILE_LAUNCH_ROWS16(5) : QVB8_TILE_LAUNCH_ROWS16(4);
 #undef QVB8_TILE_LAUNCH_ROWS16
+#undef QVB8_TILE_LAUNCH_ROWS16_P
     else if (M <= 32) rc = QVB8_TILE_LAUNCH(2, 2);
     else rc = QVB8_TILE_LAUNCH(3, 2);
 #undef QVB8_TILE_LAUNCH
+#undef QVB8_TILE_LAUNCH_P
         if (rc) return rc;
     }
     if (n_esc > 0) {

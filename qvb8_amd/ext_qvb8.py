@@ -173,6 +173,7 @@ MMA_MAX_M = 48
 MMA_GEMM_MAX_M = 256          # with a row layout (rows stored in width order, widths 4..8): the workgroup-tiled kernel
 MMA_SATURATE_X = 1
 MMA_Y_F16, MMA_Y_BF16 = 2, 4                      # qvb8_mma_flags: results stored as fp16 / bf16
+MMA_PLANES = 8                                    # qvb8_mma_flags: the pack has rows stored in planes
 
 
 def mma_prepare(row_nbits, row_bit_off, tau_s, min_s, P, ids_bytes, perm=None):
@@ -196,14 +197,38 @@ def mma_prepare(row_nbits, row_bit_off, tau_s, min_s, P, ids_bytes, perm=None):
     return out
 
 
-def sort_rows_by_width(ids, row_nbits, row_bit_off, P, perm):
+PLANE_FLAG = 1 << 62          # bit offset words: the row is stored in planes (bits 0..47 its tile, bits 48..51 its row there)
+
+
+def rows_in_planes(row_bit_off) -> bool:
+    """Whether any row of the pack is stored in planes (one host read)."""
+    return bool(((row_bit_off >> 62) & 1).any()) if row_bit_off.numel() else False
+
+
+def _plane_index(P: int, w: int, device):
+    """For one 16-row tile of width w: (dword index in planes, dword index with the rows back to back) of every dword."""
+    rows = torch.arange(16, device=device).view(16, 1, 1)
+    cg = torch.arange(P // 32, device=device).view(1, -1, 1)
+    d = torch.arange(w, device=device).view(1, 1, -1)
+    native = rows * (P // 32 * w) + cg * w + d
+    lane = rows + 16 * (cg % 4)
+    step_dw = (cg // 4) * (64 * w)
+    planes = torch.where(d < 4, step_dw + lane * 4 + d, step_dw + 256 + lane * (w - 4) + (d - 4))
+    return planes.reshape(-1), native.reshape(-1)
+
+
+def sort_rows_by_width(ids, row_nbits, row_bit_off, P, perm, planes=False):
     """Copies the rows of a pack into `perm` order (rows of one width back to back, from byte 0), once, at load: returns
     (ids_sorted, row_bit_off_sorted, layout) -- the new ids buffer, the new per-row bit offsets (still indexed by row) and
     the _lib.MmaLayout that lets mma_tiles compute row addresses instead of reading them.  None when the pack cannot be
-    laid out that way (P % 128 != 0, rows that do not start on 16-byte boundaries, more than 3 distinct widths)."""
+    laid out that way (P % 128 != 0, rows that do not start on 16-byte boundaries, more than 3 distinct widths).
+    `planes`: every whole 16-row tile (positions 16 t .. 16 t + 15) that lies inside one run of a width 4..8 is stored in
+    planes -- the same bytes, permuted inside the tile so that each request of the matrix-core kernels is one contiguous
+    run -- and its rows' offsets carry PLANE_FLAG (every kernel of the library reads such rows; callers pass
+    mma_tiles(planes=True))."""
     _lib.require_cuda(ids, row_nbits, row_bit_off, perm)
     Q, P = row_nbits.numel(), int(P)
-    if Q == 0 or P % 128 != 0 or bool((row_bit_off % 128 != 0).any()):
+    if Q == 0 or P % 128 != 0 or bool((row_bit_off % 128 != 0).any()) or rows_in_planes(row_bit_off):
         return None
     nb_sorted = row_nbits[perm.long()].to(torch.int64)
     widths, counts = torch.unique_consecutive(nb_sorted, return_counts=True)
@@ -233,13 +258,30 @@ def sort_rows_by_width(ids, row_nbits, row_bit_off, P, perm):
             dst16[d_idx] = src16[s_idx]
         pos += n
     layout.first_pos[len(widths)] = Q
+    if planes:
+        src32 = out[:total_bytes].view(torch.int32)
+        dst = out.clone()
+        dst32 = dst[:total_bytes].view(torch.int32)
+        pos = 0
+        for w, n in zip(widths, counts):
+            t_first, t_end = -(-pos // 16) * 16, (pos + n) // 16 * 16
+            if 4 <= w <= 8 and t_end > t_first:
+                to_planes, to_native = _plane_index(P, w, ids.device)
+                tile_dw0 = new_off_sorted[t_first:t_end:16] // 32          # first dword of each whole tile
+                for k in range(0, tile_dw0.numel(), 256):                  # bounded index tensors
+                    base = tile_dw0[k:k + 256, None]
+                    dst32[(base + to_planes[None, :]).reshape(-1)] = src32[(base + to_native[None, :]).reshape(-1)]
+                inside = torch.arange(t_first, t_end, device=ids.device)
+                new_off_sorted[inside] = (new_off_sorted[inside - inside % 16]) | ((inside % 16) << 48) | PLANE_FLAG
+            pos += n
+        out = dst
     new_off = torch.empty_like(row_bit_off)
     new_off[perm.long()] = new_off_sorted
     return out, new_off, layout
 
 
 def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm=None, saturate=True,
-              rowinfo=None, layout=None, out_dtype=None):
+              rowinfo=None, layout=None, out_dtype=None, planes=False):
     """Matrix-core path for P % 128 == 0: X (fp16 or bf16) times the fp32 band value, fp32 (M, Q).  1 <= M <= 48 always;
     49 <= M <= 256 (the workgroup-tiled decode + GEMM kernel) when `layout` is given and its widths are 4..8.
     `perm` (int32, position -> row) groups rows of equal width into tiles; `rowinfo` = mma_prepare(...) for the
@@ -247,7 +289,8 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
     copied into that order (needs `rowinfo`).  `saturate` (bf16 X only): X is narrowed like saturating_half while it
     is loaded and the product runs on fp16 operands, as every fp16 path of the reference does; without it bf16 X is
     multiplied as it is on bf16 operands.  `out_dtype` torch.float16 / torch.bfloat16: the kernels store the results
-    rounded to that type (the same values as casting the fp32 result; only for a weight without escapes)."""
+    rounded to that type (the same values as casting the fp32 result; only for a weight without escapes).  `planes`:
+    the pack has rows stored in planes (sort_rows_by_width(planes=True))."""
     lib = _lib.load()
     Q = _check_pack(ids, min_s, row_nbits, row_bit_off, tau_s)
     n_esc = _check_escapes(esc_idx, esc_vals)
@@ -293,7 +336,7 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
                                  Q, int(P), _lib.ptr(ei), _lib.ptr(ev), n_esc, _lib.ptr(perm),
                                  None if rowinfo is None else rowinfo.contiguous().data_ptr(),
                                  None if layout is None else ctypes.addressof(layout),
-                                 (MMA_SATURATE_X if saturate else 0) | y_flag, _lib.ptr(Y),
+                                 (MMA_SATURATE_X if saturate else 0) | y_flag | (MMA_PLANES if planes else 0), _lib.ptr(Y),
                                  None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel() * 8,
                                  _lib.stream_of(Xc)), lib)
     return Y

@@ -42,6 +42,27 @@ def test_decode_bit_exact_hand_made_packs(Q, P, widths):
     _check_decode(d, H.to_device_args(d, DEV))
 
 
+def test_fp16_restore_rounds_the_fp32_value_not_the_exact_sum():
+    """fp16 weights are fp16(fp32(fma(id, tau_s, min_s))): two roundings.  A pack big enough to hold values whose fp32
+    rounding lands on an fp16 tie (where rounding the exact sum once gives the other neighbour) restores bit for bit;
+    the results stored as fp16 by the matrix-core kernel follow the same rule."""
+    Q, P = 256, 4096
+    d = H.mixed_width_pack(Q, P, [8, 6], seed=77)
+    d["tau_s"] = d["tau_s"] * (1.0 / 64)
+    ids = d["ids_dense"]
+    w32 = O.restore(d["min_s"], d["tau_s"], ids, d["esc_idx"], d["esc_vals"], "fp32")
+    exact = d["min_s"].astype(np.float64)[:, None] + ids.astype(np.float64) * d["tau_s"].astype(np.float64)[:, None]
+    want = w32.astype(np.float16).view(np.uint16)
+    assert (want != exact.astype(np.float16).view(np.uint16)).sum() >= 8          # the case is in the pack
+    args = H.to_device_args(d, DEV)
+    assert np.array_equal(_bits(ext.decode(*args)), want)
+    rows = torch.arange(Q, device=DEV)
+    e0, v0 = torch.zeros(0, dtype=torch.int64, device=DEV), torch.zeros(0, device=DEV)
+    got = ext.lookup_rows(rows, *args[:6], e0, v0, out_dtype=torch.float16)
+    prod = (ids.astype(np.float32) * d["tau_s"][:, None]).astype(np.float32)
+    assert np.array_equal(_bits(got), (d["min_s"][:, None] + prod).astype(np.float32).astype(np.float16).view(np.uint16))
+
+
 def test_decode_golden_blob(golden):
     g = golden("ref_qvb8_blob.npz")
     d = O.parse_qvb8_blob(g["blob11"].tobytes())

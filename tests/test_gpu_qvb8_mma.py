@@ -240,3 +240,48 @@ def test_gemm_real_shapes_with_escapes(Q, P, M):
     tol = H.gemv_tolerance(ref, Wr, xs) + 2.0 ** -8 * np.abs(ref)
     diff = np.abs(y.float().cpu().numpy().astype(np.float64) - ref)
     assert np.all(diff <= tol), (float(diff.max()), float((diff / tol).max()))
+
+
+def _sorted_planes(d):
+    """As _sorted_pack, with every whole tile of one width stored in planes."""
+    a = H.to_device_args(d, DEV)
+    ids, min_s, nbits, bit_off, P, tau_s, ei, ev = a
+    perm = _perm_by_width(nbits)
+    srt = ext.sort_rows_by_width(ids, nbits, bit_off, P, perm, planes=True)
+    assert srt is not None
+    ids, bit_off, layout = srt
+    assert ext.rows_in_planes(bit_off)
+    rowinfo = ext.mma_prepare(nbits, bit_off, tau_s, min_s, P, ids.numel(), perm)
+    return (ids, min_s, nbits, bit_off, P, tau_s, ei, ev), perm, rowinfo, layout
+
+
+@pytest.mark.parametrize("Q,P,widths", [(300, 768, [7, 6, 5]), (136, 2048, [8, 4]), (64, 4096, [7]), (333, 256, [6, 9, 5])])
+def test_rows_stored_in_planes_change_no_result(Q, P, widths):
+    """The same pack with its rows back to back and with whole tiles stored in planes: the dense restore and the
+    matrix-core products of every kernel behind qvb8_mma (with and without a row layout, with escapes) agree bit for bit; the GEMV kernel reads them too."""
+    d = H.mixed_width_pack(Q, P, widths, seed=Q + P)
+    d["tau_s"] = d["tau_s"] * (1.0 / 64)
+    rng = np.random.default_rng(5)
+    flat = np.sort(rng.choice(Q * P, 40, replace=False)).astype(np.int64)
+    d["esc_idx"], d["esc_vals"] = flat, rng.normal(size=40).astype(np.float32)
+    args_n, perm, rowinfo_n, layout_n = _sorted_pack(d)
+    args_p, perm_p, rowinfo_p, layout_p = _sorted_planes(d)
+    assert torch.equal(perm, perm_p)
+    ids_n, min_s, nbits, off_n, _, tau_s, ei, ev = args_n
+    ids_p, off_p = args_p[0], args_p[3]
+    assert ids_n.numel() == ids_p.numel() and not torch.equal(ids_n, ids_p)
+    for fn in (ext.decode_f32, ext.decode, ext.decode_bf16):
+        assert torch.equal(fn(ids_n, min_s, nbits, off_n, P, tau_s, ei, ev), fn(ids_p, min_s, nbits, off_p, P, tau_s, ei, ev))
+    x8 = _x(8, P, torch.float16, 1)
+    _check(d, None, x8, ext.gemv_multi(x8, *args_p), saturate_ref=False)      # rows in planes are read element by element there
+    sliceable = all(4 <= w <= 8 for w in widths) and P % 256 == 0
+    for M in (1, 5, 16, 20, 40) + ((64, 100, 256) if sliceable else ()):
+        x = _x(M, P, torch.bfloat16, M)
+        want = ext.mma_tiles(x, *args_n, perm=perm, rowinfo=rowinfo_n, layout=layout_n)
+        got = ext.mma_tiles(x, *args_p, perm=perm, rowinfo=rowinfo_p, layout=layout_p, planes=True)
+        assert torch.equal(want, got), M
+        if M <= 40:                                            # without the layout: the row records carry the planes
+            assert torch.equal(ext.mma_tiles(x, *args_n, perm=perm, rowinfo=rowinfo_n),
+                               ext.mma_tiles(x, *args_p, perm=perm, rowinfo=rowinfo_p, planes=True)), M
+    _check(d, None, _x(3, P, torch.bfloat16, 3), ext.mma_tiles(_x(3, P, torch.bfloat16, 3), *args_p, perm=perm, rowinfo=rowinfo_p,
+                                                              layout=layout_p, planes=True), saturate_ref=True)
