@@ -55,6 +55,11 @@ WALK_CEILING_TSYM = 1.814
 MMA_FLAGS = int(os.environ.get("QVB8_BENCH_MMA_FLAGS", "1"))     # 1 = QVB8_MMA_SATURATE_X: the operator's default for bf16 x
 
 
+def mma_flags(lin) -> int:
+    """The flags the operator passes for this weight: 8 = QVB8_MMA_PLANES when its rows were stored in planes at load."""
+    return MMA_FLAGS | (8 if lin._planes else 0)
+
+
 def tile_traffic(units, n_launch):
     """Mean measured HBM bytes per launch of the step's launch mix (None when the counters' summary is not there)."""
     t = measured_traffic("tile_kernel_9b_decode_step_hbm_traffic.md", "tile_kernel")
@@ -417,7 +422,7 @@ def bench_lmhead(args, dev):
                           lin.min_s.data_ptr(), lin.tau_s.data_ptr(), lin.nbits.data_ptr(), lin.bit_off.data_ptr(), Q, P,
                           lin.esc_idx.data_ptr() if n_esc else None, lin.esc_vals.data_ptr() if n_esc else None, n_esc,
                           perm.data_ptr(), rowinfo.data_ptr(), ctypes.addressof(layout) if layout is not None else None,
-                          MMA_FLAGS, Y.data_ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
+                          mma_flags(lin), Y.data_ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
         if rc != 0:
             raise RuntimeError(lib.qvb8_last_error().decode())
     ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
@@ -548,7 +553,7 @@ def bench_floor(args, dev):
                 rc = lib.qvb8_mma(x.data_ptr(), _lib.dtype_code(x.dtype), 1, lin.ids.data_ptr(), lin.ids.numel(), lin.min_s.data_ptr(),
                                   lin.tau_s.data_ptr(), lin.nbits.data_ptr(), lin.bit_off.data_ptr(), Q, P,
                                   lin.esc_idx.data_ptr() if ne else None, lin.esc_vals.data_ptr() if ne else None, ne, perm.data_ptr(),
-                                  rowinfo.data_ptr(), ctypes.addressof(layout) if layout is not None else None, MMA_FLAGS,
+                                  rowinfo.data_ptr(), ctypes.addressof(layout) if layout is not None else None, mma_flags(lin),
                                   Y.data_ptr(), None, 0, s)
                 if rc != 0:
                     raise RuntimeError(lib.qvb8_last_error().decode())
@@ -720,7 +725,7 @@ def main():
                               lin.esc_vals.data_ptr() if u["n_esc"] else None, u["n_esc"],
                               u["perm"].data_ptr(), u["rowinfo"].data_ptr(),
                               ctypes.addressof(u["layout"]) if u["layout"] is not None else None,
-                              MMA_FLAGS, u["Y"].data_ptr(), None, 0, s)
+                              mma_flags(lin), u["Y"].data_ptr(), None, 0, s)
             if rc != 0:
                 raise RuntimeError(lib.qvb8_last_error().decode())
 

@@ -217,6 +217,84 @@ def _plane_index(P: int, w: int, device):
     return planes.reshape(-1), native.reshape(-1)
 
 
+def rows_back_to_back(ids, row_nbits, row_bit_off, P):
+    """Undoes the planes: (ids, row_bit_off) with every row of the pack stored back to back again (the bytes of each
+    tile permuted back in place, plain bit offsets).  The arguments themselves when no row is stored in planes."""
+    if not rows_in_planes(row_bit_off):
+        return ids, row_bit_off
+    P = int(P)
+    flagged = (row_bit_off >> 62) & 1 == 1
+    tile_bit = row_bit_off & ((1 << 48) - 1)
+    r_in_tile = (row_bit_off >> 48) & 15
+    nb = row_nbits.to(torch.int64)
+    new_off = torch.where(flagged, tile_bit + r_in_tile * P * nb, row_bit_off)
+    out = ids.clone()
+    src32, dst32 = ids[: ids.numel() // 4 * 4].view(torch.int32), out[: ids.numel() // 4 * 4].view(torch.int32)
+    for w in torch.unique(nb[flagged]).tolist():
+        to_planes, to_native = _plane_index(P, int(w), ids.device)
+        tile_dw0 = torch.unique(tile_bit[flagged & (nb == w)]) // 32       # a subset of the rows may not hold a tile's first
+        for k in range(0, tile_dw0.numel(), 256):                          # bounded index tensors
+            base = tile_dw0[k:k + 256, None]
+            dst32[(base + to_native[None, :]).reshape(-1)] = src32[(base + to_planes[None, :]).reshape(-1)]
+    return out, new_off
+
+
+def widen_rows_to_whole_tiles(ids, row_nbits, row_bit_off, P, tile_rows=16, top=8):
+    """Stores a few rows with more bits than they need so that, sorted by width, every run of one width is a whole number
+    of 16-row tiles: of each width (ascending) the last `count % 16` rows move up to the next width present (up to
+    `top`).  A row's ids, tau_s and min_s stay what they are -- only the field its ids are stored in gets wider, so
+    every value of the weight is unchanged -- and at most 15 rows per width grow by a bit or two each.  Returns
+    (ids, row_nbits, row_bit_off) with the widened rows appended to a copy of `ids`, or None when nothing moves."""
+    P = int(P)
+    ids, row_bit_off = rows_back_to_back(ids, row_nbits, row_bit_off, P)
+    nb = row_nbits.to(torch.int64)
+    widths, counts = torch.unique(nb, return_counts=True)
+    widths, counts = widths.tolist(), counts.tolist()                      # one host read, at load
+    moves = []                                                             # (rows, from width, to width)
+    carried = None                                                         # rows moved up into the class at hand
+    for k, (w, n) in enumerate(zip(widths, counts)):
+        rows = torch.nonzero(nb == w).reshape(-1)
+        members = [(rows, w)] if carried is None else [(rows, w)] + carried
+        total = n + (0 if carried is None else sum(int(r.numel()) for r, _ in carried))
+        carried = None
+        spill = total % tile_rows
+        if k + 1 == len(widths) or widths[k + 1] > top or spill == 0:
+            continue
+        up, out = widths[k + 1], []
+        for r, w0 in reversed(members):                                    # rows that came from below move on first
+            take = min(spill, int(r.numel()))
+            if take:
+                out.append((r[int(r.numel()) - take:], w0))
+                spill -= take
+        carried = out
+        for r, w0 in out:
+            moves.append((r, w0, up))
+    # a row moved twice is listed twice: its last move counts
+    final = {}
+    for r, w0, up in moves:
+        for q in r.tolist():
+            final[q] = (final[q][0] if q in final else w0, up)
+    if not final:
+        return None
+    new_nb, new_off = row_nbits.clone(), row_bit_off.clone()
+    base = (ids.numel() - 8 + 15) // 16 * 16                               # the pad bytes of the old end are reused
+    parts, at = [], base
+    cols = torch.arange(P, device=ids.device, dtype=torch.int64)
+    for q, (w0, up) in sorted(final.items()):
+        pos = row_bit_off[q] + cols * w0
+        byte, sh = pos >> 3, pos & 7
+        word = ids[byte].to(torch.int64) | (ids[byte + 1].to(torch.int64) << 8) | (ids[byte + 2].to(torch.int64) << 16)
+        val = (word >> sh) & ((1 << w0) - 1)
+        bits = ((val[:, None] >> torch.arange(up, device=ids.device)) & 1).reshape(-1, 8)
+        parts.append((bits << torch.arange(8, device=ids.device)).sum(1).to(torch.uint8))
+        new_nb[q], new_off[q] = up, at * 8
+        at += P * up // 8
+    out_ids = torch.zeros(at + 8, dtype=torch.uint8, device=ids.device)
+    out_ids[: ids.numel() - 8] = ids[: ids.numel() - 8]
+    out_ids[base:at] = torch.cat(parts)
+    return out_ids, new_nb, new_off
+
+
 def sort_rows_by_width(ids, row_nbits, row_bit_off, P, perm, planes=False):
     """Copies the rows of a pack into `perm` order (rows of one width back to back, from byte 0), once, at load: returns
     (ids_sorted, row_bit_off_sorted, layout) -- the new ids buffer, the new per-row bit offsets (still indexed by row) and
@@ -225,10 +303,13 @@ def sort_rows_by_width(ids, row_nbits, row_bit_off, P, perm, planes=False):
     `planes`: every whole 16-row tile (positions 16 t .. 16 t + 15) that lies inside one run of a width 4..8 is stored in
     planes -- the same bytes, permuted inside the tile so that each request of the matrix-core kernels is one contiguous
     run -- and its rows' offsets carry PLANE_FLAG (every kernel of the library reads such rows; callers pass
-    mma_tiles(planes=True))."""
+    mma_tiles(planes=True)).  A pack that already has rows in planes is read as if they were back to back."""
     _lib.require_cuda(ids, row_nbits, row_bit_off, perm)
     Q, P = row_nbits.numel(), int(P)
-    if Q == 0 or P % 128 != 0 or bool((row_bit_off % 128 != 0).any()) or rows_in_planes(row_bit_off):
+    if Q == 0 or P % 128 != 0:
+        return None
+    ids, row_bit_off = rows_back_to_back(ids, row_nbits, row_bit_off, P)
+    if bool((row_bit_off % 128 != 0).any()):
         return None
     nb_sorted = row_nbits[perm.long()].to(torch.int64)
     widths, counts = torch.unique_consecutive(nb_sorted, return_counts=True)

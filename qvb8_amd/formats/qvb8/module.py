@@ -21,6 +21,8 @@ Dispatch on the row count M of the flattened input (the reference's: module.py:3
 """
 from __future__ import annotations
 
+import os
+
 import numpy as np
 import torch
 import torch.nn as nn
@@ -58,9 +60,14 @@ class QVBandLinearV8(nn.Module):
     # `bit_off` are replaced, every kernel keeps working through bit_off), so that calls compute row addresses instead of
     # reading them.  Set False to keep the file's row order in memory.
     sort_rows = True
+    # With the sort, every whole 16-row tile of one width 4..8 is stored in planes: the same bytes, permuted inside the tile
+    # so that each request of a wave of the matrix-core kernels is one contiguous run (measured on the 9B decode step:
+    # 7 % faster than rows back to back).  QVB8_PLANES=0 in the environment or False here keeps the rows back to back.
+    plane_tiles = True
     bf16_gemm = False             # opt-in: M > 96 bf16 callers decode to bf16 and run one bf16 GEMM (module.py:60-65)
     bf16_certified = False        # the pack certifies |orig - bf16(band)| <= tau (container restore code 3)
     fp16_table_missing = False    # fp16+bf16 pack loaded without escape_tables.json: fp16 forwards refuse
+    _planes = False               # some rows are stored in planes (set with the launch data)
 
     def __init__(self, *, min_s, nbits, bit_off, ids, Q, P, tau_s, esc_idx, esc_vals, bias=None,
                  esc_idx_bf16=None, esc_vals_bf16=None):
@@ -219,12 +226,23 @@ class QVBandLinearV8(nn.Module):
             nb = self.nbits.to(torch.int16)
             if 1 <= int(nb.min()) and int(nb.max()) <= 14:
                 perm = torch.argsort(nb, stable=True).to(torch.int32).contiguous()
-                layout = None
+                layout = self.__dict__.get("_sorted_layout")                  # sorted before (the buffers have moved since)
                 row_bytes = int((self.nbits.to(torch.int64) * self.in_features).sum().item()) // 8
-                if self.sort_rows and 2 * row_bytes >= self.ids.numel():      # not for a small view into a shared stack
-                    srt = ext.sort_rows_by_width(self.ids, self.nbits, self.bit_off, self.in_features, perm)
+                if layout is None and self.sort_rows and 2 * row_bytes >= self.ids.numel():   # not for a small view into a shared stack
+                    planes = self.plane_tiles and os.environ.get("QVB8_PLANES", "1") != "0"
+                    ids, nbits, bit_off, order = self.ids, self.nbits, self.bit_off, perm
+                    # whole tiles only: a tile across two widths is read row by row, and a launch waits for its slowest
+                    # workgroup -- so up to 15 rows per width are stored one width up (their values do not change)
+                    wide = ext.widen_rows_to_whole_tiles(ids, nbits, bit_off, self.in_features) if planes else None
+                    if wide is not None:
+                        ids, nbits, bit_off = wide
+                        order = torch.argsort(nbits.to(torch.int16), stable=True).to(torch.int32).contiguous()
+                    srt = ext.sort_rows_by_width(ids, nbits, bit_off, self.in_features, order, planes=planes)
                     if srt is not None:
                         self.ids, self.bit_off, layout = srt
+                        self.nbits, perm = nbits, order
+                        self._sorted_layout = layout
+                self._planes = ext.rows_in_planes(self.bit_off)               # also a subset of, or a copy of, such a weight
                 rowinfo = ext.mma_prepare(self.nbits, self.bit_off, self.tau_s, self.min_s, self.in_features,
                                           self.ids.numel(), perm)
                 order = (perm, rowinfo, layout)
@@ -291,7 +309,8 @@ class QVBandLinearV8(nn.Module):
             # without escapes and bias the kernels round the results to the caller's type themselves: no cast pass over Y
             direct = out_dtype if (ei.numel() == 0 and self.bias is None and out_dtype in (torch.float16, torch.bfloat16)) else None
             y = ext.mma_tiles(xm, self.ids, self.min_s, self.nbits, self.bit_off, self.in_features, self.tau_s,
-                              ei, ev, perm=perm, saturate=not bf16_mode, rowinfo=rowinfo, layout=layout, out_dtype=direct)
+                              ei, ev, perm=perm, saturate=not bf16_mode, rowinfo=rowinfo, layout=layout, out_dtype=direct,
+                              planes=self._planes)
             return self._finish(y, orig, out_dtype)
         if M <= 8:
             y = ext.gemv_multi(xk, self.ids, self.min_s, self.nbits, self.bit_off, self.in_features, self.tau_s,

@@ -181,3 +181,42 @@ def test_rows_copied_into_width_order(widths, sortable):
         assert bool((lin.nbits[perm.long()][1:] >= lin.nbits[perm.long()][:-1]).all())
     after = ext.decode_f32(lin.ids, lin.min_s, lin.nbits, lin.bit_off, 256, lin.tau_s, lin.esc_idx, lin.esc_vals)
     assert torch.equal(before, after)
+
+
+def test_plane_tiles_change_no_result_and_survive_moves_subsets_and_fusion(monkeypatch):
+    """The operator stores whole tiles in planes when it sorts the rows; results are those of rows kept back to back, bit
+    for bit, at every M; a move of the module keeps the row layout; a row subset and a fusion of such modules still read
+    the rows; QVB8_PLANES=0 switches the planes off."""
+    from qvb8_amd.formats.qvb8.fuse import concat_linears
+    enc = PK.encode_tensor(H.synth_weight(520, 1024, seed=11).to(DEV), 1e-3, restore="fp16",
+                           force_escapes=[3, 1024 * 100 + 17, 1024 * 519 + 1000])
+    flat, tiled = QVBandLinearV8.from_encoded(enc), QVBandLinearV8.from_encoded(enc)
+    flat.plane_tiles = False
+    xs = {M: torch.randn(M, 1024, generator=torch.Generator().manual_seed(M)).to(torch.bfloat16).to(DEV) for M in (1, 7, 40, 64, 200)}
+    want = {M: flat(x) for M, x in xs.items()}
+    for M, x in xs.items():
+        assert torch.equal(want[M], tiled(x)), M
+    assert tiled._planes and not flat._planes
+    ref, Wr, x64 = _ref(enc, xs[7], saturate=True)
+    _close(want[7], ref, Wr, x64, torch.bfloat16)
+    tiled = tiled.to(torch.bfloat16)                          # any _apply drops the launch data; the sorted buffers stay
+    assert tiled._mma_order()[2] is not None and tiled._planes
+    for M, x in xs.items():
+        assert torch.equal(want[M], tiled(x)), M
+    rows = torch.arange(519, -1, -3, device=DEV)
+    for M in (1, 40):
+        assert torch.equal(flat.row_subset(rows)(xs[M]), tiled.row_subset(rows)(xs[M])), M
+    enc2 = PK.encode_tensor(H.synth_weight(136, 1024, seed=12).to(DEV), 1e-3, restore="fp16")
+    other = QVBandLinearV8.from_encoded(enc2).prepare()
+    fused = concat_linears([tiled, other])[0]                 # members already stored in planes: sorted again as one weight
+    assert fused._mma_order()[2] is not None and fused._planes
+    for M in (1, 20):                                         # the tile kernel on both sides
+        x = xs[200][:M].contiguous()
+        assert torch.equal(fused(x), torch.cat([tiled(x), other(x)], dim=1)), M
+    y = fused(xs[200][:100])
+    for e, part in ((enc, y[:, :520]), (enc2, y[:, 520:])):
+        ref, Wr, x64 = _ref(e, xs[200][:100], saturate=True)
+        _close(part, ref, Wr, x64, torch.bfloat16)
+    monkeypatch.setenv("QVB8_PLANES", "0")
+    off = QVBandLinearV8.from_encoded(enc)
+    assert torch.equal(want[40], off(xs[40])) and not off._planes

@@ -270,6 +270,8 @@ def test_rows_stored_in_planes_change_no_result(Q, P, widths):
     ids_n, min_s, nbits, off_n, _, tau_s, ei, ev = args_n
     ids_p, off_p = args_p[0], args_p[3]
     assert ids_n.numel() == ids_p.numel() and not torch.equal(ids_n, ids_p)
+    back_ids, back_off = ext.rows_back_to_back(ids_p, nbits, off_p, P)           # the planes undone: the same bytes again
+    assert torch.equal(back_ids, ids_n) and torch.equal(back_off, off_n)
     for fn in (ext.decode_f32, ext.decode, ext.decode_bf16):
         assert torch.equal(fn(ids_n, min_s, nbits, off_n, P, tau_s, ei, ev), fn(ids_p, min_s, nbits, off_p, P, tau_s, ei, ev))
     x8 = _x(8, P, torch.float16, 1)
@@ -285,3 +287,22 @@ def test_rows_stored_in_planes_change_no_result(Q, P, widths):
                                ext.mma_tiles(x, *args_p, perm=perm, rowinfo=rowinfo_p, planes=True)), M
     _check(d, None, _x(3, P, torch.bfloat16, 3), ext.mma_tiles(_x(3, P, torch.bfloat16, 3), *args_p, perm=perm, rowinfo=rowinfo_p,
                                                               layout=layout_p, planes=True), saturate_ref=True)
+
+
+@pytest.mark.parametrize("Q,P,widths", [(300, 768, [7, 6, 5]), (136, 256, [8, 4]), (333, 256, [6, 9, 5]), (40, 128, [5, 6, 7, 8]), (64, 128, [7])])
+def test_rows_widened_to_whole_tiles_keep_every_value(Q, P, widths):
+    """A few rows stored one width up so that every run of a width is a whole number of tiles: the dense restore is bit
+    for bit what it was, no row got narrower, and every run below the last sliceable width is a multiple of 16 rows."""
+    d = H.mixed_width_pack(Q, P, widths, seed=Q)
+    ids, min_s, nbits, bit_off, _, tau_s, ei, ev = H.to_device_args(d, DEV)
+    wide = ext.widen_rows_to_whole_tiles(ids, nbits, bit_off, P)
+    counts = {w: widths_n for w, widths_n in zip(*[t.tolist() for t in torch.unique(nbits, return_counts=True)])}
+    if all(n % 16 == 0 for w, n in sorted(counts.items())[:-1]):
+        assert wide is None
+        return
+    ids2, nbits2, off2 = wide
+    assert bool((nbits2 >= nbits).all()) and int((nbits2 != nbits).sum()) <= 15 * len(counts)
+    assert torch.equal(ext.decode_f32(ids, min_s, nbits, bit_off, P, tau_s, ei, ev), ext.decode_f32(ids2, min_s, nbits2, off2, P, tau_s, ei, ev))
+    runs = sorted(zip(*[t.tolist() for t in torch.unique(nbits2, return_counts=True)]))
+    for (w, n), (w_next, _) in zip(runs[:-1], runs[1:]):
+        assert n % 16 == 0 or w_next > 8, runs
