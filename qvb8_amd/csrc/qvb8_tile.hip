@@ -573,8 +573,10 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
         row_ok[rt] = pos < pos_end;
         row_pos[rt] = row_ok[rt] ? pos : pos_end - 1;
         // requests go out in the order lane = 2 * row + half, so that neighbouring lanes read neighbouring bytes
-        // (fewer L1 accesses per request); to_operand moves the registers into operand order (lane = row + 32 * half)
+        // (fewer L1 accesses per request); to_operand moves the registers into operand order (lane = row + 32 * half).
+        // (With rows stored in planes, requests in operand order -- contiguous, no move afterwards -- were measured: no gain.)
         const int rpos = min(pos0 + wave * kGemmWaveRows + rt * 32 + (lane >> 1), pos_end - 1);
+        const uint32_t rhalf = (uint32_t)(lane & 1);
         const uint64_t row_bytes = (uint64_t)a.P * NB / 8;
         // a row of a whole tile inside the run may be stored in planes: first / last four dwords of its slice then come
         // from the tile's two planes (the slice of 64-column step u, half h is column group 2 u + h of the row)
@@ -582,11 +584,11 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
         row_pl[rt] = a.planes != 0 && t0 >= run_first && t0 + 16 <= pos_end;
         if (row_pl[rt]) {
             const uint8_t* tile = a.ids + run_byte0 + (uint64_t)(t0 - run_first) * row_bytes;
-            const uint32_t slot = (uint32_t)(rpos & 15) + 16u * (uint32_t)(lane & 1);
+            const uint32_t slot = (uint32_t)(rpos & 15) + 16u * rhalf;
             row_ptr[rt] = tile + slot * 16u;
             row_hi[rt] = tile + 1024u + slot * (4u * (NB - 4u)) + 4u * (NB - 4u) - 16u;
         } else {
-            row_ptr[rt] = a.ids + run_byte0 + (uint64_t)(rpos - run_first) * row_bytes + (uint32_t)(lane & 1) * (4u * NB);
+            row_ptr[rt] = a.ids + run_byte0 + (uint64_t)(rpos - run_first) * row_bytes + rhalf * (4u * NB);
             row_hi[rt] = row_ptr[rt] + 4u * (NB - 4u);
         }
     }
@@ -761,8 +763,11 @@ __device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_e
         // register sets of X pieces (stage s in set s % 4, requested four stages before it is stored), two of id slices
         // (block b in set b % 2, requested two blocks before it is decoded).  Four stages per turn of the loop.
         const int p = tid - 64 * kG2Mul;
-        // ids: slice g = p % 4 of row p / 4; a position past the run reads the run's last row (never stored)
-        const int dg = p & 3, drow = p >> 2;
+        // ids: slice g = p % 4 of row p / 4 (neighbouring lanes read neighbouring bytes of a row); with rows stored in planes
+        // lane l of a wave takes entry l of its tile's planes -- row l % 16, slice l / 16 -- and a wave's request is one
+        // contiguous run.  A position past the run reads the run's last row (never stored).
+        const bool by_entry = a.planes != 0;
+        const int dg = by_entry ? (p >> 4) & 3 : p & 3, drow = by_entry ? (p & 15) + 16 * (p >> 6) : p >> 2;
         const int dpos = min(pos0 + drow, pos_end - 1);
         const uint64_t row_bytes = (uint64_t)a.P * NB / 8;
         // a row of a whole tile inside the run may be stored in planes (a wave's 16 rows x 4 slices are then the tile's two
