@@ -763,7 +763,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": tile_traffic(units, n_launch) if (MMA_FLAGS == 1 and args.model == "9b" and not args.no_fuse) else None,
-                     "kernel": "qvb8::tile_kernel<1,4,false,true,XP> (XP = 1 or 4 pieces of X per thread through LDS)" + (" / <1,5,false,true,XP> for 5120-column rows" if args.model == "27b" else ""),
+                     "kernel": "qvb8::tile_kernel<1,4,false,true,XP,PL> (XP = 1 or 4 pieces of X per thread through LDS; PL: rows stored in planes)" + (" / <1,5,false,true,XP,PL> for 5120-column rows" if args.model == "27b" else ""),
                      "bytes_per_launch": step_bytes // n_launch,
                      "launch_us": round(launch_us, 3)},
     }
