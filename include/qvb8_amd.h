@@ -51,9 +51,10 @@ enum qvb8_status {
 };
 
 /* Library identification: ABI version, bumped on any signature change or new entry point (3: row lookup, attention over
- * the banded KV cache, query preparation; 4: qvb8_moe_experts_static).  A binding compares the loaded library's answer
+ * the banded KV cache, query preparation; 4: qvb8_moe_experts_static; 5: result-type flags of qvb8_mma; 6: rows stored
+ * in planes, QVB8_MMA_PLANES).  A binding compares the loaded library's answer
  * with the QVB8_ABI_VERSION it was written for before it makes any other call. */
-#define QVB8_ABI_VERSION 5
+#define QVB8_ABI_VERSION 6
 int qvb8_abi_version(void);
 /* Message of the calling thread's most recent failure ("" if none). Valid until that thread's next call. */
 const char* qvb8_last_error(void);

@@ -12,7 +12,7 @@ import torch
 from .common.errors import NativeLibraryError
 
 _LIB = None
-EXPECTED_ABI = 5            # QVB8_ABI_VERSION of include/qvb8_amd.h that the argument lists below were written for
+EXPECTED_ABI = 6            # QVB8_ABI_VERSION of include/qvb8_amd.h that the argument lists below were written for
 F32, F16, BF16 = 0, 1, 2
 _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 

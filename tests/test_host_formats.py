@@ -180,3 +180,49 @@ def test_format_registry():
         F.require(spec, "cpu_linear")
     with pytest.raises(ValueError):
         F.get_format("fp8n")
+
+
+def test_plane_index_is_the_layout_the_header_describes():
+    """ext_qvb8._plane_index against the layout written out with loops: step s of a tile = plane A (entry l = r + 16 (g % 4):
+    dwords 0..3 of slice g of row r) then plane B (dwords 4..w-1), 256 w bytes per step."""
+    import torch
+    from qvb8_amd import ext_qvb8 as ext
+    for P, w in ((128, 4), (256, 7), (384, 8), (128, 5)):
+        to_planes, to_native = ext._plane_index(P, w, torch.device("cpu"))
+        assert sorted(to_planes.tolist()) == sorted(to_native.tolist()) == list(range(16 * P // 32 * w))
+        where = dict(zip(to_native.tolist(), to_planes.tolist()))
+        for r in range(16):
+            for g in range(P // 32):
+                for d in range(w):
+                    native = (r * (P // 32) + g) * w + d
+                    step, entry = g // 4, r + 16 * (g % 4)
+                    want = step * 64 * w + (entry * 4 + d if d < 4 else 256 + entry * (w - 4) + d - 4)
+                    assert where[native] == want
+
+
+def test_rows_widened_to_whole_tiles_on_the_host():
+    """widen_rows_to_whole_tiles on CPU tensors: every id survives (read back field by field), no row gets narrower,
+    every run of a width below the last is whole tiles."""
+    import torch
+    from qvb8_amd import ext_qvb8 as ext
+    from tests import helpers as H
+    for Q, P, widths in ((300, 128, [7, 6, 5]), (40, 128, [5, 6, 7, 8]), (31, 128, [6, 7]), (64, 128, [7]), (50, 128, [6, 9])):
+        d = H.mixed_width_pack(Q, P, widths, seed=Q)
+        ids, _, nbits, bit_off = H.to_device_args(d, "cpu")[:4]
+        wide = ext.widen_rows_to_whole_tiles(ids, nbits, bit_off, P)
+        if wide is None:
+            counts = sorted(zip(*[t.tolist() for t in torch.unique(nbits, return_counts=True)]))
+            assert all(n % 16 == 0 or nxt[0] > 8 for (_, n), nxt in zip(counts[:-1], counts[1:]))
+            continue
+        ids2, nb2, off2 = wide
+        assert bool((nb2 >= nbits).all())
+        buf = ids2.numpy()
+        for q in range(Q):
+            w = int(nb2[q])
+            for c in (0, 1, 31, 32, P // 2, P - 1):
+                pos = int(off2[q]) + c * w
+                v = int.from_bytes(buf[pos >> 3:(pos >> 3) + 4].tobytes(), "little")
+                assert (v >> (pos & 7)) & ((1 << w) - 1) == d["ids_dense"][q, c]
+        runs = sorted(zip(*[t.tolist() for t in torch.unique(nb2, return_counts=True)]))
+        for (w, n), (w_next, _) in zip(runs[:-1], runs[1:]):
+            assert n % 16 == 0 or w_next > 8, runs
