@@ -88,8 +88,17 @@ class QVBandEmbeddingV8(nn.Module):
         """The given rows as (n, P) fp32 band values, escapes NOT applied (embedding.py:97-124)."""
         return self._lookup(rows, torch.float32, False)
 
+    # An index outside 0..num_embeddings-1: the reference's gathers fail on it (IndexError on the CPU, a device-side
+    # assertion on the GPU).  Here the kernel writes a row of NaN and the call stays free of host reads, so that it can be
+    # captured in a graph; set check_indices = True to get the IndexError instead (one host read per call).
+    check_indices = False
+
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         """(*input.shape, P) in the output dtype, on the device `input` came from (embedding.py:126-158)."""
+        if self.check_indices and input.numel():
+            lo, hi = int(input.min()), int(input.max())
+            if lo < 0 or hi >= self.num_embeddings:
+                raise IndexError(f"embedding index {lo if lo < 0 else hi} outside 0..{self.num_embeddings - 1}")
         out = self._lookup(input, self._out_dtype, True)
         return out.reshape(*input.shape, self.embedding_dim).to(input.device)
 

@@ -113,33 +113,44 @@ def unband_kv_4d(banded: list, batch: int, heads: int, device="cpu") -> torch.Te
     return torch.stack(mats, dim=0).reshape(batch, heads, seq, dim)
 
 
+def _channel_grid(x, lo, span, widths):
+    """Nearest point of each channel's grid of 2^w - 1 intervals over [lo, lo + span] (w per head): (ids, step)."""
+    levels = torch.tensor([float((1 << w) - 1) for w in widths], device=x.device).view(-1, 1, 1)
+    step = (span / levels).clamp_min(STEP_FLOOR)
+    return torch.minimum(torch.round((x - lo) / step).clamp_(min=0), levels), step
+
+
 def band_kv_heads(t: torch.Tensor, orig_dtype: torch.dtype, bits: int, tau: float = 0.0, certify: bool = True) -> list:
     """(heads, seq, head_dim) -> one BandedKV per head (codec.py:175-241).  With certify and tau > 0, `bits` is a floor:
     a head's width rises (to 16 at most) until the decoder's own expression, rounded to `orig_dtype`, is within tau of
-    every element; KVCertificateError when 16 bits do not reach it."""
-    h, s, d = t.shape
+    every element; KVCertificateError when 16 bits do not reach it.  Heads are independent: only the heads that still
+    miss tau are quantised again, one host read per round."""
+    heads, seq, dim = t.shape
     x = torch.nan_to_num(t.detach().to(torch.float32), nan=0.0, posinf=0.0, neginf=0.0)
-    mn = x.amin(1, keepdim=True)
-    rng = x.amax(1, keepdim=True) - mn
-    do_cert = certify and tau > 0
-    if do_cert:
-        worst = rng.amax((1, 2)).cpu().tolist()
-        widths = [min(MAX_BITS, max(bits, math.ceil(math.log2(w / (2.0 * tau) + 1.0)))) if w > 0 else bits for w in worst]
-    else:
-        widths = [bits] * h
-    while True:
-        top = torch.tensor([float((1 << b) - 1) for b in widths], device=x.device).view(h, 1, 1)
-        step = (rng / top).clamp_min(STEP_FLOOR)
-        ids = torch.minimum(torch.round((x - mn) / step).clamp_(min=0), top)
-        if not do_cert:
+    lo = x.amin(1, keepdim=True)
+    span = x.amax(1, keepdim=True) - lo
+    widths = [bits] * heads
+    open_heads = []
+    if certify and tau > 0:
+        open_heads = list(range(heads))
+        for i, widest in enumerate(span.amax((1, 2)).cpu().tolist()):     # first guess: half a step within tau
+            if widest > 0:
+                widths[i] = min(MAX_BITS, max(bits, math.ceil(math.log2(widest / (2.0 * tau) + 1.0))))
+    ids, step = _channel_grid(x, lo, span, widths)
+    while open_heads:
+        sel = torch.tensor(open_heads, device=x.device)
+        shown = (lo[sel] + ids[sel] * step[sel]).to(orig_dtype).to(torch.float32)      # what the decoder will hand out
+        miss = (shown - x[sel]).abs().amax((1, 2)).cpu().tolist()
+        open_heads = [i for i, e in zip(open_heads, miss) if e > tau]
+        if not open_heads:
             break
-        errs = ((mn + ids * step).to(orig_dtype).to(torch.float32) - x).abs().amax((1, 2)).cpu().tolist()
-        bad = [i for i in range(h) if errs[i] > tau]
-        if not bad:
-            break
-        for i in bad:
+        worst = dict(zip(sel.tolist(), miss))
+        for i in open_heads:
             if widths[i] >= MAX_BITS:
-                raise KVCertificateError(f"head {i}: {MAX_BITS}-bit per-channel error {errs[i]:.4g} > tau={tau:g}")
+                raise KVCertificateError(f"head {i}: at {MAX_BITS} bits the per-channel grid is still {worst[i]:.4g} off, "
+                                         f"tau = {tau:g} cannot be certified for values stored as {orig_dtype}")
             widths[i] += 1
-    return [BandedKV(pack_ids(ids[i].to(torch.int64).reshape(-1), widths[i]), mn[i, 0].contiguous(), step[i, 0].contiguous(),
-                     widths[i], (s, d), orig_dtype, tau) for i in range(h)]
+        sel = torch.tensor(open_heads, device=x.device)
+        ids[sel], step[sel] = _channel_grid(x[sel], lo[sel], span[sel], [widths[i] for i in open_heads])
+    return [BandedKV(pack_ids(ids[i].to(torch.int64).reshape(-1), widths[i]), lo[i, 0].contiguous(), step[i, 0].contiguous(),
+                     widths[i], (seq, dim), orig_dtype, tau) for i in range(heads)]

@@ -114,6 +114,24 @@ def test_embedding_module_from_packfile(tmp_path):
         assert emb.tau_s.dtype == torch.float32 and torch.equal(emb.tau_s, before) and emb.esc_vals.dtype == torch.float32
 
 
+def test_embedding_index_outside_the_table():
+    """Where the reference's gathers fail on an index outside the table, this operator writes a row of NaN (no host read,
+    the other rows right); with check_indices it raises IndexError before any launch."""
+    Q, P = 40, 256
+    enc = PK.encode_tensor(H.synth_weight(Q, P, seed=5).to(DEV), 1e-3, restore="fp16")
+    a = H.pack_args(enc)
+    emb = QVBandEmbeddingV8(min_s=a[1], nbits=a[2], bit_off=a[3], ids=a[0], Q=Q, P=P, tau_s=a[5], esc_idx=a[6], esc_vals=a[7],
+                            out_dtype=torch.float32)
+    tokens = torch.tensor([3, Q, 39, -2], device=DEV)
+    y = emb(tokens)
+    assert bool(y[1].isnan().all()) and bool(y[3].isnan().all())
+    assert torch.equal(y[[0, 2]], emb(torch.tensor([3, 39], device=DEV))) and not bool(y[[0, 2]].isnan().any())
+    emb.check_indices = True
+    with pytest.raises(IndexError):
+        emb(tokens)
+    assert torch.equal(emb(torch.tensor([3, 39], device=DEV)), y[[0, 2]])
+
+
 def test_embedding_fp16_output_of_a_two_table_pack_needs_its_fp16_list(tmp_path):
     from qvb8_amd.common.errors import EscapeTableError
     W = H.synth_weight(32, 256, seed=2).to(DEV)
