@@ -210,6 +210,8 @@ def bench_moe(args, dev):
             Wd = (0.02 * torch.randn(hidden, inter, device=dev, generator=g)).to(torch.bfloat16)
             gu.append(QVBandLinearV8.from_encoded(PK.encode_tensor(Wg, 2e-3)))
             dn.append(QVBandLinearV8.from_encoded(PK.encode_tensor(Wd, 2e-3)))
+        if l == 0:                                    # an expert's bytes as encoded (the stack may store rows wider)
+            encoded_bytes_per_expert = sum(int(lin.ids.numel()) for lin in gu + dn) // E
         m = QVBandExpertsV8(gu, dn, num_experts=E)
         assert m.build_stack()
         stacks.append(m._stk)
@@ -220,7 +222,7 @@ def bench_moe(args, dev):
     # Every layer is called with several routings in turn (each its own random draw), until a step touches more than
     # 512 MB of distinct expert bytes: a replay then cannot be served from the 256 MB last-level cache.
     calls, step_bytes = [], 0
-    per_expert = (stacks[0][0]["ids"].numel() + stacks[0][1]["ids"].numel()) // E + 17 * (stacks[0][0]["Q"] + stacks[0][1]["Q"])
+    per_expert = encoded_bytes_per_expert + 17 * (stacks[0][0]["Q"] + stacks[0][1]["Q"])
     rounds = 0
     while step_bytes < (512 << 20) and rounds < 16:
         for g_, d_ in stacks:
@@ -238,7 +240,8 @@ def bench_moe(args, dev):
                                       g_["nbits"].data_ptr(), g_["bit_off"].data_ptr(), g_["Q"], g_["P"],
                                       d_["ids"].data_ptr(), d_["ids"].numel(), d_["min_s"].data_ptr(), d_["tau_s"].data_ptr(),
                                       d_["nbits"].data_ptr(), d_["bit_off"].data_ptr(), d_["Q"], d_["P"],
-                                      0, out.data_ptr(), 2, ws.data_ptr(), ws.numel(), s)
+                                      (0x100 if g_["regular"] else 0) | (0x200 if d_["regular"] else 0),   # what the operator passes
+                                      out.data_ptr(), 2, ws.data_ptr(), ws.numel(), s)
             if rc != 0:
                 raise RuntimeError(lib.qvb8_last_error().decode())
     ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)

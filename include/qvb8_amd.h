@@ -199,7 +199,15 @@ int qvb8_launch_probe(int64_t blocks, int64_t threads, int64_t lds_bytes, void* 
 
 enum qvb8_moe_act {
     QVB8_MOE_SILU_GATED = 0,  /* up rows = gate (first half) then up: H[i] = silu(Y[i]) * Y[I + i], Q_up == 2 * P_dn */
-    QVB8_MOE_RELU2 = 1        /* non-gated: H[i] = max(Y[i], 0)^2, Q_up == P_dn */
+    QVB8_MOE_RELU2 = 1,       /* non-gated: H[i] = max(Y[i], 0)^2, Q_up == P_dn */
+    /* Optional statements about a stack, ORed to the activation (a loader that stores the stack itself can make them true;
+     * no counterpart in the reference).  "Regular": every row of the stack has the width nbits[0], and row q of expert e
+     * starts at bit  bit_off[0] + e * (bit_off[Q] - bit_off[0]) + q * P * nbits[0].  The matrix-core paths (1..16 tokens)
+     * then work a row's place out instead of reading nbits / bit_off, which takes one dependent memory trip out of every
+     * launch; results are bit for bit those without the flag.  A stack for which the statement is false gives wrong
+     * results (never an access outside the ids buffer). */
+    QVB8_MOE_UP_REGULAR = 0x100,
+    QVB8_MOE_DOWN_REGULAR = 0x200
 };
 
 /* Bytes of workspace qvb8_moe_experts needs (routing plan + fp32 H (pairs, P_dn) + fp32 Yd (pairs, Q_dn)). */

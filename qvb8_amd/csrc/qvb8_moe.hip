@@ -336,7 +336,10 @@ struct MoeOneArgs {
     int tiles_per_wg;              // up: unit tiles per workgroup
 };
 
-template <int T, bool DOWN, bool XC, int DT>
+// REG: the caller states that every row of the stack has one width and that the rows lie at regular places (row q of
+// expert e at bit_off[0] + e * (bit_off[Q] - bit_off[0]) + q * P * width): the kernel then works a row's place out
+// instead of reading it, which takes one dependent memory trip out of every round.
+template <int T, bool DOWN, bool XC, int DT, bool REG>
 __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
     using F = Fmt<false>;
     using XI = XIn<false, XC>;
@@ -364,6 +367,10 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
     auto row0_of = [&](int i) { return DOWN ? (int)blockIdx.x * 16 : ((ut_first + i / RT) % UT) * 16 + (i % RT) * a.units; };
     const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
     const v4u_t ones = {F::one_bits, F::one_bits, F::one_bits, F::one_bits};
+    // REG: the stack's width, first bit and bits from one expert to the next (three reads that depend on nothing)
+    const int reg_nb = REG ? (int)a.nbits[0] : 0;
+    const int64_t reg_base = REG ? a.bit_off[0] : 0;
+    const int64_t reg_stride = REG ? a.bit_off[a.E > 1 ? a.Q : 0] - reg_base : 0;
 
     // A round = the row tiles the workgroup's waves work on at the same time.  (Two rounds of the up kernel in flight
     // together were measured: no faster -- a CU's share of the bytes, not the chain of trips, sets the time -- and the
@@ -401,8 +408,13 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
         const int64_t e = a.idx[slot_of(q.i)];
         q.e_ok = e >= 0 && e < a.E;
         const size_t mi = (size_t)(q.e_ok ? e : 0) * a.Q + row0_of(q.i) + r;
-        q.nb = a.nbits[mi];
-        q.bit0 = a.bit_off[mi];
+        if constexpr (REG) {
+            q.nb = reg_nb;
+            q.bit0 = reg_base + (int64_t)(q.e_ok ? e : 0) * reg_stride + (int64_t)(row0_of(q.i) + r) * a.P * reg_nb;
+        } else {
+            q.nb = a.nbits[mi];
+            q.bit0 = a.bit_off[mi];
+        }
         q.ts = a.tau_s[mi]; q.mn = a.min_s[mi];
     };
     auto request_ids = [&](Round& q, uint4 (&lo)[T], uint4 (&hi)[T]) {
@@ -426,8 +438,10 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) sx = F::mfma(xa[it][j], ones, sx);
         const uint32_t info = sliced ? ((uint32_t)nb | 256u) : 0u;
-        const uint32_t info0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
-        const bool uniform = __builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u;
+        // REG: one width for the whole stack, known without looking at the lanes (rows that cannot be read -- an expert
+        // number outside the stack -- decode whatever was loaded; their results are replaced by NaN below)
+        const uint32_t info0 = REG ? ((uint32_t)reg_nb | ((reg_nb >= 4 && reg_nb <= 8) ? 256u : 0u)) : (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
+        const bool uniform = REG ? (info0 >> 8) == 1u : (__builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u);
 #pragma unroll
         for (int it = 0; it < T; ++it) {
             v4u_t b[4];
@@ -443,11 +457,13 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) b[j] = v4u_t{F::bias_bits, F::bias_bits, F::bias_bits, F::bias_bits};
-                if (__builtin_amdgcn_ballot_w64(sliced && nb == 7)) { if (sliced && nb == 7) decode_slice<7, false>(lo, hi, b); }
-                if (__builtin_amdgcn_ballot_w64(sliced && nb == 6)) { if (sliced && nb == 6) decode_slice<6, false>(lo, hi, b); }
-                if (__builtin_amdgcn_ballot_w64(sliced && nb == 5)) { if (sliced && nb == 5) decode_slice<5, false>(lo, hi, b); }
-                if (__builtin_amdgcn_ballot_w64(sliced && nb == 4)) { if (sliced && nb == 4) decode_slice<4, false>(lo, hi, b); }
-                if (__builtin_amdgcn_ballot_w64(sliced && nb == 8)) { if (sliced && nb == 8) decode_slice<8, false>(lo, hi, b); }
+                if constexpr (!REG) {
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 7)) { if (sliced && nb == 7) decode_slice<7, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 6)) { if (sliced && nb == 6) decode_slice<6, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 5)) { if (sliced && nb == 5) decode_slice<5, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 4)) { if (sliced && nb == 4) decode_slice<4, false>(lo, hi, b); }
+                    if (__builtin_amdgcn_ballot_w64(sliced && nb == 8)) { if (sliced && nb == 8) decode_slice<8, false>(lo, hi, b); }
+                }
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc = F::mfma(xa[it][j], b[j], acc);
@@ -557,7 +573,7 @@ constexpr int kWalkMaxRowTiles = 16;   // row tiles per segment: one row record 
 
 struct WalkRow { int64_t bit0; int flags; float ts, mn; int nat; };       // flags = width | usable << 8 | sliced << 9; nat = place before the sort
 
-template <int T, bool DOWN, bool XC, bool TWO>
+template <int T, bool DOWN, bool XC, bool TWO, bool REG>
 __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
     using F = Fmt<false>;
     using XI = XIn<false, XC>;
@@ -584,6 +600,10 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
     const int64_t clamp_byte = (a.ids_bytes - 8) & ~(int64_t)3;
     const v4u_t ones = {F::one_bits, F::one_bits, F::one_bits, F::one_bits};
 
+    // REG (one width, rows at regular places, see moe_one_kernel): the stack's width, first bit, bits between experts
+    const int reg_nb = REG ? (int)a.nbits[0] : 0;
+    const int64_t reg_base = REG ? a.bit_off[0] : 0;
+    const int64_t reg_stride = REG ? a.bit_off[a.E > 1 ? a.Q : 0] - reg_base : 0;
     const int n_active = a.plan.n_bad[1];
     const int per_expert = max(1, (int)gridDim.x / max(1, n_active));
     const int sl = (int)blockIdx.x / per_expert;
@@ -611,9 +631,16 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
         const int n_rows = n_rt * 16;
         int key = 7, rank = 0;
         WalkRow mine{0, 0, 0.f, 0.f, 0};
-        const size_t mi = (size_t)(e_ok ? e : 0) * a.Q + (tid < n_rows ? row0_of(tid >> 4) + (tid & 15) : 0);
-        const int nb = a.nbits[mi];
-        const int64_t bit0 = a.bit_off[mi];
+        const int row_in_expert = tid < n_rows ? row0_of(tid >> 4) + (tid & 15) : 0;
+        const size_t mi = (size_t)(e_ok ? e : 0) * a.Q + row_in_expert;
+        int nb; int64_t bit0;
+        if constexpr (REG) {
+            nb = reg_nb;
+            bit0 = reg_base + (int64_t)(e_ok ? e : 0) * reg_stride + (int64_t)row_in_expert * a.P * reg_nb;
+        } else {
+            nb = a.nbits[mi];
+            bit0 = a.bit_off[mi];
+        }
         const float row_ts = a.tau_s[mi], row_mn = a.min_s[mi];
         const uint16_t* xrow = a.X + (size_t)(DOWN ? pair : pair / a.topk) * a.P;
 #pragma unroll
@@ -623,12 +650,21 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) xa[it][j] = *reinterpret_cast<const v4u_t*>(xp + 8 * j);
         }
+        bool row_usable = false;
         if (tid < n_rows) {
             const bool ok = e_ok && nb >= 1 && nb <= 14 && bit0 >= 0 && ((bit0 + (int64_t)nb * a.P + 7) >> 3) + 8 <= a.ids_bytes;
             const bool sliced = ok && nb >= 4 && nb <= 8 && (bit0 & 31) == 0;
-            mine = WalkRow{ok ? bit0 : 0, nb | (ok ? 256 : 0) | (sliced ? 512 : 0), row_ts, row_mn, tid};
+            row_usable = ok;
+            // REG: the record is complete without anything read from memory; tau_s and min_s go to LDS further down,
+            // behind the first requests for ids
+            mine = WalkRow{ok ? bit0 : 0, nb | (ok ? 256 : 0) | (sliced ? 512 : 0), REG ? 0.f : row_ts, REG ? 0.f : row_mn, tid};
             key = sliced ? nb - 4 : 5;
         }
+        if constexpr (REG) {
+            // one width: the rows stay where they are
+            if (tid < n_rows) { s_row[tid] = mine; s_pos[tid] = (uint16_t)tid; }
+            __syncthreads();
+        } else {
 #pragma unroll
         for (int c = 0; c < 6; ++c) {
             const uint64_t m = __builtin_amdgcn_ballot_w64(key == c);
@@ -647,6 +683,7 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
             s_pos[tid] = (uint16_t)(base + rank);
         }
         __syncthreads();
+        }
 
         const int n_rounds = (n_rt + G - 1) / G;
         // Requests the lane's slices of the wave's tile of round `rnd` (clamped to the last round: nothing under a branch,
@@ -668,6 +705,7 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
         };
         uint4 lo0[T], hi0[T], lo1[T], hi1[T];
         WalkRow rec0 = issue(0, lo0, hi0), rec1{0, 0, 0.f, 0.f, 0};     // by every wave: nothing under a branch
+        if constexpr (REG) { if (tid < n_rows) s_fin[tid] = float2{row_usable ? row_ts : __builtin_nanf(""), row_mn}; }
         {
             // rows past the pairs and steps past the row multiply zeros; bf16 activations are narrowed like every activation
 #pragma unroll
@@ -695,8 +733,9 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
             const int nbr = rec.flags & 255;
             const bool sliced = (rec.flags & 512) != 0;
             const uint32_t info = sliced ? ((uint32_t)nbr | 256u) : 0u;
-            const uint32_t info0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
-            const bool uniform = __builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u;
+            // REG: one width for the whole stack (rows that cannot be read decode what was loaded and end as NaN)
+            const uint32_t info0 = REG ? ((uint32_t)reg_nb | ((reg_nb >= 4 && reg_nb <= 8) ? 256u : 0u)) : (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
+            const bool uniform = REG ? (info0 >> 8) == 1u : (__builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u);
 #pragma unroll
             for (int it = 0; it < T; ++it) {
                 v4u_t b[4];
@@ -712,11 +751,13 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) b[j] = v4u_t{F::bias_bits, F::bias_bits, F::bias_bits, F::bias_bits};
-                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 7)) { if (sliced && nbr == 7) decode_slice<7, false>(lo, hi, b); }
-                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 6)) { if (sliced && nbr == 6) decode_slice<6, false>(lo, hi, b); }
-                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 5)) { if (sliced && nbr == 5) decode_slice<5, false>(lo, hi, b); }
-                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 4)) { if (sliced && nbr == 4) decode_slice<4, false>(lo, hi, b); }
-                    if (__builtin_amdgcn_ballot_w64(sliced && nbr == 8)) { if (sliced && nbr == 8) decode_slice<8, false>(lo, hi, b); }
+                    if constexpr (!REG) {
+                        if (__builtin_amdgcn_ballot_w64(sliced && nbr == 7)) { if (sliced && nbr == 7) decode_slice<7, false>(lo, hi, b); }
+                        if (__builtin_amdgcn_ballot_w64(sliced && nbr == 6)) { if (sliced && nbr == 6) decode_slice<6, false>(lo, hi, b); }
+                        if (__builtin_amdgcn_ballot_w64(sliced && nbr == 5)) { if (sliced && nbr == 5) decode_slice<5, false>(lo, hi, b); }
+                        if (__builtin_amdgcn_ballot_w64(sliced && nbr == 4)) { if (sliced && nbr == 4) decode_slice<4, false>(lo, hi, b); }
+                        if (__builtin_amdgcn_ballot_w64(sliced && nbr == 8)) { if (sliced && nbr == 8) decode_slice<8, false>(lo, hi, b); }
+                    }
                 }
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc = F::mfma(xa[it][j], b[j], acc);
@@ -728,7 +769,7 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
                     const int t = kg * 4 + k;
                     if (t < n) s_part[(((size_t)i * W + wc) * 16 + r) * n + t] = __builtin_fmaf(-F::bias, sx[k], acc[k]);
                 }
-                if (kg == 0 && wc == 0) s_fin[i * 16 + r] = float2{(rec.flags & 256) ? rec.ts : __builtin_nanf(""), rec.mn};
+                if constexpr (!REG) { if (kg == 0 && wc == 0) s_fin[i * 16 + r] = float2{(rec.flags & 256) ? rec.ts : __builtin_nanf(""), rec.mn}; }
                 // rows the slicing cannot read: element by element over this wave's columns, token by token
                 uint64_t odd = __builtin_amdgcn_ballot_w64(kg == 0 && !sliced);
                 while (odd) {
@@ -803,14 +844,14 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
 }
 
 // rows of up to 2048 columns: within 256 registers, two workgroups per CU (one starts while the other walks)
-template <int T, bool DOWN, bool XC, bool TWO>
+template <int T, bool DOWN, bool XC, bool TWO, bool REG>
 __global__ void __launch_bounds__(64 * kWalkWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) moe_walk_kernel(MoeWalkArgs a) {
-    moe_walk_body<T, DOWN, XC, TWO>(a);
+    moe_walk_body<T, DOWN, XC, TWO, REG>(a);
 }
 // longer rows: eight steps of activations per wave need more registers, one workgroup per CU
-template <bool DOWN, bool XC>
+template <bool DOWN, bool XC, bool REG>
 __global__ void __launch_bounds__(64 * kWalkWaves) moe_walk_wide_kernel(MoeWalkArgs a) {
-    moe_walk_body<8, DOWN, XC, false>(a);
+    moe_walk_body<8, DOWN, XC, false, REG>(a);
 }
 
 template <int DT>
@@ -876,19 +917,23 @@ bool moe_group_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t P_up, int64
     return moe_walk_shapes_ok(topk, x_dtype, P_up, Q_dn, P_dn) && host::env_int("QVB8_MOE_GROUPED", 1) != 0;
 }
 
-template <bool DOWN, bool XC, int DT>
-int launch_moe_one(const MoeOneArgs& a, unsigned blocks, unsigned tokens, hipStream_t s) {
+template <bool DOWN, bool XC, int DT, bool REG>
+int launch_moe_one_as(const MoeOneArgs& a, unsigned blocks, unsigned tokens, hipStream_t s) {
     const int n_steps = a.P / kStepCols;
     // six steps per wave only for the down kernel (one round in flight): a whole row of up to 768 columns per wave, so
     // that eight slots are one round
     if constexpr (DOWN) {
         if (n_steps <= 6) {
-            hipLaunchKernelGGL((moe_one_kernel<6, DOWN, XC, DT>), dim3(blocks, tokens), dim3(64 * kOneWaves), 0, s, a);
+            hipLaunchKernelGGL((moe_one_kernel<6, DOWN, XC, DT, REG>), dim3(blocks, tokens), dim3(64 * kOneWaves), 0, s, a);
             return host::check_launch("qvb8_moe_experts");
         }
     }
-    hipLaunchKernelGGL((moe_one_kernel<4, DOWN, XC, DT>), dim3(blocks, tokens), dim3(64 * kOneWaves), 0, s, a);
+    hipLaunchKernelGGL((moe_one_kernel<4, DOWN, XC, DT, REG>), dim3(blocks, tokens), dim3(64 * kOneWaves), 0, s, a);
     return host::check_launch("qvb8_moe_experts");
+}
+template <bool DOWN, bool XC, int DT>
+int launch_moe_one(const MoeOneArgs& a, bool regular, unsigned blocks, unsigned tokens, hipStream_t s) {
+    return regular ? launch_moe_one_as<DOWN, XC, DT, true>(a, blocks, tokens, s) : launch_moe_one_as<DOWN, XC, DT, false>(a, blocks, tokens, s);
 }
 
 size_t moe_walk_lds(int64_t row_tiles, int W, int max_tokens) {
@@ -897,8 +942,8 @@ size_t moe_walk_lds(int64_t row_tiles, int W, int max_tokens) {
 }
 
 // `slots`: the plan's slots (experts that can be in use)
-template <bool DOWN, bool XC>
-int launch_moe_walk(MoeWalkArgs a, int64_t slots, int64_t max_tokens, hipStream_t s) {
+template <bool DOWN, bool XC, bool REG>
+int launch_moe_walk_as(MoeWalkArgs a, int64_t slots, int64_t max_tokens, hipStream_t s) {
     const int n_steps = a.P / kStepCols;
     // steps per wave: four, with the next tile's ids in flight; a short down row (up to 768 columns) is one wave's; rows
     // beyond 2048 columns take eight steps per wave and one register set
@@ -919,13 +964,17 @@ int launch_moe_walk(MoeWalkArgs a, int64_t slots, int64_t max_tokens, hipStream_
     dim3 grid((unsigned)wgs), block(64 * kWalkWaves);
     if constexpr (DOWN) {
         if (T == 6) {
-            hipLaunchKernelGGL((moe_walk_kernel<6, true, XC, false>), grid, block, lds, s, a);
+            hipLaunchKernelGGL((moe_walk_kernel<6, true, XC, false, REG>), grid, block, lds, s, a);
             return host::check_launch("qvb8_moe_experts");
         }
     }
-    if (T == 4) hipLaunchKernelGGL((moe_walk_kernel<4, DOWN, XC, true>), grid, block, lds, s, a);
-    else hipLaunchKernelGGL((moe_walk_wide_kernel<DOWN, XC>), grid, block, lds, s, a);
+    if (T == 4) hipLaunchKernelGGL((moe_walk_kernel<4, DOWN, XC, true, REG>), grid, block, lds, s, a);
+    else hipLaunchKernelGGL((moe_walk_wide_kernel<DOWN, XC, REG>), grid, block, lds, s, a);
     return host::check_launch("qvb8_moe_experts");
+}
+template <bool DOWN, bool XC>
+int launch_moe_walk(const MoeWalkArgs& a, bool regular, int64_t slots, int64_t max_tokens, hipStream_t s) {
+    return regular ? launch_moe_walk_as<DOWN, XC, true>(a, slots, max_tokens, s) : launch_moe_walk_as<DOWN, XC, false>(a, slots, max_tokens, s);
 }
 }  // namespace
 
@@ -943,7 +992,10 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
                                 const uint8_t* dn_nb, const int64_t* dn_off, int64_t Q_dn, int64_t P_dn,
                                 int act, void* out, int out_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
     if (tokens < 0 || topk < 1 || n_experts < 1 || n_experts > 8192) return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: bad token / top-k / expert count");
-    if (act != 0 && act != 1) return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: act must be 0 (gated SiLU) or 1 (ReLU squared)");
+    if ((act & ~(QVB8_MOE_UP_REGULAR | QVB8_MOE_DOWN_REGULAR)) != 0 && (act & ~(QVB8_MOE_UP_REGULAR | QVB8_MOE_DOWN_REGULAR)) != 1)
+        return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: act must be 0 (gated SiLU) or 1 (ReLU squared), with the QVB8_MOE_*_REGULAR flags at most");
+    const bool up_regular = (act & QVB8_MOE_UP_REGULAR) != 0, dn_regular = (act & QVB8_MOE_DOWN_REGULAR) != 0;
+    act &= 0xFF;
     if (Q_up <= 0 || P_up <= 0 || Q_dn <= 0 || P_dn <= 0 || Q_up > 0x7fffffff || P_up > 0x7fffffff || Q_dn > 0x7fffffff || P_dn > 0x7fffffff)
         return host::fail(QVB8_ERR_ARG, "qvb8_moe_experts: bad shape");
     if (act == 0 ? (Q_up % 2 != 0 || Q_up / 2 != P_dn) : (Q_up != P_dn)) return host::fail(QVB8_ERR_ARG, "moe: gate_up/down shapes disagree");
@@ -982,14 +1034,14 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
         o.tiles_per_wg = (int)per_wg;
         const unsigned up_blocks = (unsigned)((total_ut + per_wg - 1) / per_wg);
         const unsigned tk = (unsigned)tokens;
-        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_one<false, true, 0>(o, up_blocks, tk, s) : launch_moe_one<false, false, 0>(o, up_blocks, tk, s)) return rc;
+        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_one<false, true, 0>(o, up_regular, up_blocks, tk, s) : launch_moe_one<false, false, 0>(o, up_regular, up_blocks, tk, s)) return rc;
         o.X = reinterpret_cast<const uint16_t*>(H); o.ids = dn_ids; o.ids_bytes = dn_ids_bytes;
         o.min_s = dn_min; o.tau_s = dn_tau; o.nbits = dn_nb; o.bit_off = dn_off; o.out = out;
         o.Q = (int)Q_dn; o.P = (int)P_dn; o.units = (int)Q_dn; o.gated = 0; o.tiles_per_wg = 0;
         const unsigned dn_blocks = (unsigned)(Q_dn / 16);
-        if (out_dtype == QVB8_F32) return launch_moe_one<true, false, 0>(o, dn_blocks, tk, s);
-        if (out_dtype == QVB8_F16) return launch_moe_one<true, false, 1>(o, dn_blocks, tk, s);
-        return launch_moe_one<true, false, 2>(o, dn_blocks, tk, s);
+        if (out_dtype == QVB8_F32) return launch_moe_one<true, false, 0>(o, dn_regular, dn_blocks, tk, s);
+        if (out_dtype == QVB8_F16) return launch_moe_one<true, false, 1>(o, dn_regular, dn_blocks, tk, s);
+        return launch_moe_one<true, false, 2>(o, dn_regular, dn_blocks, tk, s);
     }
 
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)(n_experts + 8) * 4, s, idx, (int)np, (int)n_experts, pl);
@@ -1001,11 +1053,11 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
         wa.min_s = up_min; wa.tau_s = up_tau; wa.nbits = up_nb; wa.bit_off = up_off; wa.out = H;                // H as fp16 (pairs, P_dn)
         wa.E = (int)n_experts; wa.Q = (int)Q_up; wa.P = (int)P_up; wa.topk = (int)topk; wa.units = (int)P_dn; wa.gated = act == 0 ? 1 : 0;
         wa.tiles_per_seg = 1; wa.max_tokens = 1;
-        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_walk<false, true>(wa, slots, tokens, s) : launch_moe_walk<false, false>(wa, slots, tokens, s)) return rc;
+        if (int rc = x_dtype == QVB8_BF16 ? launch_moe_walk<false, true>(wa, up_regular, slots, tokens, s) : launch_moe_walk<false, false>(wa, up_regular, slots, tokens, s)) return rc;
         wa.X = reinterpret_cast<const uint16_t*>(H); wa.ids = dn_ids; wa.ids_bytes = dn_ids_bytes;
         wa.min_s = dn_min; wa.tau_s = dn_tau; wa.nbits = dn_nb; wa.bit_off = dn_off; wa.out = Yd;
         wa.Q = (int)Q_dn; wa.P = (int)P_dn; wa.units = (int)Q_dn; wa.gated = 0;
-        if (int rc = launch_moe_walk<true, false>(wa, slots, tokens, s)) return rc;
+        if (int rc = launch_moe_walk<true, false>(wa, dn_regular, slots, tokens, s)) return rc;
         dim3 cgrid((unsigned)((Q_dn + 255) / 256), (unsigned)tokens);
         if (out_dtype == QVB8_F32) hipLaunchKernelGGL(moe_combine_kernel<0>, cgrid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);
         else if (out_dtype == QVB8_F16) hipLaunchKernelGGL(moe_combine_kernel<1>, cgrid, dim3(256), 0, s, Yd, w, out, (int)topk, (int)Q_dn, (int)tokens, pl.n_bad);

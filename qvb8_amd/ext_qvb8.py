@@ -239,6 +239,59 @@ def rows_back_to_back(ids, row_nbits, row_bit_off, P):
     return out, new_off
 
 
+def tile_uniform_widths(row_nbits, tile_rows=16, lo=4, hi=8):
+    """Per-row widths that make every tile of `tile_rows` consecutive rows (in row order) one width: each row of a tile
+    whose widths all lie in lo..hi gets the tile's largest width; other rows keep theirs.  None when nothing changes."""
+    Q = row_nbits.numel()
+    whole = Q // tile_rows * tile_rows
+    if whole == 0:
+        return None
+    nb = row_nbits[:whole].to(torch.int64).view(-1, tile_rows)
+    top, low = nb.amax(1, keepdim=True), nb.amin(1, keepdim=True)
+    target = torch.where((low >= lo) & (top <= hi), top.expand_as(nb), nb).reshape(-1)
+    if bool((target == row_nbits[:whole]).all()):
+        return None
+    out = row_nbits.clone()
+    out[:whole] = target.to(row_nbits.dtype)
+    return out
+
+
+def repack_rows(ids, row_nbits, row_bit_off, P, new_nbits, chunk_rows=256):
+    """The rows stored again back to back, in row order from byte 0, row q in fields of new_nbits[q] >= row_nbits[q] bits:
+    the ids, and with them every value of the weight, are unchanged.  Returns (ids, row_bit_off); None when P % 8 != 0."""
+    P = int(P)
+    if P % 8 != 0:
+        return None
+    ids, row_bit_off = rows_back_to_back(ids, row_nbits, row_bit_off, P)
+    old, new = row_nbits.to(torch.int64), new_nbits.to(torch.int64)
+    if bool((new < old).any()):
+        raise RuntimeError("repack_rows: a row cannot be stored in fewer bits than it has")
+    row_bits = new * P
+    new_off = torch.cumsum(row_bits, 0) - row_bits
+    total = int(row_bits.sum().item()) // 8
+    out = torch.zeros(total + 8, dtype=torch.uint8, device=ids.device)
+    dev = ids.device
+    cols = torch.arange(P, device=dev, dtype=torch.int64)
+    for w0, w1 in torch.unique(torch.stack([old, new], 1), dim=0).tolist():          # one host read, at load
+        rows = torch.nonzero((old == w0) & (new == w1)).reshape(-1)
+        nbytes = P * w1 // 8
+        span = torch.arange(nbytes, device=dev, dtype=torch.int64)
+        for k in range(0, rows.numel(), chunk_rows):
+            r = rows[k:k + chunk_rows]
+            src, dst = row_bit_off[r], new_off[r] >> 3
+            if w0 == w1 and bool((src % 8 == 0).all()):
+                out[(dst[:, None] + span[None, :]).reshape(-1)] = ids[((src >> 3)[:, None] + span[None, :]).reshape(-1)]
+                continue
+            pos = src[:, None] + cols[None, :] * w0
+            byte, sh = pos >> 3, pos & 7
+            word = ids[byte].to(torch.int64) | (ids[byte + 1].to(torch.int64) << 8) | (ids[byte + 2].to(torch.int64) << 16)
+            val = ((word >> sh) & ((1 << w0) - 1)).to(torch.int32)
+            bits = ((val[:, :, None] >> torch.arange(w1, device=dev, dtype=torch.int32)) & 1).reshape(r.numel(), -1, 8)
+            packed = (bits << torch.arange(8, device=dev, dtype=torch.int32)).sum(2).to(torch.uint8)
+            out[(dst[:, None] + span[None, :]).reshape(-1)] = packed.reshape(-1)
+    return out, new_off
+
+
 def widen_rows_to_whole_tiles(ids, row_nbits, row_bit_off, P, tile_rows=16, top=8):
     """Stores a few rows with more bits than they need so that, sorted by width, every run of one width is a whole number
     of 16-row tiles: of each width (ascending) the last `count % 16` rows move up to the next width present (up to
@@ -493,12 +546,29 @@ def _moe(act, X, idx, w, up_ids, up_min, up_tau, up_nb, up_off, Qup, Pup, dn_ids
     return out
 
 
-def moe_experts(X, idx, w, gu_ids, gu_min, gu_tau, gu_nb, gu_off, Qgu, Pgu, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn):
+MOE_UP_REGULAR, MOE_DOWN_REGULAR = 0x100, 0x200      # qvb8_moe_act flags: one width per stack, rows at regular places
+
+
+def stack_is_regular(nbits, bit_off, P) -> bool:
+    """Whether a stack's (experts, Q) tables are what QVB8_MOE_*_REGULAR states: one width, row q of expert e at
+    bit_off[0, 0] + e * (bit_off[1, 0] - bit_off[0, 0]) + q * P * width (one host read)."""
+    E, Q = nbits.shape
+    w = nbits.reshape(-1)[0].to(torch.int64)
+    base = bit_off.reshape(-1)[0]
+    stride = bit_off[1, 0] - base if E > 1 else torch.zeros((), dtype=torch.int64, device=bit_off.device)
+    want = base + torch.arange(E, device=bit_off.device).view(E, 1) * stride + torch.arange(Q, device=bit_off.device).view(1, Q) * (int(P) * w)
+    return bool((nbits == nbits.reshape(-1)[0]).all() & (bit_off == want).all())
+
+
+def moe_experts(X, idx, w, gu_ids, gu_min, gu_tau, gu_nb, gu_off, Qgu, Pgu, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn,
+                regular=(False, False)):
     """Routed gated-SiLU expert stack on the stacked layout (reference: qvb8_cuda.cu:937-992); returns (tokens, Qdn)
-    in X's dtype."""
-    return _moe(0, X, idx, w, gu_ids, gu_min, gu_tau, gu_nb, gu_off, Qgu, Pgu, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn)
+    in X's dtype.  `regular` = (up, down): the caller states that the stack is regular (stack_is_regular)."""
+    act = 0 | (MOE_UP_REGULAR if regular[0] else 0) | (MOE_DOWN_REGULAR if regular[1] else 0)
+    return _moe(act, X, idx, w, gu_ids, gu_min, gu_tau, gu_nb, gu_off, Qgu, Pgu, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn)
 
 
-def moe_experts_relu2(X, idx, w, up_ids, up_min, up_tau, up_nb, up_off, Qup, Pup, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn):
+def moe_experts_relu2(X, idx, w, up_ids, up_min, up_tau, up_nb, up_off, Qup, Pup, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn,
+                      regular=(False, False)):
     """Non-gated expert stack with H = relu(up(x))^2 (reference: qvb8_cuda.cu:1002-1055)."""
-    return _moe(1, X, idx, w, up_ids, up_min, up_tau, up_nb, up_off, Qup, Pup, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn)
+    return _moe(1 | (MOE_UP_REGULAR if regular[0] else 0) | (MOE_DOWN_REGULAR if regular[1] else 0), X, idx, w, up_ids, up_min, up_tau, up_nb, up_off, Qup, Pup, dn_ids, dn_min, dn_tau, dn_nb, dn_off, Qdn, Pdn)

@@ -263,3 +263,44 @@ def test_moe_config4_all_128_experts():
         x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(torch.bfloat16)
         out = mod(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
         _check(out, O.moe_reference(x.float().numpy(), idx, w, Wgu, Wdn), torch.bfloat16)
+
+
+@pytest.mark.parametrize("T", [1, 2, 5, 16])
+def test_moe_regular_stack_changes_no_result(T, monkeypatch):
+    """QVBandExpertsV8 stores a stack whose widths lie close together in ONE width, rows in row order at regular places,
+    and tells the kernels (QVB8_MOE_*_REGULAR): the results are bit for bit those of the stack as the files have it
+    (QVB8_MOE_UNIFORM_TILES=0), and within tolerance of the oracle; a stack that is not regular is never claimed to be."""
+    E, hidden, inter, k = 6, 256, 128, 2
+    idx, w = _route(T, E, k, seed=T)
+    x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(torch.bfloat16).to(DEV)
+    outs = {}
+    monkeypatch.setenv("QVB8_MOE_ONE_WIDTH_GROWTH", "0.25")      # the short rows of this test spread over two widths evenly
+    for flag in ("0", "1"):
+        monkeypatch.setenv("QVB8_MOE_UNIFORM_TILES", flag)
+        gu, dn, Wgu, Wdn = [], [], [], []
+        for e in range(E):                              # normal weights: rows of two neighbouring widths, mixed at random
+            for lst, Wl, (Q, P) in ((gu, Wgu, (2 * inter, hidden)), (dn, Wdn, (hidden, inter))):
+                W = (0.02 * torch.randn(Q, P, generator=torch.Generator().manual_seed(700 + 2 * e + len(lst)))).to(torch.bfloat16).to(DEV)
+                enc = PK.encode_tensor(W, 2e-3, restore="fp16")
+                assert enc["esc_idx"].numel() == 0 and int(enc["nbits"].min()) < int(enc["nbits"].max())
+                lst.append(QVBandLinearV8.from_encoded(enc))
+                v = H.oracle_view(enc)
+                Wl.append(O.reconstruct(v["min_s"], v["tau_s"], H.oracle_ids(v), v["esc_idx"], v["esc_vals"]))
+        mod = QVBandExpertsV8(gu, dn, num_experts=E)
+        assert mod.build_stack()
+        g, d = mod._stk
+        if flag == "1":
+            assert g["regular"] and d["regular"] and int(g["nbits"].min()) == int(g["nbits"].max())
+            assert ext.stack_is_regular(g["nbits"], g["bit_off"], hidden) and ext.stack_is_regular(d["nbits"], d["bit_off"], inter)
+        else:
+            assert not g["regular"] and not d["regular"]
+        outs[flag] = mod(x, torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
+        # the experts' own modules still give what they gave: the stack holds their rows, wider or not
+        one = gu[1](x)
+        ref1 = x.float().cpu().numpy().astype(np.float64) @ Wgu[1].astype(np.float64).T
+        assert float(np.abs(one.float().cpu().numpy() - ref1).max()) <= 2e-2 * float(np.abs(ref1).max())
+    assert torch.equal(outs["0"], outs["1"])
+    _check(outs["1"], O.moe_reference(x.float().cpu().numpy(), idx, w, Wgu, Wdn), torch.bfloat16)
+    # a claim that does not hold is not made for a stack built by hand
+    ops, _ = _hand_made_stack(3, 64, 128, [5, 6], seed=5)
+    assert not ext.stack_is_regular(ops[3], ops[4], 128)
