@@ -551,9 +551,10 @@ __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t* __restri
 
 // The workgroup's rows are positions [pos0, pos0 + 256) of a run of width NB that ends at pos_end and starts at byte
 // run_byte0 (position run_first) of the ids buffer.
-template <int MT, bool BF, int NB>
+template <int MT, bool BF, bool XC, int NB>
 __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_end, int run_first, uint64_t run_byte0, unsigned char* smem) {
     using F = Fmt<BF>;
+    using XI = XIn<BF, XC>;
     constexpr int TMK = 32 * MT;                   // rows of X per workgroup
     constexpr int XL = TMK * 16 / 256;             // 16-byte pieces of a stage per thread
     unsigned char* xs = smem;                                              // [2][TMK][kGemmXStride]
@@ -623,13 +624,29 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
 #pragma unroll
         for (int i = 0; i < XL; ++i) g[i] = *reinterpret_cast<const v4u_t*>(x_base + (size_t)min(tok0 + xrow + 16 * i, M - 1) * P + c);
     };
+    // XC: bf16 activations are narrowed like saturating_half on their way into LDS (every workgroup narrows the 16 KB it
+    // stages; a pass of its own over X would be one more launch per product)
     auto store_x = [=](int buf, const v4u_t (&g)[XL]) {
 #pragma unroll
-        for (int i = 0; i < XL; ++i)
-            *reinterpret_cast<v4u_t*>(xs + ((size_t)buf * TMK + xrow + 16 * i) * kGemmXStride + 16 * xch) = g[i];
+        for (int i = 0; i < XL; ++i) {
+            v4u_t v = g[i];
+            if constexpr (XC) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] = XI::pair(v[k]);
+            }
+            *reinterpret_cast<v4u_t*>(xs + ((size_t)buf * TMK + xrow + 16 * i) * kGemmXStride + 16 * xch) = v;
+        }
     };
 
     v16f_t acc[2][MT];
+    // sums of the rows of X over this workgroup's columns, as the operands see them: the product with a matrix of ones,
+    // in the accumulator layout (register i of every lane <-> the token that acc[.][mt][i] belongs to)
+    v16f_t sxa[MT];
+    const v4u_t ones = {F::one_bits, F::one_bits, F::one_bits, F::one_bits};
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sxa[mt][i] = 0.f;
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
@@ -661,6 +678,7 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
                     const v4u_t av = {v.x, v.y, v.z, v.w};
 #pragma unroll
                     for (int rt = 0; rt < 2; ++rt) acc[rt][mt] = F::mfma32(av, b[rt][j], acc[rt][mt]);
+                    sxa[mt] = F::mfma32(av, ones, sxa[mt]);
                 }
             if (h == 1) {
                 store_x(buf ^ 1, xg);
@@ -669,9 +687,6 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
         }
     }
     // ---- the end: lane holds, for row n of each row tile, tokens 32 mt + 8 (i / 4) + 4 kh + i % 4 ----
-    float* sxs = reinterpret_cast<float*>(smem);                           // the X stages are no longer read (barrier above)
-    if (tid < TMK) sxs[tid] = tok0 + tid < a.M ? a.sx[(size_t)blockIdx.z * a.M + tok0 + tid] : 0.f;
-    __syncthreads();
     float* out = a.out + (size_t)blockIdx.z * (size_t)a.M * (size_t)a.Q;
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
@@ -686,7 +701,7 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
                 const int tl = 32 * mt + 8 * (i >> 2) + 4 * kh + (i & 3);
                 const int t = tok0 + tl;
                 if (t < a.M) {
-                    const float sx = sxs[tl];
+                    const float sx = sxa[mt][i];
                     const float d = __builtin_fmaf(-F::bias, sx, acc[rt][mt][i]);
                     store_y(out, a.out_dt, (int64_t)t * a.Q + f.z, (float)(ts * (double)d + mn * (double)sx));
                 }
@@ -694,7 +709,7 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
     }
 }
 
-template <int MT, bool BF>
+template <int MT, bool BF, bool XC>
 __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     // which run of equal widths this workgroup's 256 positions belong to
@@ -708,11 +723,11 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     const int pos0 = run_first + (bx - (c == 0 ? 0 : c == 1 ? a.blocks1 : a.blocks2)) * kGemmRows;
     if (pos0 >= run_end) return;
     switch (c == 0 ? nb0 : c == 1 ? nb1 : nb2) {
-        case 4: gemm_run<MT, BF, 4>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 5: gemm_run<MT, BF, 5>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 6: gemm_run<MT, BF, 6>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 7: gemm_run<MT, BF, 7>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 8: if constexpr (!BF) gemm_run<MT, BF, 8>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 4: gemm_run<MT, BF, XC, 4>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 5: gemm_run<MT, BF, XC, 5>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 6: gemm_run<MT, BF, XC, 6>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 7: gemm_run<MT, BF, XC, 7>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 8: if constexpr (!BF) gemm_run<MT, BF, XC, 8>(a, pos0, run_end, run_first, byte0, smem); break;
         default: break;
     }
 }
@@ -1117,17 +1132,17 @@ GemmPlan plan_gemm_for(int64_t M, int64_t Q, int64_t P) { return M >= gemm2_from
 // kernel is the alternative).
 int gemm_from() { const int v = host::env_int("QVB8_MMA_GEMM_FROM", 33); return v < 17 ? 17 : (v > 49 ? 49 : v); }
 
-template <int MT, bool BF>
+template <int MT, bool BF, bool XC>
 int launch_gemm(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_t s) {
     static bool attr[64] = {false};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: no current device");
     if (!attr[dev]) {
-        if (hipFuncSetAttribute((const void*)gemm_kernel<MT, BF>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)gemm_kernel<MT, BF, XC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds) != hipSuccess)
             return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: cannot raise the kernel's LDS limit");
         attr[dev] = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<MT, BF>), dim3((unsigned)row_blocks, (unsigned)g.tok_blocks, (unsigned)g.splits), dim3(256), g.lds, s, a);
+    hipLaunchKernelGGL((gemm_kernel<MT, BF, XC>), dim3((unsigned)row_blocks, (unsigned)g.tok_blocks, (unsigned)g.splits), dim3(256), g.lds, s, a);
     return host::check_launch("qvb8_mma");
 }
 
@@ -1264,12 +1279,16 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         const int cols_per_split = g.stages_per_split * kGemmStageCols;
         const dim3 pgrid((unsigned)M, (unsigned)g.splits);
         const int tile_rows = staged ? 64 * g.MT : 0;                 // the staged kernel reads X stage by stage
-        if (mode == 0) hipLaunchKernelGGL((gemm_prep_kernel<false, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx, tile_rows);
-        else if (mode == 1) hipLaunchKernelGGL((gemm_prep_kernel<false, true>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx, tile_rows);
-        else hipLaunchKernelGGL((gemm_prep_kernel<true, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx, tile_rows);
-        if (int rc2 = host::check_launch("qvb8_mma activations")) return rc2;
+        // the activation pass (narrowed copy stored stage by stage, sums per column range) is for the staged kernel only: the
+        // register-decode kernel narrows what it stages and adds the rows of X up on the matrix cores itself
+        if (staged) {
+            if (mode == 0) hipLaunchKernelGGL((gemm_prep_kernel<false, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx, tile_rows);
+            else if (mode == 1) hipLaunchKernelGGL((gemm_prep_kernel<false, true>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx, tile_rows);
+            else hipLaunchKernelGGL((gemm_prep_kernel<true, false>), pgrid, dim3(256), 0, s, a.X, (int)M, (int)P, cols_per_split, x16, sx, tile_rows);
+            if (int rc2 = host::check_launch("qvb8_mma activations")) return rc2;
+        }
         GemmArgs ga;
-        ga.X = (mode == 1 || staged) ? x16 : a.X; ga.ids = ids; ga.fin = a.fin; ga.sx = sx; ga.out = out;
+        ga.X = staged ? x16 : a.X; ga.ids = ids; ga.fin = a.fin; ga.sx = staged ? sx : nullptr; ga.out = out;
         ga.M = (int)M; ga.Q = (int)Q; ga.P = (int)P; ga.stages_per_split = g.stages_per_split;
         ga.out_dt = g.splits > 1 ? 0 : out_dt;
         ga.planes = a.planes;
@@ -1283,8 +1302,8 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         if (staged) {
             if (g.MT == 4) rc = mode == 2 ? launch_gemm2<4, true>(ga, g, row_blocks, s) : launch_gemm2<4, false>(ga, g, row_blocks, s);
             else rc = mode == 2 ? launch_gemm2<2, true>(ga, g, row_blocks, s) : launch_gemm2<2, false>(ga, g, row_blocks, s);
-        } else if (g.MT == 4) rc = mode == 2 ? launch_gemm<4, true>(ga, g, row_blocks, s) : launch_gemm<4, false>(ga, g, row_blocks, s);
-        else rc = mode == 2 ? launch_gemm<2, true>(ga, g, row_blocks, s) : launch_gemm<2, false>(ga, g, row_blocks, s);
+        } else if (g.MT == 4) rc = mode == 2 ? launch_gemm<4, true, false>(ga, g, row_blocks, s) : mode == 1 ? launch_gemm<4, false, true>(ga, g, row_blocks, s) : launch_gemm<4, false, false>(ga, g, row_blocks, s);
+        else rc = mode == 2 ? launch_gemm<2, true, false>(ga, g, row_blocks, s) : mode == 1 ? launch_gemm<2, false, true>(ga, g, row_blocks, s) : launch_gemm<2, false, false>(ga, g, row_blocks, s);
         if (rc) return rc;
         if (g.splits > 1) {
             const int64_t n = M * Q;
