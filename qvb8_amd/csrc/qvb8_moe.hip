@@ -417,13 +417,28 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
         }
         q.ts = a.tau_s[mi]; q.mn = a.min_s[mi];
     };
+    // REG: a row's place is arithmetic, so a lane can ask for ANOTHER row's bytes: requests go out in the order lane = 4 * row
+    // + chunk (four neighbouring lanes read 16 nb consecutive bytes of one row: far fewer L1 accesses per request than a row
+    // per lane) and to_operand moves the registers into operand order (lane = row + 16 * chunk) across the wave.
+    const int pull = 4 * (4 * r + kg);
+    auto to_operand = [&](const uint4& v) -> uint4 {
+        if constexpr (!REG) return v;
+        return uint4{(uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y),
+                     (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w)};
+    };
     auto request_ids = [&](Round& q, uint4 (&lo)[T], uint4 (&hi)[T]) {
         q.ok = q.e_ok && q.nb >= 1 && q.nb <= 14 && q.bit0 >= 0 && ((q.bit0 + (int64_t)q.nb * a.P + 7) >> 3) + 8 <= a.ids_bytes;
         q.sliced = q.ok && q.nb >= 4 && q.nb <= 8 && (q.bit0 & 31) == 0;
-        const uint64_t row_off = (uint64_t)(q.bit0 >> 3) + (uint64_t)(step0 * 4 + kg) * (4u * (uint32_t)q.nb);
+        // the row and chunk this lane asks for: its own (row r, chunk kg), or in REG mode row lane / 4, chunk lane % 4 of the
+        // same tile (rows of a tile follow each other at P * nb bits; all 16 are usable or none is)
+        const int64_t ask_bit0 = REG ? q.bit0 + (int64_t)((lane >> 2) - r) * a.P * q.nb : q.bit0;
+        const int ask_chunk = REG ? (lane & 3) : kg;
+        const bool ask_sliced = !REG ? q.sliced : (q.e_ok && q.nb >= 4 && q.nb <= 8 && ask_bit0 >= 0 && (ask_bit0 & 31) == 0
+                                                   && ((ask_bit0 + (int64_t)q.nb * a.P + 7) >> 3) + 8 <= a.ids_bytes);
+        const uint64_t row_off = (uint64_t)(ask_bit0 >> 3) + (uint64_t)(step0 * 4 + ask_chunk) * (4u * (uint32_t)q.nb);
 #pragma unroll
         for (int it = 0; it < T; ++it) {
-            const bool use = q.sliced && (step0 + it) < n_steps;       // a wave without a tile reads tile 0's again: no address shared by the whole chip
+            const bool use = ask_sliced && (step0 + it) < n_steps;     // a wave without a tile reads tile 0's again: no address shared by the whole chip
             const uint64_t off = use ? row_off + (uint64_t)it * (16u * (uint32_t)q.nb) : 0;
             lo[it] = *reinterpret_cast<const uint4*>(a.ids + off);
             hi[it] = *reinterpret_cast<const uint4*>(a.ids + off + (use ? 4u * (uint32_t)(q.nb - 4) : 16u));
@@ -445,7 +460,7 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
 #pragma unroll
         for (int it = 0; it < T; ++it) {
             v4u_t b[4];
-            const uint4 lo = lo_[it], hi = hi_[it];
+            const uint4 lo = to_operand(lo_[it]), hi = to_operand(hi_[it]);
             if (uniform) {
                 switch (info0 & 0xFFu) {
                     case 7: decode_slice<7, false>(lo, hi, b); break;
@@ -691,9 +706,13 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
         auto issue = [&](int rnd, uint4 (&lo)[T], uint4 (&hi)[T]) __attribute__((always_inline)) -> WalkRow {
             const int i = min(g + min(rnd, n_rounds - 1) * G, n_rt - 1);
             const WalkRow rec = s_row[i * 16 + r];
-            const uint32_t nbr = (uint32_t)rec.flags & 255u;
-            const bool sliced = (rec.flags & 512) != 0;
-            const uint64_t row_off = (uint64_t)(rec.bit0 >> 3) + (uint64_t)(step0 * 4 + kg) * (4u * nbr);
+            // REG: the lane asks for chunk lane % 4 of row lane / 4 of the tile (neighbouring lanes, neighbouring bytes: far
+            // fewer L1 accesses per request than a row per lane); to_operand brings the registers into operand order
+            const WalkRow ask = REG ? s_row[i * 16 + (lane >> 2)] : rec;
+            const int ask_chunk = REG ? (lane & 3) : kg;
+            const uint32_t nbr = (uint32_t)ask.flags & 255u;
+            const bool sliced = (ask.flags & 512) != 0;
+            const uint64_t row_off = (uint64_t)(ask.bit0 >> 3) + (uint64_t)(step0 * 4 + ask_chunk) * (4u * nbr);
 #pragma unroll
             for (int it = 0; it < T; ++it) {
                 const bool use = sliced && (step0 + it) < n_steps;
@@ -702,6 +721,12 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
                 hi[it] = *reinterpret_cast<const uint4*>(a.ids + off + (use ? 4u * (nbr - 4u) : 16u));
             }
             return rec;
+        };
+        const int pull = 4 * (4 * r + kg);
+        auto to_operand = [&](const uint4& v) __attribute__((always_inline)) -> uint4 {
+            if constexpr (!REG) return v;
+            return uint4{(uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y),
+                         (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w)};
         };
         uint4 lo0[T], hi0[T], lo1[T], hi1[T];
         WalkRow rec0 = issue(0, lo0, hi0), rec1{0, 0, 0.f, 0.f, 0};     // by every wave: nothing under a branch
@@ -739,7 +764,7 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
 #pragma unroll
             for (int it = 0; it < T; ++it) {
                 v4u_t b[4];
-                const uint4 lo = lo_[it], hi = hi_[it];
+                const uint4 lo = to_operand(lo_[it]), hi = to_operand(hi_[it]);
                 if (uniform) {
                     switch (info0 & 0xFFu) {
                         case 7: decode_slice<7, false>(lo, hi, b); break;
