@@ -1130,7 +1130,9 @@ GemmPlan plan_gemm_for(int64_t M, int64_t Q, int64_t P) { return M >= gemm2_from
 
 // Fewest rows of X that go to the workgroup-tiled kernel when it can read the weight (49..: always; below that the tile
 // kernel is the alternative).
-int gemm_from() { const int v = host::env_int("QVB8_MMA_GEMM_FROM", 33); return v < 17 ? 17 : (v > 49 ? 49 : v); }
+// from 21 rows of X on the register-decode kernel is the faster one (measured on the 9B projections, 8 layers: M = 20 0.791 ms
+// against 0.799 for the tile kernel, M = 24 0.80 / 0.83, M = 32 0.83 / 0.87; M = 17 0.78 / 0.72)
+int gemm_from() { const int v = host::env_int("QVB8_MMA_GEMM_FROM", 21); return v < 17 ? 17 : (v > 49 ? 49 : v); }
 
 template <int MT, bool BF, bool XC>
 int launch_gemm(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_t s) {
@@ -1253,7 +1255,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     // mode 0: fp16 X, fp16 operands; 1: bf16 X narrowed to saturated fp16 on the way in, fp16 operands; 2: bf16 operands
     const int mode = x_dtype == QVB8_F16 ? 0 : (flags & QVB8_MMA_SATURATE_X) ? 1 : 2;
     int rc;
-    // Many rows of X: the workgroup-tiled kernel.  It addresses rows arithmetically and decodes whole slices only; from 33
+    // Many rows of X: the workgroup-tiled kernel.  It addresses rows arithmetically and decodes whole slices only; from 21
     // rows on it is also the faster one (the tile kernel then keeps too few bytes in flight), so it is taken whenever it
     // can read the weight and the caller brought its workspace.
     bool tiled = M > 48;
