@@ -160,8 +160,8 @@ typedef struct qvb8_mma_layout {
     int32_t nbits[QVB8_MMA_MAX_CLASSES];
 } qvb8_mma_layout;
 
-/* Workspace qvb8_mma needs: up to 20 rows of X only when it is called WITHOUT row records (it then builds them itself
- * first); from 21 rows on, when P % 256 == 0, what the workgroup-tiled kernels need (narrowed activations, their sums per
+/* Workspace qvb8_mma needs: up to 16 rows of X only when it is called WITHOUT row records (it then builds them itself
+ * first); from 17 rows on, when P % 256 == 0, what the workgroup-tiled kernels need (narrowed activations, their sums per
  * column range, partial results of the column ranges). */
 int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
 
@@ -177,8 +177,8 @@ int64_t qvb8_mma_workspace_bytes(int64_t M, int64_t Q, int64_t P);
  * by element.
  * 49 <= M <= 256 runs a workgroup-tiled decode + GEMM (X staged in LDS, v_mfma 32x32x16, column ranges added in a fixed
  * order): it needs `layout` with widths 4..8 (4..7 for bf16 operands), P % 256 == 0 and `workspace`; otherwise
- * QVB8_ERR_UNSUPPORTED / QVB8_ERR_WORKSPACE.  21 <= M <= 48 takes the same kernel when those conditions hold and the
- * workspace is there (it is the faster one from 21 rows on), else the 16-row tile kernel.  Above 48 rows the reference
+ * QVB8_ERR_UNSUPPORTED / QVB8_ERR_WORKSPACE.  17 <= M <= 48 takes the same kernel when those conditions hold and the
+ * workspace is there (it is the faster one from 17 rows on), else the 16-row tile kernel.  Above 48 rows the reference
  * restores the weight and calls a library GEMM (formats/qvb8/module.py:402-457).
  * Replaces: ext.mma_multi  qvb8_mma_multi_forward qvb8_cuda.cu:2566-2671 (kernels :2321-2441, escape fix
  * :2503-2548), and, through the Python module, the M <= 8 GEMV of :1059-1166 when P % 128 == 0. */

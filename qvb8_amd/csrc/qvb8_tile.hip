@@ -1075,6 +1075,7 @@ GemmPlan plan_gemm(int64_t M, int64_t Q, int64_t P) {
     const int mt_env = host::env_int("QVB8_GEMM_MT", 0);
     g.MT = mt_env == 2 || mt_env == 4 ? mt_env : (M > 192 ? 4 : 2);
     if (M <= 64) g.MT = 2;
+    if (M <= 32 && host::env_int("QVB8_GEMM_MT1", 1) != 0) g.MT = 1;      // one token tile of 32: half the matrix instructions per step
     const int TMK = 32 * g.MT;
     g.tok_blocks = (int)((M + TMK - 1) / TMK);
     g.row_blocks = (int)((Q + kGemmRows - 1) / kGemmRows);
@@ -1130,9 +1131,9 @@ GemmPlan plan_gemm_for(int64_t M, int64_t Q, int64_t P) { return M >= gemm2_from
 
 // Fewest rows of X that go to the workgroup-tiled kernel when it can read the weight (49..: always; below that the tile
 // kernel is the alternative).
-// from 21 rows of X on the register-decode kernel is the faster one (measured on the 9B projections, 8 layers: M = 20 0.791 ms
-// against 0.799 for the tile kernel, M = 24 0.80 / 0.83, M = 32 0.83 / 0.87; M = 17 0.78 / 0.72)
-int gemm_from() { const int v = host::env_int("QVB8_MMA_GEMM_FROM", 21); return v < 17 ? 17 : (v > 49 ? 49 : v); }
+// from 17 rows of X on the register-decode kernel (one token tile of 32 up to 32 rows) is the faster one (measured on the 9B
+// projections, 8 layers: M = 17 0.641 ms against 0.721 for the tile kernel with two token tiles, M = 32 0.70 / 0.87)
+int gemm_from() { const int v = host::env_int("QVB8_MMA_GEMM_FROM", 17); return v < 17 ? 17 : (v > 49 ? 49 : v); }
 
 template <int MT, bool BF, bool XC>
 int launch_gemm(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_t s) {
@@ -1255,7 +1256,7 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     // mode 0: fp16 X, fp16 operands; 1: bf16 X narrowed to saturated fp16 on the way in, fp16 operands; 2: bf16 operands
     const int mode = x_dtype == QVB8_F16 ? 0 : (flags & QVB8_MMA_SATURATE_X) ? 1 : 2;
     int rc;
-    // Many rows of X: the workgroup-tiled kernel.  It addresses rows arithmetically and decodes whole slices only; from 21
+    // Many rows of X: the workgroup-tiled kernel.  It addresses rows arithmetically and decodes whole slices only; from 17
     // rows on it is also the faster one (the tile kernel then keeps too few bytes in flight), so it is taken whenever it
     // can read the weight and the caller brought its workspace.
     bool tiled = M > 48;
@@ -1304,7 +1305,8 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
         if (staged) {
             if (g.MT == 4) rc = mode == 2 ? launch_gemm2<4, true>(ga, g, row_blocks, s) : launch_gemm2<4, false>(ga, g, row_blocks, s);
             else rc = mode == 2 ? launch_gemm2<2, true>(ga, g, row_blocks, s) : launch_gemm2<2, false>(ga, g, row_blocks, s);
-        } else if (g.MT == 4) rc = mode == 2 ? launch_gemm<4, true, false>(ga, g, row_blocks, s) : mode == 1 ? launch_gemm<4, false, true>(ga, g, row_blocks, s) : launch_gemm<4, false, false>(ga, g, row_blocks, s);
+        } else if (g.MT == 1) rc = mode == 2 ? launch_gemm<1, true, false>(ga, g, row_blocks, s) : mode == 1 ? launch_gemm<1, false, true>(ga, g, row_blocks, s) : launch_gemm<1, false, false>(ga, g, row_blocks, s);
+        else if (g.MT == 4) rc = mode == 2 ? launch_gemm<4, true, false>(ga, g, row_blocks, s) : mode == 1 ? launch_gemm<4, false, true>(ga, g, row_blocks, s) : launch_gemm<4, false, false>(ga, g, row_blocks, s);
         else rc = mode == 2 ? launch_gemm<2, true, false>(ga, g, row_blocks, s) : mode == 1 ? launch_gemm<2, false, true>(ga, g, row_blocks, s) : launch_gemm<2, false, false>(ga, g, row_blocks, s);
         if (rc) return rc;
         if (g.splits > 1) {
