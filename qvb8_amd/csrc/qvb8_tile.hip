@@ -1077,7 +1077,7 @@ GemmPlan plan_gemm(int64_t M, int64_t Q, int64_t P) {
     const int mt_env = host::env_int("QVB8_GEMM_MT", 0);
     g.MT = mt_env == 2 || mt_env == 4 ? mt_env : (M > 192 ? 4 : 2);
     if (M <= 64) g.MT = 2;
-    if (M <= 32 && host::env_int("QVB8_GEMM_MT1", 1) != 0) g.MT = 1;      // one token tile of 32: half the matrix instructions per step
+    if (M <= host::env_int("QVB8_GEMM_MT1_UPTO", 32)) g.MT = 1;           // one token tile of 32: half the matrix instructions per step
     const int TMK = 32 * g.MT;
     g.tok_blocks = (int)((M + TMK - 1) / TMK);
     g.row_blocks = (int)((Q + kGemmRows - 1) / kGemmRows);
