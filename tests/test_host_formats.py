@@ -226,3 +226,45 @@ def test_rows_widened_to_whole_tiles_on_the_host():
         runs = sorted(zip(*[t.tolist() for t in torch.unique(nb2, return_counts=True)]))
         for (w, n), (w_next, _) in zip(runs[:-1], runs[1:]):
             assert n % 16 == 0 or w_next > 8, runs
+
+
+def test_tile_uniform_widths_and_repack_rows_on_the_host():
+    """tile_uniform_widths gives every whole 16-row tile whose widths lie in 4..8 its largest width and leaves other rows
+    alone; repack_rows stores the rows again in those widths, in row order from byte 0, every id unchanged (read back field
+    by field); a regular stack is recognised, an irregular one is not."""
+    import torch
+    from qvb8_amd import ext_qvb8 as ext
+    from tests import helpers as H
+    for Q, P, widths in ((96, 128, [5, 6, 6, 6, 7]), (40, 64, [5, 6, 7, 8]), (64, 128, [7]), (50, 96, [6, 9, 3]), (37, 40, [4, 5])):
+        d = H.mixed_width_pack(Q, P, widths, seed=Q)
+        ids, _, nbits, bit_off = H.to_device_args(d, "cpu")[:4]
+        target = ext.tile_uniform_widths(nbits)
+        nb = nbits.to(torch.int64)
+        whole = Q // 16 * 16
+        tiles = nb[:whole].view(-1, 16)
+        sliced = (tiles.amin(1) >= 4) & (tiles.amax(1) <= 8)
+        want = torch.where(sliced[:, None], tiles.amax(1, keepdim=True).expand_as(tiles), tiles).reshape(-1)
+        if target is None:
+            assert torch.equal(want, nb[:whole])
+            target = nbits
+        else:
+            assert torch.equal(target[:whole].to(torch.int64), want) and torch.equal(target[whole:], nbits[whole:])
+        ids2, off2 = ext.repack_rows(ids, nbits, bit_off, P, target)
+        row_bits = target.to(torch.int64) * P
+        assert torch.equal(off2, torch.cumsum(row_bits, 0) - row_bits) and ids2.numel() == int(row_bits.sum()) // 8 + 8
+        buf = ids2.numpy()
+        for q in range(Q):
+            w = int(target[q])
+            for c in (0, 1, P // 2, P - 1):
+                pos = int(off2[q]) + c * w
+                v = int.from_bytes(buf[pos >> 3:(pos >> 3) + 4].tobytes(), "little")
+                assert (v >> (pos & 7)) & ((1 << w) - 1) == d["ids_dense"][q, c]
+    with pytest.raises(RuntimeError):
+        ext.repack_rows(ids, nbits, bit_off, P, torch.full_like(nbits, 3))
+    # two experts of 32 rows x 64 columns in 6 bits, back to back at a stride of 1600 bytes
+    nb = torch.full((2, 32), 6, dtype=torch.uint8)
+    off = (torch.arange(2).view(2, 1) * 1600 * 8 + torch.arange(32).view(1, 32) * 64 * 6).to(torch.int64)
+    assert ext.stack_is_regular(nb, off, 64)
+    off2 = off.clone(); off2[1, 5] += 8
+    nb2 = nb.clone(); nb2[0, 3] = 5
+    assert not ext.stack_is_regular(nb, off2, 64) and not ext.stack_is_regular(nb2, off, 64)
