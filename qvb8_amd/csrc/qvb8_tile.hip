@@ -1017,7 +1017,9 @@ bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl) {
         int64_t even = (tiles + blocks - 1) / blocks;
         even = (even + pl.G - 1) / pl.G * pl.G;
         if (even < tw) tw = even;
-        blocks = (tiles + tw - 1) / tw;
+        // the rounded number of workgroups is kept (tile t goes to workgroup t % blocks, so each gets tiles / blocks of them,
+        // give or take one): ceil(tiles / tw) workgroups would again leave CUs idle in the last round
+        if ((tiles + blocks - 1) / blocks > tw) blocks = (tiles + tw - 1) / tw;
     }
     pl.TW = (int)tw;
     pl.blocks = (unsigned)blocks;
