@@ -220,3 +220,43 @@ def test_plane_tiles_change_no_result_and_survive_moves_subsets_and_fusion(monke
     monkeypatch.setenv("QVB8_PLANES", "0")
     off = QVBandLinearV8.from_encoded(enc)
     assert torch.equal(want[40], off(xs[40])) and not off._planes
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_plane_tiles_seeded_shapes(seed):
+    """Seeded random shapes and width mixes (rows that are no multiple of 16, runs shorter than a tile, widths the slicing
+    cannot read, escapes): the operator with whole tiles in planes gives, bit for bit, what it gives with the rows back to
+    back, and both agree with the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    Q = int(rng.integers(17, 400))
+    P = int(rng.choice([128, 256, 384, 512, 1024]))
+    pool = [list(range(4, 9)), [6, 7], [7], [5, 6, 7, 8], [4, 8], [6, 9, 7], [3, 6, 7]][int(rng.integers(0, 7))]
+    n_kinds = int(rng.integers(1, len(pool) + 1))
+    widths = [int(w) for w in rng.choice(pool, size=n_kinds, replace=False)]
+    reps = [int(rng.integers(1, 40)) for _ in widths]
+    pattern = [w for w, n in zip(widths, reps) for _ in range(n)]
+    d = H.mixed_width_pack(Q, P, pattern, seed=seed)
+    d["tau_s"] = d["tau_s"] * (1.0 / 64)
+    n_esc = int(rng.integers(0, 6))
+    if n_esc:
+        d["esc_idx"] = np.sort(rng.choice(Q * P, n_esc, replace=False)).astype(np.int64)
+        d["esc_vals"] = rng.normal(size=n_esc).astype(np.float32)
+    a = H.to_device_args(d, DEV)
+
+    def make(planes):
+        m = QVBandLinearV8(min_s=a[1].clone(), nbits=a[2].clone(), bit_off=a[3].clone(), ids=a[0].clone(), Q=Q, P=P, tau_s=a[5].clone(),
+                           esc_idx=a[6], esc_vals=a[7])
+        m.plane_tiles = planes
+        return m
+    flat, tiled = make(False), make(True)
+    Wr = O.reconstruct(d["min_s"], d["tau_s"], d["ids_dense"], d["esc_idx"], d["esc_vals"])
+    for M in (1, 13, 40, 70):
+        x = torch.randn(M, P, generator=torch.Generator().manual_seed(seed * 100 + M)).to(torch.bfloat16).to(DEV)
+        y0, y1 = flat(x), tiled(x)
+        assert torch.equal(y0, y1), (Q, P, pattern[:8], M)
+        xs = O.sat_half(x.float().cpu().numpy())
+        _close(y1, O.linear_f64(xs, Wr), Wr, xs, torch.bfloat16)
+    assert not flat._planes
+    from qvb8_amd import ext_qvb8 as ext
+    dense = ext.decode_f32(tiled.ids, tiled.min_s, tiled.nbits, tiled.bit_off, P, tiled.tau_s, tiled.esc_idx, tiled.esc_vals)
+    assert np.array_equal(dense.cpu().numpy().view(np.uint32), Wr.astype(np.float32).view(np.uint32))
