@@ -41,6 +41,7 @@ def _operands(stk, x, idx, w, act, out):
 def _both(lib, stk, T, k, seed, act=0, dtype=torch.bfloat16):
     g, d = stk
     E = g["min_s"].shape[0]
+    act |= (0x100 if g["regular"] else 0) | (0x200 if d["regular"] else 0)      # what the operator states about its stacks
     rng = np.random.default_rng(seed)
     idx_h, w_h = O.router_topk(rng.normal(size=(T, E)), k)
     idx, w = torch.from_numpy(idx_h).to(DEV), torch.from_numpy(w_h).to(DEV)
