@@ -274,6 +274,10 @@ def test_rows_stored_in_planes_change_no_result(Q, P, widths):
     assert torch.equal(back_ids, ids_n) and torch.equal(back_off, off_n)
     for fn in (ext.decode_f32, ext.decode, ext.decode_bf16):
         assert torch.equal(fn(ids_n, min_s, nbits, off_n, P, tau_s, ei, ev), fn(ids_p, min_s, nbits, off_p, P, tau_s, ei, ev))
+    rows = torch.tensor([0, Q - 1, Q // 2, 17, 16, 0], device=DEV)               # the row lookup (embedding read) as well
+    for dt in (torch.float32, torch.bfloat16):
+        assert torch.equal(ext.lookup_rows(rows, ids_n, min_s, nbits, off_n, P, tau_s, ei, ev, dt),
+                           ext.lookup_rows(rows, ids_p, min_s, nbits, off_p, P, tau_s, ei, ev, dt))
     x8 = _x(8, P, torch.float16, 1)
     _check(d, None, x8, ext.gemv_multi(x8, *args_p), saturate_ref=False)      # rows in planes are read element by element there
     sliceable = all(4 <= w <= 8 for w in widths) and P % 256 == 0
