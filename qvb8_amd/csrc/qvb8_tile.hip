@@ -551,12 +551,14 @@ __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t* __restri
 
 // The workgroup's rows are positions [pos0, pos0 + 256) of a run of width NB that ends at pos_end and starts at byte
 // run_byte0 (position run_first) of the ids buffer.
-template <int MT, bool BF, bool XC, int NB>
+template <int MT, bool BF, bool XC, int NB, int RT>
 __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_end, int run_first, uint64_t run_byte0, unsigned char* smem) {
     using F = Fmt<BF>;
     using XI = XIn<BF, XC>;
     constexpr int TMK = 32 * MT;                   // rows of X per workgroup
-    constexpr int XL = TMK * 16 / 256;             // 16-byte pieces of a stage per thread
+    constexpr int THREADS = 64 * (kGemmRows / (32 * RT));          // RT row tiles of 32 per wave: 4 waves (RT = 2) or 8 (RT = 1)
+    constexpr int XROWS = THREADS / 16;            // rows of X staged per pass of the workgroup
+    constexpr int XL = (TMK * 16 + THREADS - 1) / THREADS;          // 16-byte pieces of a stage per thread
     unsigned char* xs = smem;                                              // [2][TMK][kGemmXStride]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 31, kh = lane >> 5;
@@ -566,17 +568,17 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
     const int u_begin = 2 * s_begin, u_end = 2 * s_end;                    // 64-column steps; u_end - u_begin is a multiple of 4
     if (u_begin >= u_end) return;
 
-    // ---- this lane's two rows; a position past the run reads the run's last row (finite operands, result not stored) ----
-    const uint8_t* row_ptr[2]; const uint8_t* row_hi[2]; int row_pos[2]; bool row_ok[2], row_pl[2];
+    // ---- this lane's RT rows; a position past the run reads the run's last row (finite operands, result not stored) ----
+    const uint8_t* row_ptr[RT]; const uint8_t* row_hi[RT]; int row_pos[RT]; bool row_ok[RT], row_pl[RT];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        const int pos = pos0 + wave * kGemmWaveRows + rt * 32 + n;
+    for (int rt = 0; rt < RT; ++rt) {
+        const int pos = pos0 + wave * (32 * RT) + rt * 32 + n;
         row_ok[rt] = pos < pos_end;
         row_pos[rt] = row_ok[rt] ? pos : pos_end - 1;
         // requests go out in the order lane = 2 * row + half, so that neighbouring lanes read neighbouring bytes
         // (fewer L1 accesses per request); to_operand moves the registers into operand order (lane = row + 32 * half).
         // (With rows stored in planes, requests in operand order -- contiguous, no move afterwards -- were measured: no gain.)
-        const int rpos = min(pos0 + wave * kGemmWaveRows + rt * 32 + (lane >> 1), pos_end - 1);
+        const int rpos = min(pos0 + wave * (32 * RT) + rt * 32 + (lane >> 1), pos_end - 1);
         const uint32_t rhalf = (uint32_t)(lane & 1);
         const uint64_t row_bytes = (uint64_t)a.P * NB / 8;
         // a row of a whole tile inside the run may be stored in planes: first / last four dwords of its slice then come
@@ -598,31 +600,27 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
         return uint4{(uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.x), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.y),
                      (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.z), (uint32_t)__builtin_amdgcn_ds_bpermute(pull, (int)v.w)};
     };
-    uint4 raw[4][2][2];                            // [step % 4][row tile][first / last four dwords]
-    const uint8_t* const rp0 = row_ptr[0];
-    const uint8_t* const rp1 = row_ptr[1];
-    const uint8_t* const rh0 = row_hi[0];
-    const uint8_t* const rh1 = row_hi[1];
-    const bool pl0 = row_pl[0], pl1 = row_pl[1];
-    auto request_ids = [u_end, rp0, rp1, rh0, rh1, pl0, pl1](int u, uint4 (&w)[2][2]) {
+    uint4 raw[4][RT][2];                            // [step % 4][row tile][first / last four dwords]
+    auto request_ids = [&](int u, uint4 (&w)[RT][2]) {
         const uint32_t uc = (uint32_t)min(u, u_end - 1);
         const uint32_t off = uc * (8u * NB);                               // a step is 64 columns = 8 NB bytes of a row
         const uint32_t pa = (uc >> 1) * (256u * NB) + (uc & 1u) * 512u;    // in planes: step u / 2, column groups 2 (u % 2) + half
         const uint32_t pb = (uc >> 1) * (256u * NB) + (uc & 1u) * (128u * (NB - 4u));
-        w[0][0] = *reinterpret_cast<const uint4*>(rp0 + (pl0 ? pa : off));
-        w[0][1] = *reinterpret_cast<const uint4*>(rh0 + (pl0 ? pb : off));
-        w[1][0] = *reinterpret_cast<const uint4*>(rp1 + (pl1 ? pa : off));
-        w[1][1] = *reinterpret_cast<const uint4*>(rh1 + (pl1 ? pb : off));
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            w[rt][0] = *reinterpret_cast<const uint4*>(row_ptr[rt] + (row_pl[rt] ? pa : off));
+            w[rt][1] = *reinterpret_cast<const uint4*>(row_hi[rt] + (row_pl[rt] ? pb : off));
+        }
     };
     // ---- X: thread tid stages piece tid % 16 (8 columns) of rows tid / 16 + 16 * i; rows past M read row M - 1 (not stored at the end) ----
-    const int xch = tid & 15, xrow = tid >> 4;
+    const int xch = tid & 15, xrow = tid >> 4;                  // with 512 threads a stage of 32 rows of X is one piece for every thread
     const uint16_t* const x_base = a.X + 8 * xch;
     const int M = a.M, P = a.P;
     v4u_t xg[XL];
     auto request_x = [=](int st, v4u_t (&g)[XL]) {
         const uint32_t c = (uint32_t)min(st, s_end - 1) * kGemmStageCols;
 #pragma unroll
-        for (int i = 0; i < XL; ++i) g[i] = *reinterpret_cast<const v4u_t*>(x_base + (size_t)min(tok0 + xrow + 16 * i, M - 1) * P + c);
+        for (int i = 0; i < XL; ++i) g[i] = *reinterpret_cast<const v4u_t*>(x_base + (size_t)min(tok0 + xrow + XROWS * i, M - 1) * P + c);
     };
     // XC: bf16 activations are narrowed like saturating_half on their way into LDS (every workgroup narrows the 16 KB it
     // stages; a pass of its own over X would be one more launch per product)
@@ -634,11 +632,11 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
 #pragma unroll
                 for (int k = 0; k < 4; ++k) v[k] = XI::pair(v[k]);
             }
-            *reinterpret_cast<v4u_t*>(xs + ((size_t)buf * TMK + xrow + 16 * i) * kGemmXStride + 16 * xch) = v;
+            *reinterpret_cast<v4u_t*>(xs + ((size_t)buf * TMK + xrow + XROWS * i) * kGemmXStride + 16 * xch) = v;
         }
     };
 
-    v16f_t acc[2][MT];
+    v16f_t acc[RT][MT];
     // sums of the rows of X over this workgroup's columns, as the operands see them: the product with a matrix of ones,
     // in the accumulator layout (register i of every lane <-> the token that acc[.][mt][i] belongs to).  (Added up on the
     // vector ALU while X is staged instead -- a third fewer matrix instructions -- was measured slower: M = 64 0.995 against
@@ -650,7 +648,7 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
 #pragma unroll
         for (int i = 0; i < 16; ++i) sxa[mt][i] = 0.f;
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -666,9 +664,9 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
         for (int k = 0; k < 4; ++k) {
             const int h = k & 1, buf = k >> 1;
             if (h == 0) request_x((u0 >> 1) + buf + 1, xg);
-            v4u_t b[2][4];
+            v4u_t b[RT][4];
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) decode_slice<NB, BF>(to_operand(raw[k][rt][0]), to_operand(raw[k][rt][1]), b[rt]);
+            for (int rt = 0; rt < RT; ++rt) decode_slice<NB, BF>(to_operand(raw[k][rt][0]), to_operand(raw[k][rt][1]), b[rt]);
             request_ids(u0 + k + 4, raw[k]);
             __builtin_amdgcn_sched_barrier(0);                             // the requests stay ahead of the products
             const unsigned char* xb = xs + (size_t)buf * TMK * kGemmXStride + (size_t)n * kGemmXStride + 2 * (64 * h + 32 * kh);
@@ -679,8 +677,9 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
                     const uint4 v = *reinterpret_cast<const uint4*>(xb + (size_t)(32 * mt) * kGemmXStride + 16 * j);
                     const v4u_t av = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                    for (int rt = 0; rt < 2; ++rt) acc[rt][mt] = F::mfma32(av, b[rt][j], acc[rt][mt]);
-                    sxa[mt] = F::mfma32(av, ones, sxa[mt]);
+                    for (int rt = 0; rt < RT; ++rt) acc[rt][mt] = F::mfma32(av, b[rt][j], acc[rt][mt]);
+                    // eight waves: the sums are shared work -- wave w < 4 adds up the columns of operand j = w, joined at the end
+                    if (RT == 2 || j == wave) sxa[mt] = F::mfma32(av, ones, sxa[mt]);
                 }
             if (h == 1) {
                 store_x(buf ^ 1, xg);
@@ -689,9 +688,19 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
         }
     }
     // ---- the end: lane holds, for row n of each row tile, tokens 32 mt + 8 (i / 4) + 4 kh + i % 4 ----
+    float* sxs = reinterpret_cast<float*>(smem);                           // [4][TMK]; the X stages are no longer read (barrier above)
+    if constexpr (RT == 1) {
+        if (wave < 4 && n == 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) sxs[wave * TMK + 32 * mt + 8 * (i >> 2) + 4 * kh + (i & 3)] = sxa[mt][i];
+        }
+        __syncthreads();
+    }
     float* out = a.out + (size_t)blockIdx.z * (size_t)a.M * (size_t)a.Q;
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
+    for (int rt = 0; rt < RT; ++rt) {
         if (!row_ok[rt]) continue;
         const uint4 f = a.fin[row_pos[rt]];
         if (f.z >= (uint32_t)a.Q) continue;
@@ -703,7 +712,7 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
                 const int tl = 32 * mt + 8 * (i >> 2) + 4 * kh + (i & 3);
                 const int t = tok0 + tl;
                 if (t < a.M) {
-                    const float sx = sxa[mt][i];
+                    const float sx = RT == 1 ? ((sxs[tl] + sxs[TMK + tl]) + sxs[2 * TMK + tl]) + sxs[3 * TMK + tl] : sxa[mt][i];
                     const float d = __builtin_fmaf(-F::bias, sx, acc[rt][mt][i]);
                     store_y(out, a.out_dt, (int64_t)t * a.Q + f.z, (float)(ts * (double)d + mn * (double)sx));
                 }
@@ -711,8 +720,8 @@ __device__ __forceinline__ void gemm_run(const GemmArgs& a, int pos0, int pos_en
     }
 }
 
-template <int MT, bool BF, bool XC>
-__global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
+template <int MT, bool BF, bool XC, int RT>
+__global__ void __launch_bounds__(64 * (kGemmRows / (32 * RT))) gemm_kernel(GemmArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     // which run of equal widths this workgroup's 256 positions belong to
     const int bx = (int)blockIdx.x;
@@ -725,11 +734,11 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     const int pos0 = run_first + (bx - (c == 0 ? 0 : c == 1 ? a.blocks1 : a.blocks2)) * kGemmRows;
     if (pos0 >= run_end) return;
     switch (c == 0 ? nb0 : c == 1 ? nb1 : nb2) {
-        case 4: gemm_run<MT, BF, XC, 4>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 5: gemm_run<MT, BF, XC, 5>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 6: gemm_run<MT, BF, XC, 6>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 7: gemm_run<MT, BF, XC, 7>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 8: if constexpr (!BF) gemm_run<MT, BF, XC, 8>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 4: gemm_run<MT, BF, XC, 4, RT>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 5: gemm_run<MT, BF, XC, 5, RT>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 6: gemm_run<MT, BF, XC, 6, RT>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 7: gemm_run<MT, BF, XC, 7, RT>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 8: if constexpr (!BF) gemm_run<MT, BF, XC, 8, RT>(a, pos0, run_end, run_first, byte0, smem); break;
         default: break;
     }
 }
@@ -1139,18 +1148,25 @@ GemmPlan plan_gemm_for(int64_t M, int64_t Q, int64_t P) { return M >= gemm2_from
 // projections, 8 layers: M = 17 0.641 ms against 0.721 for the tile kernel with two token tiles, M = 32 0.70 / 0.87)
 int gemm_from() { const int v = host::env_int("QVB8_MMA_GEMM_FROM", 17); return v < 17 ? 17 : (v > 49 ? 49 : v); }
 
-template <int MT, bool BF, bool XC>
-int launch_gemm(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_t s) {
+template <int MT, bool BF, bool XC, int RT>
+int launch_gemm_as(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_t s) {
     static bool attr[64] = {false};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: no current device");
     if (!attr[dev]) {
-        if (hipFuncSetAttribute((const void*)gemm_kernel<MT, BF, XC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds) != hipSuccess)
+        if (hipFuncSetAttribute((const void*)gemm_kernel<MT, BF, XC, RT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds) != hipSuccess)
             return host::fail(QVB8_ERR_LAUNCH, "qvb8_mma: cannot raise the kernel's LDS limit");
         attr[dev] = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<MT, BF, XC>), dim3((unsigned)row_blocks, (unsigned)g.tok_blocks, (unsigned)g.splits), dim3(256), g.lds, s, a);
+    hipLaunchKernelGGL((gemm_kernel<MT, BF, XC, RT>), dim3((unsigned)row_blocks, (unsigned)g.tok_blocks, (unsigned)g.splits),
+                       dim3(64 * (kGemmRows / (32 * RT))), g.lds, s, a);
     return host::check_launch("qvb8_mma");
+}
+// eight waves with one row tile each (two waves per SIMD: one decodes while the other's products run) or four with two
+template <int MT, bool BF, bool XC>
+int launch_gemm(const GemmArgs& a, const GemmPlan& g, int row_blocks, hipStream_t s) {
+    if (host::env_int("QVB8_GEMM_WAVES", 8) == 8 && MT <= 2) return launch_gemm_as<MT, BF, XC, 1>(a, g, row_blocks, s);
+    return launch_gemm_as<MT, BF, XC, 2>(a, g, row_blocks, s);
 }
 
 template <int WM, bool BF>
