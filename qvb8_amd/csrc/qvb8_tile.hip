@@ -106,8 +106,12 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
 // slots.  After one barrier the whole workgroup combines the column ranges of each row in a fixed order.
 // The kernel's arguments are 56 bytes of scalars (measured: every further 64 bytes of kernel arguments cost about a
 // microsecond per launch): fin follows loc, n_steps follows P, the small counts share one word.
+// Waves a workgroup of this variant may have: twelve (three per SIMD) where the registers allow it -- long rows then take
+// fewer panels (12288 columns: two instead of three) --, else eight.
+template <int NT, int T, bool BF, bool PL> constexpr int tile_max_waves() { return (NT == 1 && T == 4 && PL && !BF) ? 12 : 8; }
+
 template <int NT, int T, bool BF, bool XC, int XP = 0, bool PL = false>
-__global__ void __launch_bounds__(512) tile_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ ids,
+__global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_kernel(const uint16_t* __restrict__ X, const uint8_t* __restrict__ ids,
                                                    const uint64_t* __restrict__ loc, float* __restrict__ Y, int64_t ids_bytes,
                                                    int Q, int P, uint32_t counts, int TW, int first1, int first2, uint32_t widths) {
     static_assert(!(BF && XC), "narrowing on the way in exists for fp16 operands only");
@@ -993,10 +997,11 @@ constexpr size_t kTileLdsLimit = 128 * 1024;
 constexpr size_t kTileXLdsLimit = 64 * 1024;     // X through LDS: up to this many bytes of activations on top
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;
 
-bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl) {
+bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int wave_cap = 8) {
     const int n_steps = (int)(P / kStepCols);
     const int ranges = (n_steps + T - 1) / T;                 // column ranges of T steps
-    const int max_waves = 8;
+    // more than eight waves only where that saves a panel
+    const int max_waves = (wave_cap > 8 && (ranges + wave_cap - 1) / wave_cap < (ranges + 7) / 8) ? wave_cap : 8;
     pl.panels = (ranges + max_waves - 1) / max_waves;
     pl.W = (ranges + pl.panels - 1) / pl.panels;
     pl.G = pl.panels == 1 ? max_waves / pl.W : 1;
@@ -1038,7 +1043,8 @@ bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl) {
 template <int NT, int T, bool BF, bool XC, int XP = 0, bool PL = false>
 int launch_tile(TileArgs& a, hipStream_t s) {
     TilePlan pl;
-    if (!plan_tile(NT, T, a.M, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
+    if (!plan_tile(NT, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<NT, T, BF, PL>() : 8))
+        return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
     if constexpr (XP > 0) pl.lds += (size_t)a.M * (size_t)a.P * 2;
     a.W = pl.W; a.G = pl.G; a.panels = pl.panels; a.TW = pl.TW;
     static bool attr[64] = {false};                           // per device: the attribute belongs to the device's copy of the kernel
@@ -1062,7 +1068,8 @@ int launch_tile(TileArgs& a, hipStream_t s) {
 template <int T, bool BF, bool XC, bool PL = false>
 int launch_tile_rows16(TileArgs& a, hipStream_t s) {
     TilePlan pl;
-    if (!plan_tile(1, T, a.M, a.Q, a.P, pl)) return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
+    if (!plan_tile(1, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<1, T, BF, PL>() : 8))
+        return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
     const size_t x_bytes = (size_t)a.M * (size_t)a.P * 2;
     const size_t per_thread = (x_bytes / 16 + pl.threads - 1) / pl.threads;
     const bool fits = x_bytes <= kTileXLdsLimit && pl.lds + x_bytes <= kLdsPerWorkgroup && host::env_int("QVB8_TILE_X_LDS", 1) != 0;
@@ -1342,7 +1349,9 @@ extern "C" int qvb8_mma(const void* X, int x_dtype, int64_t M,
     const int n_steps_all = (int)(P / kStepCols);
 #define QVB8_TILE_LAUNCH_ROWS16_P(T_, PL_) (mode == 0 ? launch_tile_rows16<T_, false, false, PL_>(a, s) : mode == 1 ? launch_tile_rows16<T_, false, true, PL_>(a, s) : launch_tile_rows16<T_, true, false, PL_>(a, s))
 #define QVB8_TILE_LAUNCH_ROWS16(T_) (a.planes ? QVB8_TILE_LAUNCH_ROWS16_P(T_, true) : QVB8_TILE_LAUNCH_ROWS16_P(T_, false))
-        if (M <= 16) rc = n_steps_all > 32 && n_steps_all <= 40 ? QVB8_TILE_LAUNCH_ROWS16(5) : QVB8_TILE_LAUNCH_ROWS16(4);
+        // (with twelve waves four steps each cover up to 48 steps in one panel: QVB8_TILE_T5=0 tries that instead)
+        const bool five = n_steps_all > 32 && n_steps_all <= 40 && !(a.planes && mode != 2 && host::env_int("QVB8_TILE_T5", 1) == 0);
+        if (M <= 16) rc = five ? QVB8_TILE_LAUNCH_ROWS16(5) : QVB8_TILE_LAUNCH_ROWS16(4);
 #undef QVB8_TILE_LAUNCH_ROWS16
 #undef QVB8_TILE_LAUNCH_ROWS16_P
     else if (M <= 32) rc = QVB8_TILE_LAUNCH(2, 2);
