@@ -55,6 +55,19 @@ def apply_keeping_fp32_metadata(module: nn.Module, fn, recurse=True):
     return result
 
 
+def _ascending(positions, values):
+    """An escape list in ascending flat positions (the correction kernels add a row's escapes in list order, so a sorted
+    list makes results reproducible); returned as it is when it already is."""
+    if positions.numel() < 2 or bool((positions[1:] >= positions[:-1]).all()):
+        return positions, values
+    order = torch.argsort(positions, stable=True)
+    return positions[order].contiguous(), values[order].contiguous()
+
+
+def _on(dev, array, dtype):
+    return torch.from_numpy(np.ascontiguousarray(array, dtype)).to(dev)
+
+
 class QVBandLinearV8(nn.Module):
     # The first call of the matrix-core path copies the rows once into width-sorted order (same total size; `ids` and
     # `bit_off` are replaced, every kernel keeps working through bit_off), so that calls compute row addresses instead of
@@ -72,30 +85,15 @@ class QVBandLinearV8(nn.Module):
     def __init__(self, *, min_s, nbits, bit_off, ids, Q, P, tau_s, esc_idx, esc_vals, bias=None,
                  esc_idx_bf16=None, esc_vals_bf16=None):
         super().__init__()
-        self.in_features = int(P)
-        self.out_features = int(Q)
-        self.register_buffer("tau_s", tau_s, persistent=False)
-        self.register_buffer("min_s", min_s, persistent=False)
-        self.register_buffer("nbits", nbits, persistent=False)
-        self.register_buffer("bit_off", bit_off, persistent=False)
-        self.register_buffer("ids", ids, persistent=False)
-
-        def _sorted(ei, ev):
-            # the correction kernels add a row's escapes in list order: ascending positions make results reproducible
-            if ei.numel() > 1 and not bool((ei[1:] >= ei[:-1]).all()):
-                o = torch.argsort(ei, stable=True)
-                ei, ev = ei[o].contiguous(), ev[o].contiguous()
-            return ei, ev
-        esc_idx, esc_vals = _sorted(esc_idx, esc_vals)
-        if esc_idx_bf16 is None:
-            esc_idx_bf16, esc_vals_bf16 = esc_idx, esc_vals
-        else:
-            esc_idx_bf16, esc_vals_bf16 = _sorted(esc_idx_bf16, esc_vals_bf16)
-        self.register_buffer("esc_idx", esc_idx, persistent=False)
-        self.register_buffer("esc_vals", esc_vals, persistent=False)
-        self.register_buffer("esc_idx_bf16", esc_idx_bf16, persistent=False)
-        self.register_buffer("esc_vals_bf16", esc_vals_bf16, persistent=False)
-        self.bias = None if bias is None else nn.Parameter(bias, requires_grad=False)
+        self.out_features, self.in_features = int(Q), int(P)
+        fp16_table = _ascending(esc_idx, esc_vals)
+        # one table serves both modes unless the pack certifies bf16 separately (then the bf16 list is the full one)
+        bf16_table = fp16_table if esc_idx_bf16 is None else _ascending(esc_idx_bf16, esc_vals_bf16)
+        held = dict(tau_s=tau_s, min_s=min_s, nbits=nbits, bit_off=bit_off, ids=ids,
+                    esc_idx=fp16_table[0], esc_vals=fp16_table[1], esc_idx_bf16=bf16_table[0], esc_vals_bf16=bf16_table[1])
+        for name, tensor in held.items():               # none of them is saved with a state dict: the pack file is the source
+            self.register_buffer(name, tensor, persistent=False)
+        self.bias = nn.Parameter(bias, requires_grad=False) if bias is not None else None
 
     # ---- construction ------------------------------------------------------------------------------------------
 
@@ -119,59 +117,58 @@ class QVBandLinearV8(nn.Module):
         """Reads a `.qvband` / legacy QVB8 pack (module.py:162-218).  `tau` is accepted for call-site compatibility
         and ignored: every pack carries its own certified tau."""
         del tau
-        if blob is None:
-            with open(path, "rb") as fh:
-                blob = fh.read()
         dev = torch.device(device)
-        b = None
-        if bias is not None:
-            b = (bias.detach() if isinstance(bias, torch.Tensor) else torch.tensor(bias)).to(dev)
-        esc_bf16 = (None, None)
-        fp16_missing = False
-        certified = False
-        if blob[:4] != b"QVBD":
-            from qvb8_amd.formats.qvb8.decode import unpack_tensor
-            (min_s, tau_s, nb, bit_off, buf, Q, P, _tau, esc_idx, esc_vals) = unpack_tensor(blob)
-        else:
-            from qvb8_amd.formats.qvb8.pack_container import calc_method_of, unpack_formula, CALC_TABLE
-            if calc_method_of(blob) == CALC_TABLE:
-                raise NotImplementedError("qvb8 table (calc_method=1) packs are not read by QVBandLinearV8; "
-                                          "this is a pre-unification file, re-pack it.")
+        raw = blob if blob is not None else open(path, "rb").read()
+        tables = dict(fp16=None, bf16=None)             # (positions, values) per mode; bf16 stays None when one table serves both
+        flags = dict(bf16_certified=False, fp16_table_missing=False)
+        if raw[:4] == b"QVBD":
             from qvb8_amd.formats.qvb8.escape_split import fp16_list_for
-            d = unpack_formula(blob, skip_bit_decode=True, fp16_list=fp16_list_for(path), where=str(path))
-            min_s, tau_s, nb, bit_off, buf = d["min_s"], d["tau_s"], d["nbits"], d["bit_off"], d["buf"]
-            Q, P = d["Q"], d["P"]
-            certified = d.get("restore") == "fp16+bf16"
-            if d["esc_idx_fp16"] is None:
-                esc_idx, esc_vals = d["esc_idx"], d["esc_vals"]
-                fp16_missing = True
+            from qvb8_amd.formats.qvb8.pack_container import CALC_TABLE, calc_method_of, unpack_formula
+            if calc_method_of(raw) == CALC_TABLE:
+                raise NotImplementedError("QVBandLinearV8 reads formula packs only: this file keeps a value table per row "
+                                          "(calc_method = 1, written before the formats were unified) and has to be packed again")
+            rec = unpack_formula(raw, skip_bit_decode=True, fp16_list=fp16_list_for(path), where=str(path))
+            flags["bf16_certified"] = rec.get("restore") == "fp16+bf16"
+            full = (rec["esc_idx"], rec["esc_vals"])
+            if rec["esc_idx_fp16"] is None:             # a two-table pack whose fp16 list is not at hand: bf16 callers only
+                tables["fp16"], flags["fp16_table_missing"] = full, True
             else:
-                esc_idx, esc_vals = d["esc_idx_fp16"], d["esc_vals_fp16"]
-                if d["esc_idx_fp16"] is not d["esc_idx"]:
-                    esc_bf16 = (torch.from_numpy(d["esc_idx"].astype(np.int64)).to(dev),
-                                torch.from_numpy(d["esc_vals"].astype(np.float32)).to(dev))
-        mod = cls(min_s=torch.from_numpy(np.ascontiguousarray(min_s, np.float32)).to(dev),
-                  nbits=torch.from_numpy(np.ascontiguousarray(nb, np.uint8)).to(dev),
-                  bit_off=torch.from_numpy(np.ascontiguousarray(bit_off, np.int64)).to(dev),
-                  ids=torch.from_numpy(np.ascontiguousarray(buf)).to(dev),
-                  Q=Q, P=P, tau_s=torch.from_numpy(np.ascontiguousarray(tau_s, np.float32)).to(dev),
-                  esc_idx=torch.from_numpy(np.ascontiguousarray(esc_idx, np.int64)).to(dev),
-                  esc_vals=torch.from_numpy(np.ascontiguousarray(esc_vals, np.float32)).to(dev),
-                  bias=b, esc_idx_bf16=esc_bf16[0], esc_vals_bf16=esc_bf16[1])
-        mod.bf16_certified = certified
-        mod.fp16_table_missing = fp16_missing
+                tables["fp16"] = (rec["esc_idx_fp16"], rec["esc_vals_fp16"])
+                if rec["esc_idx_fp16"] is not rec["esc_idx"]:
+                    tables["bf16"] = full
+        else:
+            from qvb8_amd.formats.qvb8.decode import unpack_tensor
+            names = ("min_s", "tau_s", "nbits", "bit_off", "buf", "Q", "P", "tau", "esc_idx", "esc_vals")
+            rec = dict(zip(names, unpack_tensor(raw)))
+            tables["fp16"] = (rec["esc_idx"], rec["esc_vals"])
+        if isinstance(bias, torch.Tensor):
+            bias = bias.detach().to(dev)
+        elif bias is not None:
+            bias = torch.tensor(bias).to(dev)
+        second = tables["bf16"]
+        mod = cls(min_s=_on(dev, rec["min_s"], np.float32), tau_s=_on(dev, rec["tau_s"], np.float32),
+                  nbits=_on(dev, rec["nbits"], np.uint8), bit_off=_on(dev, rec["bit_off"], np.int64),
+                  ids=_on(dev, rec["buf"], None), Q=rec["Q"], P=rec["P"], bias=bias,
+                  esc_idx=_on(dev, tables["fp16"][0], np.int64), esc_vals=_on(dev, tables["fp16"][1], np.float32),
+                  esc_idx_bf16=None if second is None else _on(dev, second[0], np.int64),
+                  esc_vals_bf16=None if second is None else _on(dev, second[1], np.float32))
+        mod.bf16_certified, mod.fp16_table_missing = flags["bf16_certified"], flags["fp16_table_missing"]
         mod._where = str(path)
         return mod
 
     def escapes(self, dtype=torch.float16):
         """The escape table that goes with a weight rounded to `dtype`: the full list for bf16, the fp16 table otherwise
         (reference: module.py:116-124).  An fp16+bf16 pack whose fp16 table could not be determined refuses fp16."""
-        if dtype == torch.bfloat16:
-            return self.esc_idx_bf16, self.esc_vals_bf16
-        if dtype == torch.float16 and self.fp16_table_missing:
+        wants_bf16 = dtype == torch.bfloat16
+        if not wants_bf16:
+            self._need_fp16_table(dtype == torch.float16)
+        return (self.esc_idx_bf16, self.esc_vals_bf16) if wants_bf16 else (self.esc_idx, self.esc_vals)
+
+    def _need_fp16_table(self, asked: bool = True):
+        """Raises when an fp16 result is asked of a two-table pack whose fp16 escape list could not be determined."""
+        if asked and self.fp16_table_missing:
             from qvb8_amd.formats.qvb8.escape_split import fp16_missing_error
-            raise fp16_missing_error(getattr(self, "_where", "QVBandLinearV8"))
-        return self.esc_idx, self.esc_vals
+            raise fp16_missing_error(getattr(self, "_where", type(self).__name__))
 
     def row_subset(self, rows: torch.Tensor) -> "QVBandLinearV8":
         """The linear restricted to output rows `rows` (in that order).  A pack's rows are independent -- each has its own
@@ -265,34 +262,35 @@ class QVBandLinearV8(nn.Module):
     # ---- forward -----------------------------------------------------------------------------------------------
 
     def _finish(self, y, orig, out_dtype):
-        y = y.reshape(*orig[:-1], self.out_features)
+        """(M, Q) results of a kernel -> the caller's leading dimensions, bias added, in the caller's type."""
+        lead = tuple(orig[:-1])
         if self.bias is not None:
             y = y + self.bias.to(y.dtype)
-        return y.to(out_dtype)
+        return y.reshape(*lead, self.out_features).to(out_dtype)
+
+    def _rows_of(self, x: torch.Tensor):
+        """x as (M, P) rows on the weight's device and the type results go back in.  Under autocast an fp32 input is
+        computed and returned in the autocast type, as nn.Linear does (module.py:336-344)."""
+        rows = x.reshape(-1, x.shape[-1]).to(self.min_s.device)
+        result_dtype = x.dtype
+        if rows.dtype == torch.float32 and torch.is_autocast_enabled(rows.device.type):
+            low = torch.get_autocast_dtype(rows.device.type)
+            if low in (torch.float16, torch.bfloat16):
+                rows, result_dtype = rows.to(low), low
+        return rows.contiguous(), result_dtype
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         orig = x.shape
-        x2d = x.reshape(-1, orig[-1])
-        if x2d.device != self.min_s.device:
-            x2d = x2d.to(self.min_s.device)
-        out_dtype = x.dtype
-        if x2d.dtype == torch.float32 and torch.is_autocast_enabled(x2d.device.type):
-            ad = torch.get_autocast_dtype(x2d.device.type)          # honour autocast like nn.Linear (module.py:336-344)
-            if ad in (torch.bfloat16, torch.float16):
-                x2d = x2d.to(ad)
-                out_dtype = ad
-        M = x2d.shape[0]
-        if self.fp16_table_missing and x2d.dtype == torch.float16:
-            from qvb8_amd.formats.qvb8.escape_split import fp16_missing_error
-            raise fp16_missing_error(getattr(self, "_where", "QVBandLinearV8"))
-        if M == 0:
-            return x2d.new_zeros((*orig[:-1], self.out_features), dtype=out_dtype)
-        xk = x2d.contiguous()
+        xk, out_dtype = self._rows_of(x)
+        M = xk.shape[0]
+        # the mode decides the escape table: bf16 rows of a pack that certifies bf16 separately take the full list, every other
+        # call the fp16 table -- which a two-table pack may lack
         bf16_mode = bool(self.bf16_certified) and xk.dtype == torch.bfloat16
-        if self.fp16_table_missing and not bf16_mode:
-            from qvb8_amd.formats.qvb8.escape_split import fp16_missing_error
-            raise fp16_missing_error(getattr(self, "_where", "QVBandLinearV8"))
-        ei, ev = (self.esc_idx_bf16, self.esc_vals_bf16) if bf16_mode else (self.esc_idx, self.esc_vals)
+        self._need_fp16_table(xk.dtype == torch.float16)
+        if M == 0:
+            return xk.new_zeros((*orig[:-1], self.out_features), dtype=out_dtype)
+        self._need_fp16_table(not bf16_mode)
+        ei, ev = self.escapes(torch.bfloat16 if bf16_mode else torch.float32)
 
         order = self._mma_order() if M <= max(_MMA_SPLIT_MAX, ext.MMA_GEMM_MAX_M) else None
         if order is not None and M > _MMA_MAX_M and not self._gemm_ok(order[2], bf16_mode):
@@ -334,14 +332,11 @@ class QVBandLinearV8(nn.Module):
 def enable_bf16_gemm(model: nn.Module) -> tuple[int, int]:
     """Put every bf16-certified QVBandLinearV8 in `model` on the bf16 GEMM for large M; returns
     (switched, packed_linears) (module.py:506-524)."""
-    n = tot = 0
-    for m in model.modules():
-        if isinstance(m, QVBandLinearV8):
-            tot += 1
-            if m.bf16_certified:
-                m.bf16_gemm = True
-                n += 1
-    return n, tot
+    packed = [m for m in model.modules() if isinstance(m, QVBandLinearV8)]
+    certified = [m for m in packed if m.bf16_certified]
+    for m in certified:
+        m.bf16_gemm = True
+    return len(certified), len(packed)
 
 
 def footprint_report(module) -> dict:
