@@ -64,6 +64,18 @@ def _ascending(positions, values):
     return positions[order].contiguous(), values[order].contiguous()
 
 
+def activation_rows(x: torch.Tensor, device):
+    """x as contiguous (M, P) rows on `device`, and the type results go back in.  Under autocast an fp32 input is computed
+    and returned in the autocast type, as nn.Linear does (module.py:336-344)."""
+    rows = x.reshape(-1, x.shape[-1]).to(device)
+    result_dtype = x.dtype
+    if rows.dtype == torch.float32 and torch.is_autocast_enabled(rows.device.type):
+        low = torch.get_autocast_dtype(rows.device.type)
+        if low in (torch.float16, torch.bfloat16):
+            rows, result_dtype = rows.to(low), low
+    return rows.contiguous(), result_dtype
+
+
 def _on(dev, array, dtype):
     return torch.from_numpy(np.ascontiguousarray(array, dtype)).to(dev)
 
@@ -269,15 +281,7 @@ class QVBandLinearV8(nn.Module):
         return y.reshape(*lead, self.out_features).to(out_dtype)
 
     def _rows_of(self, x: torch.Tensor):
-        """x as (M, P) rows on the weight's device and the type results go back in.  Under autocast an fp32 input is
-        computed and returned in the autocast type, as nn.Linear does (module.py:336-344)."""
-        rows = x.reshape(-1, x.shape[-1]).to(self.min_s.device)
-        result_dtype = x.dtype
-        if rows.dtype == torch.float32 and torch.is_autocast_enabled(rows.device.type):
-            low = torch.get_autocast_dtype(rows.device.type)
-            if low in (torch.float16, torch.bfloat16):
-                rows, result_dtype = rows.to(low), low
-        return rows.contiguous(), result_dtype
+        return activation_rows(x, self.min_s.device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         orig = x.shape

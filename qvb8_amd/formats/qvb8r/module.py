@@ -15,7 +15,7 @@ import torch
 import torch.nn as nn
 
 from qvb8_amd import ext_qvb8r as ext
-from qvb8_amd.formats.qvb8.module import apply_keeping_fp32_metadata  # noqa: F401  (same metadata rule)
+from qvb8_amd.formats.qvb8.module import activation_rows, apply_keeping_fp32_metadata  # noqa: F401  (same metadata rule)
 from . import container as QF
 
 WPB = 8                    # tiles per block of the schedule the kernels use
@@ -42,6 +42,49 @@ def _apply_keeping_fp32(module: nn.Module, fn, recurse=True):
     return out
 
 
+def _register_walk_operands(module: nn.Module, d: dict, dev) -> tuple:
+    """Registers what every QVB8R kernel walks -- coded words and tile offsets, initial states, tile and block tables, slot
+    tables, row order, row constants -- as buffers of `module` (names of the reference's modules); returns (tiles, blocks)
+    as host arrays for the caller's own planning."""
+    tab, tiles, words, off = QF.runtime_tables(d)
+    blocks = QF.blocks_for(tiles, WPB)
+    operands = {
+        "words": words.view(np.int32), "off": off, "states": np.asarray(d["states"], np.uint64).view(np.int64), "tiles": tiles,
+        "drow": np.asarray(d["drow"]).astype(np.int32), "tab": tab.view(np.int32), "perm": np.asarray(d["perm"], np.int32),
+        "blocks8": blocks, "min_s": np.asarray(d["min_s"], np.float32), "tau_s": np.asarray(d["tau_s"], np.float32),
+    }
+    for name, array in operands.items():
+        module.register_buffer(name, _t(array, dev), persistent=False)
+    return tiles, blocks
+
+
+def _fp16_subset(positions: np.ndarray, path, certified_bf16: bool):
+    """Which entries of the file's (full, bf16) escape list also belong to the fp16 table: all of them for a one-table pack;
+    for an fp16+bf16 pack those that escape_tables.json names -- None when that file is not there."""
+    if not certified_bf16:
+        return np.ones(len(positions), bool)
+    from qvb8_amd.formats.qvb8.escape_split import fp16_list_for, select_fp16
+    listed = fp16_list_for(path)
+    return None if listed is None else select_fp16(positions, listed, str(path))
+
+
+def _plan_chunks(tiles, blocks, budget_rows: int) -> list:
+    """Runs of whole blocks with at most `budget_rows` rows each (a single block may exceed it): (first block, blocks, first
+    sorted row, rows)."""
+    plan, start = [], 0
+    while start < len(blocks):
+        stop, rows = start, 0
+        while stop < len(blocks):
+            block_rows = int(tiles[blocks[stop][1]:blocks[stop][1] + blocks[stop][2], 2].sum())
+            if rows and rows + block_rows > budget_rows:
+                break
+            rows += block_rows
+            stop += 1
+        plan.append((start, stop - start, int(tiles[blocks[start][1], 1]), rows))
+        start = stop
+    return plan
+
+
 class QVBandLinearV8R(nn.Module):
     CHUNK_BYTES = 512 << 20
     bf16_gemm = False
@@ -49,61 +92,35 @@ class QVBandLinearV8R(nn.Module):
 
     def __init__(self, d: dict, bias=None, device="cuda", path: str | None = None):
         super().__init__()
-        self.path = path
+        self.path, self._where = path, str(path)
         self._arrays = None if path else d               # built from arrays, not from a file: kept for host_arrays()
-        tab, tiles, words, off = QF.runtime_tables(d)
-        Q, P = int(d["Q"]), int(d["P"])
-        self.out_features, self.in_features, self.T = Q, P, int(d["T"])
         dev = torch.device(device)
-        buf = lambda name, a: self.register_buffer(name, _t(a, dev), persistent=False)
-        buf("words", words.view(np.int32)); buf("off", off)
-        buf("states", np.asarray(d["states"], np.uint64).view(np.int64)); buf("tiles", tiles)
-        buf("drow", np.asarray(d["drow"]).astype(np.int32))
-        buf("tab", tab.view(np.int32)); buf("perm", np.asarray(d["perm"], np.int32))
-        blocks8 = QF.blocks_for(tiles, WPB)
-        buf("blocks8", blocks8)
-        buf("min_s", np.asarray(d["min_s"], np.float32)); buf("tau_s", np.asarray(d["tau_s"], np.float32))
+        self.out_features, self.in_features, self.T = int(d["Q"]), int(d["P"]), int(d["T"])
+        P = self.in_features
+        tiles, blocks = _register_walk_operands(self, d, dev)
         self.cert = d.get("cert", {}) or {}
         self.bf16_certified = self.cert.get("restore") == "fp16+bf16"
-        # two escape tables (module.py:100-118): the file holds the full (bf16) list; the fp16 table comes only from
-        # escape_tables.json.  No file on an fp16+bf16 pack: one table, and fp16 forwards refuse.
-        ei_b = np.asarray(d["esc_idx"]).astype(np.int64)
-        ev_b = np.asarray(d["esc_val"], np.float32)
-        ed_b = np.asarray(d["esc_delta"], np.float32)
-        need = np.ones(len(ei_b), bool)
-        self.fp16_table_missing = False
-        self._where = str(path)
-        if self.bf16_certified:
-            from qvb8_amd.formats.qvb8.escape_split import fp16_list_for, select_fp16
-            lst = fp16_list_for(path)
-            if lst is None:
-                self.fp16_table_missing = True
-            else:
-                need = select_fp16(ei_b, lst, str(path))
-        ei, ev, ed = ei_b[need], ev_b[need], ed_b[need]
-        # correction tables grouped by output row (CSR, sorted by row then column): one thread per (m, q) adds its
-        # group in this order -- reproducible
-        o = np.argsort(ei, kind="stable")
-        es = ei[o]
-        uq, cnt = np.unique(es // P, return_counts=True) if len(es) else (np.zeros(0, np.int64), np.zeros(0, np.int64))
-        buf("esc_uq", uq.astype(np.int64)); buf("esc_ptr", np.concatenate([[0], np.cumsum(cnt)]).astype(np.int64))
-        buf("esc_c", (es % P).astype(np.int64)); buf("esc_delta", ed[o].astype(np.float32))
-        buf("esc_flat", ei); buf("esc_val", ev)
-        buf("esc_flat_bf16", ei_b); buf("esc_val_bf16", ev_b)
-        self.bias = None if bias is None else nn.Parameter(bias.detach().to(dev), requires_grad=False)
-        # M > 48: chunks of whole blocks, about CHUNK_BYTES of decoded 16-bit weight each:
-        # (first block, blocks, first sorted row, rows)
-        rows_per_block = [int(tiles[t0:t0 + n, 2].sum()) for _, t0, n in blocks8]
-        first_row = [int(tiles[t0, 1]) for _, t0, n in blocks8]
-        budget = max(1, self.CHUNK_BYTES // (2 * P))
-        self.chunks, b = [], 0
-        while b < len(blocks8):
-            b1, rows = b, 0
-            while b1 < len(blocks8) and (rows == 0 or rows + rows_per_block[b1] <= budget):
-                rows += rows_per_block[b1]
-                b1 += 1
-            self.chunks.append((b, b1 - b, first_row[b], rows))
-            b = b1
+        # Two escape tables (module.py:100-118): the file holds the full list, which is the bf16 table; the fp16 table is the
+        # subset escape_tables.json names.  Without that file an fp16+bf16 pack has one table, and fp16 forwards refuse.
+        full_pos = np.asarray(d["esc_idx"]).astype(np.int64)
+        full_val = np.asarray(d["esc_val"], np.float32)
+        subset = _fp16_subset(full_pos, path, self.bf16_certified)
+        self.fp16_table_missing = subset is None
+        if subset is None:
+            subset = np.ones(len(full_pos), bool)
+        pos, val, delta = full_pos[subset], full_val[subset], np.asarray(d["esc_delta"], np.float32)[subset]
+        # the correction after a fused product runs per output row: escapes grouped by row, columns ascending inside a row
+        # (one thread per (m, q) adds its group in that order -- reproducible)
+        by_row = np.argsort(pos, kind="stable")
+        rows_hit, per_row = np.unique(pos[by_row] // P, return_counts=True) if len(pos) else (np.zeros(0, np.int64), np.zeros(0, np.int64))
+        tables = {"esc_uq": rows_hit.astype(np.int64), "esc_ptr": np.concatenate([[0], np.cumsum(per_row)]).astype(np.int64),
+                  "esc_c": (pos[by_row] % P).astype(np.int64), "esc_delta": delta[by_row].astype(np.float32),
+                  "esc_flat": pos, "esc_val": val, "esc_flat_bf16": full_pos, "esc_val_bf16": full_val}
+        for name, array in tables.items():
+            self.register_buffer(name, _t(array, dev), persistent=False)
+        self.bias = nn.Parameter(bias.detach().to(dev), requires_grad=False) if bias is not None else None
+        # beyond 48 rows of X: dense restore of about CHUNK_BYTES of 16-bit weight at a time
+        self.chunks = _plan_chunks(tiles, blocks, max(1, self.CHUNK_BYTES // (2 * P)))
 
     @classmethod
     def from_packfile(cls, path: str, *, bias=None, tau: float | None = None, device: str = "cuda", blob: bytes | None = None):
@@ -163,44 +180,38 @@ class QVBandLinearV8R(nn.Module):
         return y
 
     def forward(self, x):
-        shp = x.shape
-        x2 = x.reshape(-1, shp[-1])
-        if x2.device != self.words.device:
-            x2 = x2.to(self.words.device)
-        out_dtype = x.dtype
-        if x2.dtype == torch.float32 and torch.is_autocast_enabled(x2.device.type):
-            ad = torch.get_autocast_dtype(x2.device.type)
-            if ad in (torch.bfloat16, torch.float16):
-                x2, out_dtype = x2.to(ad), ad
-        M = x2.shape[0]
+        lead = tuple(x.shape[:-1])
+        rows, out_dtype = activation_rows(x, self.words.device)
+        M = rows.shape[0]
         if M == 0:
-            return x2.new_empty(*shp[:-1], self.out_features, dtype=out_dtype)
-        if self.fp16_table_missing and not (x2.dtype == torch.bfloat16 and self.bf16_gemm and M > self._TC_SPLIT_MAX):
+            return rows.new_empty(*lead, self.out_features, dtype=out_dtype)
+        dense_bf16 = bool(self.bf16_gemm and rows.dtype == torch.bfloat16 and M > self._TC_SPLIT_MAX)
+        if self.fp16_table_missing and not dense_bf16:
             from qvb8_amd.formats.qvb8.escape_split import fp16_missing_error
             raise fp16_missing_error(self._where)
-        if M <= ext.MAX_M:
-            y = self._small(x2)
-        elif M <= self._TC_SPLIT_MAX:
-            n = -(-M // ext.MAX_M)
-            step = -(-M // n)
-            y = torch.cat([self._small(x2[i:i + step]) for i in range(0, M, step)])
+        if M <= self._TC_SPLIT_MAX:
+            # one fused walk per call of at most ext.MAX_M rows; more rows are split evenly
+            calls = -(-M // ext.MAX_M)
+            per_call = -(-M // calls)
+            parts = [self._small(rows[at:at + per_call]) for at in range(0, M, per_call)]
+            y = parts[0] if len(parts) == 1 else torch.cat(parts)
         else:
-            y = self._chunked(x2, bf16=bool(self.bf16_gemm and self.bf16_certified and x2.dtype == torch.bfloat16))
+            y = self._chunked(rows, bf16=dense_bf16 and bool(self.bf16_certified))
         if self.bias is not None:
             y = y + self.bias.to(y.dtype)
-        return y.to(out_dtype).reshape(*shp[:-1], self.out_features)
+        return y.reshape(*lead, self.out_features).to(out_dtype)
 
     def dense(self, dtype=torch.bfloat16):
         """The exact weight (Q, P) in `dtype` (escapes applied): for audits and re-packing, never on the hot path
         (module.py:313-325)."""
-        code = {torch.float16: 0, torch.bfloat16: 1}.get(dtype, 2)
         if dtype == torch.float16 and self.fp16_table_missing:
             from qvb8_amd.formats.qvb8.escape_split import fp16_missing_error
             raise fp16_missing_error(self._where)
-        W = ext.decode(*self._core(), self.in_features, code, 0, self.blocks8.shape[0], -1, 0, T=self.T)
-        ef, ev = (self.esc_flat_bf16, self.esc_val_bf16) if dtype == torch.bfloat16 else (self.esc_flat, self.esc_val)
-        if ef.numel():
-            W.view(-1)[ef] = ev.to(W.dtype)
+        restore_code = 0 if dtype == torch.float16 else 1 if dtype == torch.bfloat16 else 2
+        W = ext.decode(*self._core(), self.in_features, restore_code, 0, self.blocks8.shape[0], -1, 0, T=self.T)
+        positions, values = (self.esc_flat_bf16, self.esc_val_bf16) if dtype == torch.bfloat16 else (self.esc_flat, self.esc_val)
+        if positions.numel():
+            W.view(-1).index_copy_(0, positions, values.to(W.dtype))
         return W.to(dtype)
 
 
@@ -214,18 +225,11 @@ class QVBandEmbeddingV8R(nn.Module):
     def __init__(self, d: dict, out_dtype=torch.bfloat16, device="cuda", path: str | None = None):
         super().__init__()
         self.path = path
-        tab, tiles, words, off = QF.runtime_tables(d)
         Q, P = int(d["Q"]), int(d["P"])
         self.num_embeddings, self.embedding_dim, self._out_dtype, self.T = Q, P, out_dtype, int(d["T"])
         dev = torch.device(device)
+        tiles, blocks8 = _register_walk_operands(self, d, dev)
         buf = lambda name, a: self.register_buffer(name, _t(a, dev), persistent=False)
-        buf("words", words.view(np.int32)); buf("off", off)
-        buf("states", np.asarray(d["states"], np.uint64).view(np.int64)); buf("tiles", tiles)
-        buf("drow", np.asarray(d["drow"]).astype(np.int32))
-        buf("tab", tab.view(np.int32)); buf("perm", np.asarray(d["perm"], np.int32))
-        blocks8 = QF.blocks_for(tiles, WPB)
-        buf("blocks8", blocks8)
-        buf("min_s", np.asarray(d["min_s"], np.float32)); buf("tau_s", np.asarray(d["tau_s"], np.float32))
         # original row -> slot of its decoded copy inside its block: block number and (tile in block) * T + row in tile
         perm = np.asarray(d["perm"]).astype(np.int64)
         sorted_pos = np.empty(Q, np.int64)
@@ -239,14 +243,13 @@ class QVBandEmbeddingV8R(nn.Module):
         # pack (named by escape_tables.json), the file's full list otherwise; grouped by row
         ei = np.asarray(d["esc_idx"]).astype(np.int64)
         ev = np.asarray(d["esc_val"], np.float32)
-        cert = d.get("cert", {}) or {}
-        if out_dtype == torch.float16 and cert.get("restore") == "fp16+bf16":
-            from qvb8_amd.formats.qvb8.escape_split import fp16_list_for, fp16_missing_error, select_fp16
-            lst = fp16_list_for(path)
-            if lst is None:
+        two_tables = (d.get("cert", {}) or {}).get("restore") == "fp16+bf16"
+        if out_dtype == torch.float16 and two_tables:
+            subset = _fp16_subset(ei, path, True)
+            if subset is None:
+                from qvb8_amd.formats.qvb8.escape_split import fp16_missing_error
                 raise fp16_missing_error(str(path))
-            need = select_fp16(ei, lst, str(path))
-            ei, ev = ei[need], ev[need]
+            ei, ev = ei[subset], ev[subset]
         order = np.argsort(ei, kind="stable")
         ei, ev = ei[order], ev[order]
         counts = np.bincount(ei // P, minlength=Q) if len(ei) else np.zeros(Q, np.int64)
