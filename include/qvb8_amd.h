@@ -221,9 +221,9 @@ int64_t qvb8_moe_workspace_bytes(int64_t tokens, int64_t topk, int64_t n_experts
  * NaN: in every output row of the token that holds it, and in the whole output on the paths that group by expert.
  * Up to 16 tokens with topk <= 8, fp16 / bf16 X, P_up and P_dn multiples of 128 up to 4096 and Q_dn a multiple of 16 run
  * on the matrix cores, H handed over as saturated fp16:
- *   1 or 2 tokens: two launches, every token a problem of its own (slot j = expert idx[t][j]); the down projection adds
- *     the slots up with their routing weights;
- *   3 .. 16 tokens: four launches (plan, up, down, combine): the (token, choice) pairs are grouped by expert, the tokens
+ *   1 .. 6 tokens: two launches, every token a problem of its own (slot j = expert idx[t][j]; an expert is read once per
+ *     token that chose it); the down projection adds the slots up with their routing weights;
+ *   7 .. 16 tokens: four launches (plan, up, down, combine): the (token, choice) pairs are grouped by expert, the tokens
  *     that chose an expert are the token rows of one MFMA operand, and every selected expert is read ONCE however many
  *     tokens chose it.
  * Everything else takes the general path (four launches, H in fp32, an expert read once for up to 8 of its tokens).

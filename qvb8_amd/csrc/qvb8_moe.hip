@@ -347,6 +347,7 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
     __shared__ float s_sx[kOneMaxTiles][kOneWaves];          // sum of the activations over the column range
     __shared__ float2 s_fin[kOneMaxTiles][16];               // tau_s, min_s of the tile's rows
     __shared__ int s_ok[kOneMaxTiles];                       // the slot's expert number is inside the stack
+    __shared__ __align__(16) uint16_t s_x[kOneWaves][T * kStepCols];   // each wave's activations, narrowed (private to the wave)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, kg = lane >> 4;
@@ -380,25 +381,30 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
     struct Round { int i; bool has; int nb; int64_t bit0; float ts, mn; bool e_ok, ok, sliced; };
     Round rd[R];
     uint4 wlo[R][T], whi[R][T];
-    v4u_t xa[T][4];
+    // The wave's 128 T columns of the token are 16 T pieces of 16 bytes: a lane requests one (or two) of them, narrows it
+    // like every activation when it arrives as bf16 (zero past the end of the row) and leaves it in the wave's own part
+    // of LDS; multiply reads the MFMA operands from there just before it needs them (every operand row holds the token:
+    // only result row 0 is used).  Four registers instead of the 16 T of operands held across the wait for the ids, and
+    // one narrowing per value instead of sixteen.
+    constexpr int XP = (16 * T + kWave - 1) / kWave;
+    v4u_t xc[XP];
     auto request_x = [&](const uint16_t* xrow) {
 #pragma unroll
-        for (int it = 0; it < T; ++it) {
-            const bool on = (step0 + it) < n_steps;
-            const uint16_t* xp = xrow + (on ? (size_t)(step0 + it) * kStepCols + kg * 32 : (size_t)0);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) xa[it][j] = *reinterpret_cast<const v4u_t*>(xp + 8 * j);
+        for (int i = 0; i < XP; ++i) {
+            const int piece = lane + kWave * i;
+            const bool on = piece < 16 * T && (step0 + (piece >> 4)) < n_steps;
+            xc[i] = *reinterpret_cast<const v4u_t*>(xrow + (on ? (size_t)step0 * kStepCols + (size_t)piece * 8 : (size_t)0));
         }
     };
-    // the token sits in row 0 of its operand; narrowed like every activation when it arrives as bf16
     auto finish_x = [&]() {
 #pragma unroll
-        for (int it = 0; it < T; ++it) {
-            const bool on = (step0 + it) < n_steps && r == 0;
+        for (int i = 0; i < XP; ++i) {
+            const int piece = lane + kWave * i;
+            const bool on = (step0 + (piece >> 4)) < n_steps;
+            v4u_t v;
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int k = 0; k < 4; ++k) xa[it][j][k] = on ? XI::pair(xa[it][j][k]) : 0u;
+            for (int k = 0; k < 4; ++k) v[k] = on ? XI::pair(xc[i][k]) : 0u;
+            if (piece < 16 * T) *reinterpret_cast<v4u_t*>(&s_x[wave][piece * 8]) = v;
         }
     };
     // nothing here is under a branch: a wave without a tile in this round reads the metadata of tile 0 and the start of ids
@@ -448,10 +454,6 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
         const int nb = q.nb;
         const bool sliced = q.sliced;
         v4f_t sx = {0.f, 0.f, 0.f, 0.f}, acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int it = 0; it < T; ++it)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) sx = F::mfma(xa[it][j], ones, sx);
         const uint32_t info = sliced ? ((uint32_t)nb | 256u) : 0u;
         // REG: one width for the whole stack, known without looking at the lanes (rows that cannot be read -- an expert
         // number outside the stack -- decode whatever was loaded; their results are replaced by NaN below)
@@ -480,8 +482,13 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
                     if (__builtin_amdgcn_ballot_w64(sliced && nb == 8)) { if (sliced && nb == 8) decode_slice<8, false>(lo, hi, b); }
                 }
             }
+            v4u_t xa[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc = F::mfma(xa[it][j], b[j], acc);
+            for (int j = 0; j < 4; ++j) xa[j] = *reinterpret_cast<const v4u_t*>(&s_x[wave][it * kStepCols + kg * 32 + 8 * j]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sx = F::mfma(xa[j], ones, sx);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc = F::mfma(xa[j], b[j], acc);
         }
         if (!q.has) return;                                   // wave-uniform
         const int i = q.i;
@@ -936,9 +943,10 @@ bool moe_one_token_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t P_up, i
     if (tokens > host::env_int("QVB8_MOE_TILE_TOKENS", 16) || topk > 8) return false;
     return moe_walk_shapes_ok(topk, x_dtype, P_up, Q_dn, P_dn) && host::env_int("QVB8_MOE_ONE_TOKEN", 1) != 0;
 }
-// grouped by expert (3..16 tokens; two tokens are faster one by one: 36 against 40 us per layer at the 35B-A3B shapes)
+// grouped by expert (7..16 tokens; fewer are faster one by one although an expert is then read once per token that chose it:
+// 31 against 44 us per layer at 3 tokens, 53 against 56 at 6, 67 against 66 at 8 at the 35B-A3B shapes)
 bool moe_group_ok(int64_t tokens, int64_t topk, int x_dtype, int64_t P_up, int64_t Q_dn, int64_t P_dn) {
-    if (tokens < host::env_int("QVB8_MOE_GROUP_FROM", 3) || tokens > 16) return false;
+    if (tokens < host::env_int("QVB8_MOE_GROUP_FROM", 7) || tokens > 16) return false;
     return moe_walk_shapes_ok(topk, x_dtype, P_up, Q_dn, P_dn) && host::env_int("QVB8_MOE_GROUPED", 1) != 0;
 }
 
@@ -1049,10 +1057,13 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
         o.X = reinterpret_cast<const uint16_t*>(X); o.idx = idx; o.w = w; o.ids = up_ids; o.ids_bytes = up_ids_bytes;
         o.min_s = up_min; o.tau_s = up_tau; o.nbits = up_nb; o.bit_off = up_off; o.out = H;
         o.E = (int)n_experts; o.Q = (int)Q_up; o.P = (int)P_up; o.topk = (int)topk; o.units = (int)P_dn; o.gated = act == 0 ? 1 : 0;
-        // unit tiles per workgroup: about one workgroup per CU, within what the rounds of a workgroup can take
+        // unit tiles per workgroup: two workgroups fit a CU (at most 128 registers per lane), and a workgroup that takes its
+        // tiles in one round has all its requests out at once -- so as few tiles each as 2 x CUs workgroups allow, within
+        // what the rounds of a workgroup can take
         const int RT = o.gated ? 2 : 1;
         const int64_t total_ut = topk * (P_dn / 16);
-        int64_t per_wg = (total_ut + host::device_cus() - 1) / host::device_cus();
+        const int64_t places = (int64_t)host::device_cus() * host::env_int("QVB8_MOE_ONE_WGS_PER_CU", 2);
+        int64_t per_wg = (total_ut + places - 1) / places;
         const int64_t cap = kOneMaxTiles / RT;
         if (per_wg > cap) per_wg = cap;
         if (per_wg < 1) per_wg = 1;

@@ -184,8 +184,10 @@ def test_moe_refusals():
 
 @pytest.mark.parametrize("T,k,dtype", [(2, 2, torch.bfloat16), (3, 2, torch.bfloat16), (5, 4, torch.float16), (16, 8, torch.bfloat16),
                                        (9, 1, torch.float16)])
-def test_moe_few_tokens_share_each_expert(T, k, dtype):
-    """2..16 tokens on the matrix cores: from three tokens on, the tokens that chose an expert share one walk over it.  Shapes the grouped
+@pytest.mark.parametrize("group_from", ["3", None])
+def test_moe_few_tokens_share_each_expert(T, k, dtype, group_from, monkeypatch):
+    """2..16 tokens on the matrix cores: one grid row per token through the one-token kernels, or (from seven tokens on by
+    default, from three with QVB8_MOE_GROUP_FROM=3) the tokens that chose an expert share one walk over it.  Shapes the grouped
     kernels take (row lengths that are multiples of 128), more experts than get selected and experts selected by many
     tokens at once; against the oracle, reproducible, and equal to the per-token result of the same library."""
     E, hidden, inter = 12, 384, 128
@@ -197,6 +199,8 @@ def test_moe_few_tokens_share_each_expert(T, k, dtype):
             others = [e for e in range(E) if e != 3]
             idx[t, 1:] = np.random.default_rng(t).choice(others, k - 1, replace=False)
     x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(dtype)
+    if group_from is not None:
+        monkeypatch.setenv("QVB8_MOE_GROUP_FROM", group_from)
     mod = QVBandExpertsV8(gu, dn, num_experts=E)
     args = (x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
     out = mod(*args)
@@ -210,8 +214,9 @@ def test_moe_few_tokens_share_each_expert(T, k, dtype):
     assert torch.isnan(mod(args[0], bad, args[2]).float()[T - 1]).all()
 
 
-def test_moe_few_tokens_relu2_and_rows_the_slicing_cannot_read():
-    """The grouped kernels on hand-made packs: non-gated ReLU^2, every width 1..14 among the up rows (the element-wise
+@pytest.mark.parametrize("group_from", ["3", None])
+def test_moe_few_tokens_relu2_and_rows_the_slicing_cannot_read(group_from, monkeypatch):
+    """The few-token kernels (6 tokens: grouped walk or one grid row per token; 13: grouped walk) on hand-made packs: non-gated ReLU^2, every width 1..14 among the up rows (the element-wise
     path inside the grouped kernel), row lengths of 128 and 256."""
     E, hidden, inter = 4, 256, 128
     ups, dns, Wup, Wdn = [], [], [], []
@@ -233,6 +238,8 @@ def test_moe_few_tokens_relu2_and_rows_the_slicing_cannot_read():
             ids[o:o + t["ids"].numel()] = t["ids"]
         return (ids, torch.stack([t["min_s"] for t in lst]), torch.stack([t["tau_s"] for t in lst]),
                 torch.stack([t["nbits"] for t in lst]), torch.stack([t["bit_off"] + 8 * o for t, o in zip(lst, offs)]))
+    if group_from is not None:
+        monkeypatch.setenv("QVB8_MOE_GROUP_FROM", group_from)
     for T, k in ((6, 2), (13, 3)):
         idx, w = _route(T, E, k, seed=T)
         x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(torch.float16)
@@ -241,11 +248,12 @@ def test_moe_few_tokens_relu2_and_rows_the_slicing_cannot_read():
         _check(out, O.moe_reference(x.float().numpy(), idx, w, Wup, Wdn, act="relu2"), torch.float16)
 
 
-def test_moe_few_tokens_rows_longer_than_2048_columns():
-    """The grouped walk with rows of 2304 columns in the up projection (eight steps per wave, one register set) and of
+def test_moe_few_tokens_rows_longer_than_2048_columns(monkeypatch):
+    """The grouped walk (asked for from three tokens on) with rows of 2304 columns in the up projection (eight steps per wave, one register set) and of
     640 in the down projection; 4 tokens, top-2 of 4 experts."""
     E, hidden, inter = 4, 2304, 640
     gu, dn, Wgu, Wdn = _experts(E, hidden, inter, 2e-3, seed=4100)
+    monkeypatch.setenv("QVB8_MOE_GROUP_FROM", "3")
     mod = QVBandExpertsV8(gu, dn, num_experts=E)
     idx, w = _route(4, E, 2, seed=77)
     x = torch.randn(4, hidden, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
