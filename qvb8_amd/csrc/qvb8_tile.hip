@@ -145,6 +145,9 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
     // pieces before anything else, the first tile's ids follow at once, and the workgroup shares X after one barrier --
     // so the trip of the activations and the first trip of the ids overlap, and later panels need no trip for theirs.
     unsigned char* xs = reinterpret_cast<unsigned char*>(part + (size_t)rows_cap * ranges * MS);     // [M][P] in operand format
+    // JIT: with one token tile and X in LDS a step's operands are read from LDS when the step is multiplied instead of being
+    // held in 16 T registers for the whole panel (lanes without a row of X, and steps past the end, read 64 bytes of zeros)
+    constexpr bool JIT = XL && NT == 1;
     const int x_pieces = (a.M * a.P) >> 3;
     v4u_t xg[XL ? XP : 1];
     if constexpr (XL) {
@@ -275,6 +278,7 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
             if (idx < x_pieces) reinterpret_cast<v4u_t*>(xs)[idx] = v;
             __builtin_amdgcn_sched_barrier(0);
         }
+        if constexpr (JIT) { if (tid < 16) reinterpret_cast<uint32_t*>(xs + (size_t)x_pieces * 16)[tid] = 0u; }   // 64 bytes of zeros behind X
         // A bare barrier behind this wave's own LDS writes: __syncthreads() carries a release fence that would also wait
         // for the ids just requested.
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -293,8 +297,15 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
         // ---- activations of this wave's columns, in MFMA operand layout: lane (t = l % 16, kg) holds
         //      X[16*nt + t][128*(step0+it) + 32*kg + 8*j + 0..7] ----
         v4u_t xa[NT][T][4];
+        const uint32_t x_zero = (uint32_t)x_pieces * 16u;
+        auto x_operand = [&](int it, v4u_t (&xv)[4]) __attribute__((always_inline)) {
+            const bool on = active && r < a.M && (step0 + it) < a.n_steps;
+            const uint32_t at = on ? 2u * ((uint32_t)r * (uint32_t)a.P + (uint32_t)(step0 + it) * kStepCols + (uint32_t)kg * 32u) : x_zero;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
+            for (int j = 0; j < 4; ++j) xv[j] = *reinterpret_cast<const v4u_t*>(xs + at + 16 * j);
+        };
+#pragma unroll
+        for (int nt = 0; nt < (JIT ? 0 : NT); ++nt) {
             const int t = nt * 16 + r;
 #pragma unroll
             for (int it = 0; it < T; ++it) {
@@ -333,20 +344,26 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             sx[nt] = v4f_t{0.f, 0.f, 0.f, 0.f};
+            if constexpr (!JIT) {
 #pragma unroll
-            for (int it = 0; it < T; ++it)
+                for (int it = 0; it < T; ++it)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) sx[nt] = F::mfma(xa[nt][it][j], ones, sx[nt]);
+                    for (int j = 0; j < 4; ++j) sx[nt] = F::mfma(xa[nt][it][j], ones, sx[nt]);
+            }
         }
-        if (active && g == 0 && r == 0) {
+        // JIT: the sums are taken while the wave's first tile is multiplied (its operands are in registers then)
+        auto put_sums = [&]() __attribute__((always_inline)) {
+            if (active && g == 0 && r == 0) {
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+                for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float* dst = sxs + range * TM + nt * 16 + kg * 4 + e;
-                    *dst = first_panel ? sx[nt][e] : *dst + sx[nt][e];
-                }
-        }
+                    for (int e = 0; e < 4; ++e) {
+                        float* dst = sxs + range * TM + nt * 16 + kg * 4 + e;
+                        *dst = first_panel ? sx[nt][e] : *dst + sx[nt][e];
+                    }
+            }
+        };
+        if constexpr (!JIT) put_sums();
         // The first tile's ids are requested only now, after the activations have ARRIVED: requesting them earlier --
         // before the activations, or right behind them -- was measured to cost about a microsecond per launch (the few
         // activation requests then compete with the flood of id requests of the whole chip).
@@ -364,6 +381,14 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
 #pragma unroll
             for (int it = 0; it < T; ++it) {
                 v4u_t b[4];
+                const int xi = JIT ? 0 : it;
+                if constexpr (JIT) {
+                    x_operand(it, xa[0][0]);                       // this step's operands, in the first register set
+                    if (tk == 0) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) sx[0] = F::mfma(xa[0][0][j], ones, sx[0]);
+                    }
+                }
                 const uint4 lo = to_operand(wlo[it]), hi = to_operand(whi[it]);
                 if (uniform) {
                     switch (info0 & 0xFFu) {
@@ -391,19 +416,20 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
 #pragma unroll
                             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                                for (int j = 0; j < 4; ++j) acc_top[nt] = F::mfma(xa[nt][it][j], bt[j], acc_top[nt]);
+                                for (int j = 0; j < 4; ++j) acc_top[nt] = F::mfma(xa[nt][xi][j], bt[j], acc_top[nt]);
                         }
                     }
                 }
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[nt] = F::mfma(xa[nt][it][j], b[j], acc[nt]);
+                    for (int j = 0; j < 4; ++j) acc[nt] = F::mfma(xa[nt][xi][j], b[j], acc[nt]);
             }
             // the next tile's ids (after the last tile: the next panel's first) are requested before this tile's sums
             // are put away
             if (tk + 1 < n_mine) info = issue_tile(tk + 1, step0, wlo, whi);
             else if (more) info = issue_tile(0, step0_next, wlo, whi);
+            if constexpr (JIT) { if (tk == 0) put_sums(); }
 
             // ---- tile done for this wave: remove the bias, store into the wave's own LDS slots ----
             const int lt = g + a.G * tk;                                // the workgroup's local tile
@@ -997,7 +1023,7 @@ constexpr size_t kTileLdsLimit = 128 * 1024;
 constexpr size_t kTileXLdsLimit = 64 * 1024;     // X through LDS: up to this many bytes of activations on top
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;
 
-bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int wave_cap = 8) {
+bool plan_tile_for(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int wave_cap, int per_cu) {
     const int n_steps = (int)(P / kStepCols);
     const int ranges = (n_steps + T - 1) / T;                 // column ranges of T steps
     // more than eight waves only where that saves a panel
@@ -1009,7 +1035,6 @@ bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int
     pl.threads = 64 * pl.W * pl.G;
     const int64_t tiles = (Q + kTileRows - 1) / kTileRows;
     const int cus = host::device_cus();
-    const int per_cu = host::env_int("QVB8_TILE_WGS_PER_CU", 1);
     int64_t target = (int64_t)cus * (per_cu > 0 ? per_cu : 1);
     int64_t tw = (tiles + target - 1) / target;
     tw = (tw + pl.G - 1) / pl.G * pl.G;
@@ -1039,13 +1064,43 @@ bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int
     pl.blocks = (unsigned)blocks;
     return true;
 }
+// Workgroups per CU the plan aims at: two where two fit a CU at the same time -- eight waves each (one panel), a kernel of
+// at most 128 registers per lane (`pair_fits`: the one-token-tile kernel that reads its operands from LDS step by step),
+// and LDS for both (`x_lds` = the activations' bytes on top of the plan's own) -- else one.  Two resident workgroups keep
+// more requests in flight and let one's epilogue overlap the other's stream (9B gate+up 19.5 -> 18.4 us); where only one
+// fits, twice the workgroups would just be a second round (27B down, twelve waves: 23.2 -> 26.7 us).
+bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int wave_cap = 8, bool pair_fits = false, size_t x_lds = 0) {
+    const int forced = host::env_int("QVB8_TILE_WGS_PER_CU", 0);
+    if (forced > 0) return plan_tile_for(NT, T, M, Q, P, pl, wave_cap, forced);
+    if (pair_fits && plan_tile_for(NT, T, M, Q, P, pl, wave_cap, 2) && pl.panels == 1 && pl.threads <= 512
+        && 2 * (pl.lds + x_lds) <= kLdsPerWorkgroup) return true;
+    return plan_tile_for(NT, T, M, Q, P, pl, wave_cap, 1);
+}
+
+// Whether the registers of this kernel let two workgroups of eight waves share a CU (asked of the runtime once per device).
+template <int NT, int T, bool BF, bool XC, int XP, bool PL>
+bool tile_pair_fits() {
+    if constexpr (!(XP > 0 && NT == 1)) return false;
+    static int known[64] = {0};                               // 0 not asked yet, 1 no, 2 yes
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    if (known[dev] == 0) {
+        int n = 0;
+        const bool ok = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)tile_kernel<NT, T, BF, XC, XP, PL>, 512, 0) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+        known[dev] = ok && n >= 2 ? 2 : 1;
+    }
+    return known[dev] == 2;
+}
 
 template <int NT, int T, bool BF, bool XC, int XP = 0, bool PL = false>
 int launch_tile(TileArgs& a, hipStream_t s) {
     TilePlan pl;
-    if (!plan_tile(NT, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<NT, T, BF, PL>() : 8))
+    const bool jit = tile_pair_fits<NT, T, BF, XC, XP, PL>();
+    const size_t x_lds = XP > 0 ? (size_t)a.M * (size_t)a.P * 2 + 64 : 0;
+    if (!plan_tile(NT, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<NT, T, BF, PL>() : 8, jit, x_lds))
         return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
-    if constexpr (XP > 0) pl.lds += (size_t)a.M * (size_t)a.P * 2;
+    pl.lds += x_lds;
     a.W = pl.W; a.G = pl.G; a.panels = pl.panels; a.TW = pl.TW;
     static bool attr[64] = {false};                           // per device: the attribute belongs to the device's copy of the kernel
     int dev = 0;
@@ -1068,11 +1123,11 @@ int launch_tile(TileArgs& a, hipStream_t s) {
 template <int T, bool BF, bool XC, bool PL = false>
 int launch_tile_rows16(TileArgs& a, hipStream_t s) {
     TilePlan pl;
-    if (!plan_tile(1, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<1, T, BF, PL>() : 8))
-        return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
     const size_t x_bytes = (size_t)a.M * (size_t)a.P * 2;
+    if (!plan_tile(1, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<1, T, BF, PL>() : 8, tile_pair_fits<1, T, BF, XC, 1, PL>(), x_bytes + 64))
+        return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
     const size_t per_thread = (x_bytes / 16 + pl.threads - 1) / pl.threads;
-    const bool fits = x_bytes <= kTileXLdsLimit && pl.lds + x_bytes <= kLdsPerWorkgroup && host::env_int("QVB8_TILE_X_LDS", 1) != 0;
+    const bool fits = x_bytes <= kTileXLdsLimit && pl.lds + x_bytes + 64 <= kLdsPerWorkgroup && host::env_int("QVB8_TILE_X_LDS", 1) != 0;
     if (fits && per_thread <= 1) return launch_tile<1, T, BF, XC, 1, PL>(a, s);
     if (fits && per_thread <= 4) return launch_tile<1, T, BF, XC, 4, PL>(a, s);
     if (fits && per_thread <= 8) return launch_tile<1, T, BF, XC, 8, PL>(a, s);
