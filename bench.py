@@ -63,10 +63,9 @@ def mma_flags(lin) -> int:
 def tile_traffic(units, n_launch):
     """Mean measured HBM bytes per launch of the step's launch mix (None when the counters' summary is not there)."""
     t = measured_traffic("tile_kernel_9b_decode_step_hbm_traffic.md", "tile_kernel")
-    cls = {"q+k+v": "q+k+v", "o": "o,gate+up", "gate+up": "o,gate+up", "down": "down"}
-    if any(cls.get(u["name"]) not in t for u in units):
+    if any(u["name"] not in t for u in units):
         return None
-    return round(sum(t[cls[u["name"]]] for u in units) / n_launch)
+    return round(sum(t[u["name"]] for u in units) / n_launch)
 
 
 def algorithmic_bytes(enc, M):
@@ -260,7 +259,7 @@ def bench_moe(args, dev):
                          "frac": round(gbs / HBM_PEAK_GBS, 4),
                          # HBM bytes of one layer's launches from hardware counters, where the summary holds this token count
                          "traffic": measured_traffic("moe_kernels_35b_a3b_layer_kernel_trace.md", "moe_layer").get("tokens=%d" % T),
-                         "kernel": ("qvb8::moe_one_kernel<4,false,..> + moe_one_kernel<6,true,..> (one layer = 2 launches)" if T <= 2 else
+                         "kernel": ("qvb8::moe_one_kernel<4,false,..> + moe_one_kernel<6,true,..> (one layer = 2 launches)" if T <= 6 else
                                     "qvb8::moe_plan_kernel + moe_walk_kernel<4,false,..> + moe_walk_kernel<6,true,..> + "
                                     "moe_combine_kernel (one layer = 4 launches)" if T <= 16 else
                                     "qvb8::moe_plan_kernel + moe_gemv_kernel<0> + moe_gemv_kernel<1> + moe_combine_kernel "
