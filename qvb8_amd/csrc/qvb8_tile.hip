@@ -106,6 +106,15 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
 // slots.  After one barrier the whole workgroup combines the column ranges of each row in a fixed order.
 // The kernel's arguments are 56 bytes of scalars (measured: every further 64 bytes of kernel arguments cost about a
 // microsecond per launch): fin follows loc, n_steps follows P, the small counts share one word.
+// the value lane l + O of the same row of sixteen lanes holds (zero past the row's end): DPP row_shl, no trip to LDS
+template <int O>
+__device__ __forceinline__ double row16_from(double v) {
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)b, 0x100 + O, 0xF, 0xF, true);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(b >> 32), 0x100 + O, 0xF, 0xF, true);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+
 // Waves a workgroup of this variant may have: twelve (three per SIMD) where the registers allow it -- long rows then take
 // fewer panels (12288 columns: two instead of three) --, else eight.
 template <int NT, int T, bool BF, bool PL> constexpr int tile_max_waves() { return (NT == 1 && T == 4 && PL && !BF) ? 12 : 8; }
@@ -482,7 +491,32 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
     // ---- combine the column ranges of each row in ascending order ----
     const int all_ranges = (a.n_steps + T - 1) / T;
     const int valid_ranges = all_ranges < ranges ? all_ranges : ranges;      // waves without any column never stored
-    for (int i = tid; i < tiles_here * kTileRows * a.M; i += blockDim.x) {
+    const int n_items = tiles_here * kTileRows * a.M;
+    const int n_waves_here = (int)blockDim.x >> 6;
+    if (n_items <= 4 * n_waves_here) {
+        // Few results (one token, a few tiles): a thread per (result, range) instead of a thread per result that walks
+        // the ranges one LDS trip after the other while every other wave idles.  Sixteen neighbouring lanes hold a result's
+        // terms (zero past the last range) and add them up as a fixed tree -- (0+8)+(4+12) ... -- in double; four results
+        // per wave and pass.
+        for (int first = wave * 4; first < n_items; first += n_waves_here * 4) {
+            const int i = first + (lane >> 4), w = lane & 15;
+            const bool item = i < n_items;
+            const int rl = item ? i / a.M : 0, t = item ? i - rl * a.M : 0;
+            const bool live = item && w < valid_ranges;
+            const int wr = live ? w : 0;
+            const float pv = part[((size_t)rl * ranges + wr) * MS + t], sv = sxs[wr * TM + t];
+            double dsum = live ? (double)pv : 0.0, xsum = live ? (double)sv : 0.0;
+            dsum += row16_from<8>(dsum); xsum += row16_from<8>(xsum);
+            dsum += row16_from<4>(dsum); xsum += row16_from<4>(xsum);
+            dsum += row16_from<2>(dsum); xsum += row16_from<2>(xsum);
+            dsum += row16_from<1>(dsum); xsum += row16_from<1>(xsum);
+            const uint4 f = s_fin[rl];
+            if (item && w == 0 && f.z < (uint32_t)a.Q)
+                store_y(a.Y, a.out_dt, (int64_t)t * a.Q + f.z, (float)((double)__uint_as_float(f.x) * dsum + (double)__uint_as_float(f.y) * xsum));
+        }
+        return;
+    }
+    for (int i = tid; i < n_items; i += blockDim.x) {
         const int rl = i / a.M, t = i - rl * a.M;
         const uint4 f = s_fin[rl];
         if (f.z >= (uint32_t)a.Q) continue;
