@@ -347,6 +347,7 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
     __shared__ float s_sx[kOneMaxTiles][kOneWaves];          // sum of the activations over the column range
     __shared__ float2 s_fin[kOneMaxTiles][16];               // tau_s, min_s of the tile's rows
     __shared__ int s_ok[kOneMaxTiles];                       // the slot's expert number is inside the stack
+    __shared__ float s_y[kOneMaxTiles][16];                  // a row tile's finished values
     __shared__ __align__(16) uint16_t s_x[kOneWaves][T * kStepCols];   // each wave's activations, narrowed (private to the wave)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -532,26 +533,31 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
     }
     __syncthreads();
 
-    auto row_value = [&](int i, int u) {                      // tau_s * sum(x * id) + min_s * sum(x), the ranges added in order
+    // tau_s * sum(x * id) + min_s * sum(x) of every row the workgroup worked on, the ranges added in order: a thread per
+    // row (not per output, which would leave one wave walking the slots' or the gate / up rows' ranges one LDS trip after
+    // the other), the values handed on through LDS
+    for (int o = tid; o < n_rt * 16; o += blockDim.x) {
+        const int i = o >> 4, u = o & 15;
         double d = 0.0, xs = 0.0;
         for (int w = 0; w < W; ++w) { d += (double)s_part[i][w][u]; xs += (double)s_sx[i][w]; }
         const float2 f = s_fin[i][u];
         const float y = (float)((double)f.x * d + (double)f.y * xs);
-        return s_ok[i] ? y : __builtin_nanf("");
-    };
+        s_y[i][u] = s_ok[i] ? y : __builtin_nanf("");
+    }
+    __syncthreads();
     if constexpr (DOWN) {
         if (tid < 16) {
             float acc = 0.f;
-            for (int j = 0; j < a.topk; ++j) acc = __builtin_fmaf(a.w[j], row_value(j, tid), acc);
+            for (int j = 0; j < a.topk; ++j) acc = __builtin_fmaf(a.w[j], s_y[j][tid], acc);
             store_from_f32<DT>(a.out, (int64_t)blockIdx.x * 16 + tid, acc);
         }
     } else {
         const int n_ut = n_rt / RT;
         for (int o = tid; o < n_ut * 16; o += blockDim.x) {
             const int lut = o >> 4, u = o & 15, i0 = lut * RT;
-            const float y0 = row_value(i0, u);
+            const float y0 = s_y[i0][u];
             float h;
-            if (a.gated) h = (y0 / (1.0f + __expf(-y0))) * row_value(i0 + 1, u);
+            if (a.gated) h = (y0 / (1.0f + __expf(-y0))) * s_y[i0 + 1][u];
             else { const float p = fmaxf(y0, 0.f); h = y0 != y0 ? y0 : p * p; }
             const int ut = ut_first + lut;
             reinterpret_cast<uint16_t*>(a.out)[(size_t)(ut / UT) * a.units + (ut % UT) * 16 + u] = (uint16_t)sat_half_bits(h);
