@@ -260,3 +260,27 @@ def test_plane_tiles_seeded_shapes(seed):
     from qvb8_amd import ext_qvb8 as ext
     dense = ext.decode_f32(tiled.ids, tiled.min_s, tiled.nbits, tiled.bit_off, P, tiled.tau_s, tiled.esc_idx, tiled.esc_vals)
     assert np.array_equal(dense.cpu().numpy().view(np.uint32), Wr.astype(np.float32).view(np.uint32))
+
+
+@pytest.mark.parametrize("P,M", [(6144, 1), (6144, 8), (12288, 1), (12288, 3)])
+def test_plane_tiles_long_rows_agree_with_the_oracle(P, M):
+    """Rows beyond 4096 columns: with the rows in planes a workgroup may have twelve waves, so a row's partial sums are
+    grouped differently than with the rows back to back and the two products may differ in the last bit -- each of them
+    stays inside the oracle's bound, and the restored weight is the same bit for bit."""
+    Q = 72
+    d = H.mixed_width_pack(Q, P, [6] * 40 + [7] * 32, seed=P + M)
+    d["tau_s"] = d["tau_s"] * (1.0 / 64)
+    a = H.to_device_args(d, DEV)
+    Wr = O.reconstruct(d["min_s"], d["tau_s"], d["ids_dense"], d["esc_idx"], d["esc_vals"])
+    x = torch.randn(M, P, generator=torch.Generator().manual_seed(P + M)).to(torch.bfloat16).to(DEV)
+    xs = O.sat_half(x.float().cpu().numpy())
+    for planes in (False, True):
+        m = QVBandLinearV8(min_s=a[1].clone(), nbits=a[2].clone(), bit_off=a[3].clone(), ids=a[0].clone(), Q=Q, P=P, tau_s=a[5].clone(),
+                           esc_idx=a[6], esc_vals=a[7])
+        m.plane_tiles = planes
+        y = m(x)
+        assert m._planes == planes
+        _close(y, O.linear_f64(xs, Wr), Wr, xs, torch.bfloat16)
+        from qvb8_amd import ext_qvb8 as ext
+        dense = ext.decode_f32(m.ids, m.min_s, m.nbits, m.bit_off, P, m.tau_s, m.esc_idx, m.esc_vals)
+        assert np.array_equal(dense.cpu().numpy().view(np.uint32), Wr.astype(np.float32).view(np.uint32))

@@ -262,11 +262,12 @@ def test_moe_few_tokens_rows_longer_than_2048_columns(monkeypatch):
 
 
 def test_moe_config4_all_128_experts():
-    """The 35B-A3B-shape layer with all 128 experts resident (hidden 2048, gate/up 2048->768, top-8): 1 and 8 tokens."""
+    """The 35B-A3B-shape layer with all 128 experts resident (hidden 2048, gate/up 2048->768, top-8): 1, 4 and 6 tokens (one
+    grid row per token) and 8 (the grouped walk)."""
     E, hidden, inter = 128, 2048, 768
     gu, dn, Wgu, Wdn = _experts(E, hidden, inter, 2e-3, seed=7000)
     mod = QVBandExpertsV8(gu, dn, num_experts=E)
-    for T in (1, 8):
+    for T in (1, 4, 6, 8):
         idx, w = _route(T, E, 8, seed=30 + T)
         x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(torch.bfloat16)
         out = mod(x.to(DEV), torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV))
