@@ -165,11 +165,16 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
         for (int i = 0; i < XP; ++i) xg[i] = xsrc[min(tid + i * (int)blockDim.x, x_pieces - 1)];
         __builtin_amdgcn_sched_barrier(0);                     // these requests stay where they are: ahead of everything
     }
-    // The workgroup's local tile lt is global tile lt * gridDim.x + blockIdx.x: at any moment the workgroups of the
-    // grid read neighbouring tiles, so the whole chip walks through memory together (spread over all channels).
+    // The workgroup's local tile lt is global tile lt * gridDim.x + vb (vb: the workgroup's number, see below): at any moment the
+    // workgroups of the grid read neighbouring tiles, so the whole chip walks through memory together (spread over all channels).
     const int total_tiles = (a.Q + kTileRows - 1) / kTileRows;
-    const int tiles_here = (int)blockIdx.x < total_tiles ? min(a.TW, (total_tiles - 1 - (int)blockIdx.x) / (int)gridDim.x + 1) : 0;
-    auto local_to_pos = [&](int lrow) { return ((lrow >> 4) * (int)gridDim.x + (int)blockIdx.x) * kTileRows + (lrow & 15); };
+    // Workgroup b runs on XCD b % 8 (workgroups are dealt to the eight XCDs in turn): the workgroups of one XCD take
+    // neighbouring tiles, so each XCD's L2 and its path to memory see one contiguous eighth of the window the chip is
+    // reading (measured: 0.4 % of the 9B decode step, o and q+k+v 0.05-0.1 us each; nothing on the long launches).
+    const int nblk = (int)gridDim.x;
+    const int vb = (nblk & 7) == 0 ? ((int)blockIdx.x & 7) * (nblk >> 3) + ((int)blockIdx.x >> 3) : (int)blockIdx.x;
+    const int tiles_here = vb < total_tiles ? min(a.TW, (total_tiles - 1 - vb) / nblk + 1) : 0;
+    auto local_to_pos = [&](int lrow) { return ((lrow >> 4) * nblk + vb) * kTileRows + (lrow & 15); };
     const int n_tiles = tiles_here > g ? (tiles_here - g + a.G - 1) / a.G : 0;    // tiles of this wave's group
 
     // ---- the records of this wave's rows into its own LDS copy (a wave's LDS accesses stay in order, so the copy
