@@ -52,9 +52,9 @@ enum qvb8_status {
 
 /* Library identification: ABI version, bumped on any signature change or new entry point (3: row lookup, attention over
  * the banded KV cache, query preparation; 4: qvb8_moe_experts_static; 5: result-type flags of qvb8_mma; 6: rows stored
- * in planes, QVB8_MMA_PLANES).  A binding compares the loaded library's answer
+ * in planes, QVB8_MMA_PLANES; 7: qvb8_mlp).  A binding compares the loaded library's answer
  * with the QVB8_ABI_VERSION it was written for before it makes any other call. */
-#define QVB8_ABI_VERSION 6
+#define QVB8_ABI_VERSION 7
 int qvb8_abi_version(void);
 /* Message of the calling thread's most recent failure ("" if none). Valid until that thread's next call. */
 const char* qvb8_last_error(void);
@@ -194,6 +194,43 @@ int qvb8_mma(const void* X, int x_dtype, int64_t M,
  * machine before any byte moves, the floor under every per-launch figure of the benchmark (bench.py --workload floor).
  * No counterpart in the reference. */
 int qvb8_launch_probe(int64_t blocks, int64_t threads, int64_t lds_bytes, void* stream);
+
+/* ---- the MLP of a decoder layer in ONE launch (decode: 1..4 rows) ---------------------------------------------- */
+
+/* Y = down( act(gate(x)) * up(x) ) for 1 <= M <= QVB8_MLP_MAX_ROWS rows of X, as one kernel: the gate+up product, the
+ * activation and the down product run in one grid of one workgroup per CU (all resident at once), and H = act(gate) * up
+ * is handed from its producers to the down rows' workgroups INSIDE the grid, through `workspace`, while the down
+ * weight's first ids are already on their way.  Launched separately the two products each pay a launch's fixed cost;
+ * this call pays it once.
+ * Values are those of the separate calls and the caller's elementwise code between them: gate and up results rounded to
+ * `mid_dtype` (QVB8_F32 = not rounded), SiLU computed in fp32 and rounded to it, the product rounded to it, then narrowed
+ * to saturated fp16 (what qvb8_mma's QVB8_MMA_SATURATE_X does to the down product's input); Y rounded to `y_dtype`.
+ * X: (M, hidden) fp16, or bf16 narrowed like QVB8_MMA_SATURATE_X; 16-byte aligned.
+ * Both weights: rows stored in planes in position order with a row layout (see qvb8_mma; widths 4..8, every run of one
+ * width whole tiles, no escapes), row records from qvb8_mma_prepare for the same order.  gate+up is ONE pack of 2 * inter
+ * rows (rows 0..inter-1 gate, the rest up) whose position order goes unit by unit: positions 32 u .. 32 u + 15 hold 16
+ * gate rows, 32 u + 16 .. 32 u + 31 the up rows of the same outputs (position 32 u + 16 + r is row inter + j when position
+ * 32 u + r is row j; a pair that breaks this gives NaN for that output).  down: out_features rows of inter columns.
+ * hidden % 128 == 0, inter % 128 == 0, out_features % 16 == 0; anything else: QVB8_ERR_UNSUPPORTED (call the products
+ * separately).
+ * `workspace`: qvb8_mlp_workspace_bytes(inter) bytes, 16-byte aligned, ZEROED ONCE by the caller before its first use and
+ * then left to the library; it carries the state of the hand-over from call to call, so calls that share it must not
+ * overlap (one per layer, or one per stream).  Its first words: [0] workgroups of the running call that have taken H,
+ * [1] error, sticky: nonzero once a call's bounded wait for H ran out (QVB8_MLP_WAIT_US microseconds, default 20000;
+ * that call's Y is NaN) -- it can only run out when the grid is not resident as a whole, e.g. while other kernels hold
+ * CUs for that long.
+ * `act`: QVB8_MLP_SILU_GATED.  QVB8_MLP_TEST_STALE_TAG ORed in makes the producers label H as another call's, so that the
+ * wait runs out: for tests of that path only.
+ * No single counterpart in the reference, which launches the products separately and removes the launch cost from the host's
+ * side by replaying the MLP as a graph (install_mlp_graphs  formats/qvb8/moe_graph.py:145-178); the products are
+ * qvb8_mma_multi_forward / the GEMV of qvb8_cuda.cu:1059-1166, 2566-2671. */
+#define QVB8_MLP_MAX_ROWS 4
+enum qvb8_mlp_act { QVB8_MLP_SILU_GATED = 0, QVB8_MLP_TEST_STALE_TAG = 0x100 };
+int64_t qvb8_mlp_workspace_bytes(int64_t inter);
+int qvb8_mlp(const void* X, int x_dtype, int64_t M, int64_t hidden, int64_t inter, int64_t out_features,
+             const uint8_t* gu_ids, int64_t gu_ids_bytes, const uint64_t* gu_rowinfo, const qvb8_mma_layout* gu_layout,
+             const uint8_t* dn_ids, int64_t dn_ids_bytes, const uint64_t* dn_rowinfo, const qvb8_mma_layout* dn_layout,
+             int act, int mid_dtype, void* Y, int y_dtype, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- routed MoE expert stack (decode: a few tokens, top-k experts each) ---------------------------------------- */
 

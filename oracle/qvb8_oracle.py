@@ -449,6 +449,38 @@ def silu(v):
     return v / (1.0 + np.exp(-v))
 
 
+def round_to(v, dtype: str) -> np.ndarray:
+    """v (float64 or float32) rounded once, to nearest even, to "fp32" / "fp16" / "bf16", returned as float32."""
+    v32 = np.asarray(v, np.float64).astype(np.float32)
+    if dtype == "fp16":
+        return narrow_fp16(v32)
+    if dtype == "bf16":
+        return narrow_bf16(v32)
+    return v32
+
+
+def swiglu(gate, up, dtype: str) -> np.ndarray:
+    """silu(gate) * up as a model in `dtype` computes it: silu rounded to `dtype` before the multiply, the product rounded
+    again (decode/fused_pointwise.py:60-67 `_swiglu_k`: "silu() returns the input dtype"; the eager code it replaces is
+    `act_fn(gate_proj(x)) * up_proj(x)`, :143-148).  gate and up are taken as already holding values of `dtype`."""
+    g = np.asarray(gate, np.float32).astype(np.float64)
+    s = round_to(g / (1.0 + np.exp(-g)), dtype).astype(np.float64)
+    return round_to(s * np.asarray(up, np.float32).astype(np.float64), dtype)
+
+
+def mlp_reference(x, W_gate, W_up, W_down, dtype: str):
+    """down_proj(act_fn(gate_proj(x)) * up_proj(x)) with packed linears, as the reference runs a dense MLP at decode
+    (decode/fused_pointwise.py:194-204; each product = X saturated to fp16 times the fp32 band value, module.py:455-464,
+    its result cast to the caller's `dtype`).  Products in float64.  Returns (y, h): y rounded to `dtype`, h = the
+    intermediate in `dtype` (before the down product narrows it to saturated fp16)."""
+    xs = sat_half(np.asarray(x, np.float32))
+    g = round_to(linear_f64(xs, W_gate), dtype)
+    u = round_to(linear_f64(xs, W_up), dtype)
+    h = swiglu(g, u, dtype)
+    y = linear_f64(sat_half(h), W_down)
+    return round_to(y, dtype), h
+
+
 def moe_reference(x, top_idx, top_w, W_gu: list, W_dn: list, act="silu") -> np.ndarray:
     """Per-token loop over the routed experts (backends_experts.py:228-272 semantics;
     fused kernel: qvb8_cuda.cu:937-992): h = act(gate)*up with gate = first half of the

@@ -12,13 +12,13 @@ import torch
 from .common.errors import NativeLibraryError
 
 _LIB = None
-EXPECTED_ABI = 6            # QVB8_ABI_VERSION of include/qvb8_amd.h that the argument lists below were written for
+EXPECTED_ABI = 7            # QVB8_ABI_VERSION of include/qvb8_amd.h that the argument lists below were written for
 F32, F16, BF16 = 0, 1, 2
 _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 # every symbol include/qvb8_amd.h declares
 SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_lookup_rows", "qvb8_scatter_escapes", "qvb8_certify",
-           "qvb8_sat_half", "qvb8_scale_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma", "qvb8_launch_probe",
+           "qvb8_sat_half", "qvb8_scale_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma", "qvb8_launch_probe", "qvb8_mlp_workspace_bytes", "qvb8_mlp",
            "qvb8_moe_workspace_bytes", "qvb8_moe_experts", "qvb8_moe_experts_static",
            "qvb8r_decode", "qvb8r_decode_blocks", "qvb8r_gemv_workspace_bytes", "qvb8r_gemv", "qvb8r_fix_escapes", "qvb8_attn_fwd", "qvb8_attn_combine")
 
@@ -72,6 +72,9 @@ def load(build_if_missing: bool = True):
     lib.qvb8_mma_prepare.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, vp]
     lib.qvb8_mma.argtypes = [vp, i32, i64, vp, i64, vp, vp, vp, vp, i64, i64, vp, vp, i64, vp, vp, vp, i32, vp, vp, i64, vp]
     lib.qvb8_launch_probe.argtypes = [i64, i64, i64, vp]
+    lib.qvb8_mlp_workspace_bytes.argtypes = [i64]
+    lib.qvb8_mlp_workspace_bytes.restype = i64
+    lib.qvb8_mlp.argtypes = [vp, i32, i64, i64, i64, i64, vp, i64, vp, vp, vp, i64, vp, vp, i32, i32, vp, i32, vp, i64, vp]
     lib.qvb8_moe_workspace_bytes.argtypes = [i64] * 6
     lib.qvb8_moe_workspace_bytes.restype = i64
     lib.qvb8_moe_experts.argtypes = ([vp, i32, i64, vp, vp, i64, i64] + [vp, i64, vp, vp, vp, vp, i64, i64] * 2

@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libqvb8_amd.so")
-SOURCES = ["qvb8_kernels.hip", "qvb8_tile.hip", "qvb8_moe.hip", "qvb8r.hip", "qvb8_attn.hip"]
+SOURCES = ["qvb8_kernels.hip", "qvb8_tile.hip", "qvb8_mlp.hip", "qvb8_moe.hip", "qvb8r.hip", "qvb8_attn.hip"]
 ARCH = "gfx950"
 # packed-fp32 VALU forms are switched off for every device compile of this library
 DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

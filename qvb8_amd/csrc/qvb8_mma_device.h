@@ -107,4 +107,21 @@ __device__ __forceinline__ void decode_slice(const uint4& lo, const uint4& hi, v
     for (int p = 0; p < 16; ++p) b[p / 4][p % 4] = and_or3(e[p], m, bias);
 }
 
+// the value lane l + O of the same row of sixteen lanes holds (zero past the row's end): DPP row_shl, no trip to LDS
+template <int O>
+__device__ __forceinline__ double row16_from(double v) {
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)b, 0x100 + O, 0xF, 0xF, true);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(b >> 32), 0x100 + O, 0xF, 0xF, true);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+// the sum of a value over the sixteen lanes of a row, as a fixed tree (0+8)+(4+12)...: valid in the row's first lane
+__device__ __forceinline__ double row16_sum(double v) {
+    v += row16_from<8>(v);
+    v += row16_from<4>(v);
+    v += row16_from<2>(v);
+    v += row16_from<1>(v);
+    return v;
+}
+
 }  // namespace qvb8

@@ -106,15 +106,6 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
 // slots.  After one barrier the whole workgroup combines the column ranges of each row in a fixed order.
 // The kernel's arguments are 56 bytes of scalars (measured: every further 64 bytes of kernel arguments cost about a
 // microsecond per launch): fin follows loc, n_steps follows P, the small counts share one word.
-// the value lane l + O of the same row of sixteen lanes holds (zero past the row's end): DPP row_shl, no trip to LDS
-template <int O>
-__device__ __forceinline__ double row16_from(double v) {
-    const uint64_t b = __builtin_bit_cast(uint64_t, v);
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)b, 0x100 + O, 0xF, 0xF, true);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(b >> 32), 0x100 + O, 0xF, 0xF, true);
-    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
-}
-
 // Waves a workgroup of this variant may have: twelve (three per SIMD) where the registers allow it -- long rows then take
 // fewer panels (12288 columns: two instead of three) --, else eight.
 template <int NT, int T, bool BF, bool PL> constexpr int tile_max_waves() { return (NT == 1 && T == 4 && PL && !BF) ? 12 : 8; }

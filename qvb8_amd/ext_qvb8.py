@@ -476,6 +476,45 @@ def mma_tiles(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals
     return Y
 
 
+MLP_MAX_ROWS = 4                                  # QVB8_MLP_MAX_ROWS
+MLP_SILU_GATED, MLP_TEST_STALE_TAG = 0, 0x100     # qvb8_mlp_act
+
+
+def mlp_workspace(inter: int, device) -> torch.Tensor:
+    """The workspace of mlp_fused for an MLP of `inter` hidden units: zeroed here, once; afterwards the library's (it carries
+    the hand-over's state from call to call, so calls that share it must not overlap).  Words 0 and 1 (int32 view): workgroups
+    of a running call that have taken H, and the sticky error word."""
+    lib = _lib.load()
+    return torch.zeros(int(lib.qvb8_mlp_workspace_bytes(int(inter))), dtype=torch.uint8, device=device)
+
+
+def mlp_fused(X, gu_ids, gu_rowinfo, gu_layout, dn_ids, dn_rowinfo, dn_layout, hidden, inter, out_features, workspace,
+              mid_dtype=None, out_dtype=None, act=MLP_SILU_GATED):
+    """down(silu(gate(x)) * up(x)) for 1..4 rows of X as ONE launch (qvb8_mlp): the gate+up pack in unit order and the
+    down pack, both stored in planes with a row layout (see formats/qvb8/mlp.py, which builds them), `workspace` from
+    mlp_workspace.  `mid_dtype`: the type the values between the products are rounded to (X's by default), `out_dtype`
+    the result's (X's by default).  Raises RuntimeError for what the kernel does not cover: callers fall back to the
+    separate products."""
+    lib = _lib.load()
+    _lib.require_cuda(X, gu_ids, gu_rowinfo, dn_ids, dn_rowinfo, workspace)
+    if X.dim() != 2 or X.shape[1] != int(hidden):
+        raise RuntimeError(f"X must be (M, {int(hidden)})")
+    if X.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("qvb8 mlp: X must be fp16 or bf16")
+    M = X.shape[0]
+    mid_dtype = X.dtype if mid_dtype is None else mid_dtype
+    out_dtype = X.dtype if out_dtype is None else out_dtype
+    Xc = X.contiguous()
+    with torch.cuda.device(Xc.device):
+        Y = torch.empty((M, int(out_features)), dtype=out_dtype, device=Xc.device)
+        _lib._check(lib.qvb8_mlp(_lib.ptr(Xc), _lib.dtype_code(Xc.dtype), M, int(hidden), int(inter), int(out_features),
+                                 gu_ids.data_ptr(), gu_ids.numel(), gu_rowinfo.data_ptr(), ctypes.addressof(gu_layout),
+                                 dn_ids.data_ptr(), dn_ids.numel(), dn_rowinfo.data_ptr(), ctypes.addressof(dn_layout),
+                                 int(act), _lib.dtype_code(mid_dtype), Y.data_ptr(), _lib.dtype_code(out_dtype),
+                                 workspace.data_ptr(), workspace.numel(), _lib.stream_of(Xc)), lib)
+    return Y
+
+
 def mma_multi(X, ids, min_s, row_nbits, row_bit_off, P, tau_s, esc_idx, esc_vals, perm, tile_nb,
               bf16=False, esc_starts=None, general=-1):
     """QVB8 tensor-core multi-row product (M <= 48), bf16.  fp16 mode (bf16=False): X saturated to fp16;

@@ -234,8 +234,10 @@ class QVBandLinearV8(nn.Module):
         if self.ids.is_cuda and self.in_features % 128 == 0 and self.ids.data_ptr() % 4 == 0 and self.out_features > 0:
             nb = self.nbits.to(torch.int16)
             if 1 <= int(nb.min()) and int(nb.max()) <= 14:
-                perm = torch.argsort(nb, stable=True).to(torch.int32).contiguous()
                 layout = self.__dict__.get("_sorted_layout")                  # sorted before (the buffers have moved since)
+                stored = self.__dict__.get("_stored_perm") if layout is not None else None
+                # the order the rows were stored in, when a caller chose it (store_in_order); else by width
+                perm = stored.to(self.ids.device) if stored is not None else torch.argsort(nb, stable=True).to(torch.int32).contiguous()
                 row_bytes = int((self.nbits.to(torch.int64) * self.in_features).sum().item()) // 8
                 if layout is None and self.sort_rows and 2 * row_bytes >= self.ids.numel():   # not for a small view into a shared stack
                     planes = self.plane_tiles and os.environ.get("QVB8_PLANES", "1") != "0"
@@ -257,6 +259,36 @@ class QVBandLinearV8(nn.Module):
                 order = (perm, rowinfo, layout)
         self._mma_cache = order
         return order
+
+    def store_in_order(self, perm: torch.Tensor, new_nbits: torch.Tensor | None = None) -> bool:
+        """Stores the rows once more, in the position order `perm` (int32, position -> row) instead of sorted by width,
+        row q in fields of new_nbits[q] >= nbits[q] bits (its ids, and so every value, unchanged), whole tiles in planes;
+        along `perm` the widths must not decrease and take at most three values.  For callers whose kernel wants rows that
+        belong together side by side (the MLP's gate and up rows of the same outputs).  Every other path of this module
+        keeps working on the new bytes.  False, and nothing changed, when the pack cannot be stored that way."""
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("QVBandLinearV8.store_in_order: not inside a graph capture")
+        P = self.in_features
+        if not self.ids.is_cuda or P % 128 != 0 or self.esc_idx.numel() or self.esc_idx_bf16.numel():
+            return False
+        ids, bit_off, nbits = self.ids, self.bit_off, self.nbits
+        if new_nbits is not None and not bool((new_nbits == nbits).all()):
+            packed = ext.repack_rows(ids, nbits, bit_off, P, new_nbits)
+            if packed is None:
+                return False
+            ids, bit_off = packed
+            nbits = new_nbits.to(torch.uint8)
+        perm = perm.to(device=ids.device, dtype=torch.int32).contiguous()
+        srt = ext.sort_rows_by_width(ids, nbits, bit_off, P, perm, planes=True)
+        if srt is None:
+            return False
+        self.ids, self.bit_off, layout = srt
+        self.nbits = nbits
+        self._sorted_layout, self._stored_perm = layout, perm
+        self._planes = ext.rows_in_planes(self.bit_off)
+        rowinfo = ext.mma_prepare(self.nbits, self.bit_off, self.tau_s, self.min_s, P, self.ids.numel(), perm)
+        self._mma_cache = (perm, rowinfo, layout)
+        return True
 
     def prepare(self) -> "QVBandLinearV8":
         """Builds the per-weight launch data now (load time) instead of on the first forward; returns self."""
