@@ -9,7 +9,7 @@ HIP graph and replayed; `value` is the algorithmic bytes of a step (packed ids +
 in and out) divided by the measured time per step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--no-cpu] [--no-fuse] [--no-sort] [--copy-probe]
-                    [--workload decode9b|smallm|moe|qvb8r|lmhead|embed] [--tokens T]
+                    [--workload decode9b|smallm|moe|qvb8r|lmhead|embed|attn|floor|mlp] [--tokens T]
 
 Prints ONE JSON line.  `roofline` covers the dominant kernel (the tile kernel, every launch of the step):
 algorithmic bytes per launch / average launch time, timed with HIP events on the launch stream over the timed region.
@@ -513,6 +513,75 @@ def bench_attn(args, dev):
             "cpu_baseline": None}
 
 
+def bench_mlp(args, dev):
+    """One decoder layer's MLP at decode, both ways: qvb8_mlp (gate+up, SiLU, down in ONE launch, the hand-over inside the
+    grid) against the two separate qvb8_mma launches on the same bytes.  `--layers` distinct MLPs of the `--model` shapes
+    (9b: hidden 4096, inter 12288; 27b: 5120 / 17408) per graph replay; `value` is the one-launch path's GB/s on the packed
+    bytes, config carries microseconds per layer of both."""
+    import torch
+    from qvb8_amd import _lib
+    from qvb8_amd.formats.qvb8 import pack as PK
+    from qvb8_amd.formats.qvb8.mlp import QVBandMLPV8
+    from qvb8_amd.formats.qvb8.module import QVBandLinearV8
+    lib = _lib.load()
+    hidden, inter = (5120, 17408) if args.model == "27b" else (4096, 12288)
+    M = max(1, min(4, args.tokens))
+    mlps = []
+    for li in range(args.layers):
+        mods = []
+        for pi, (Q, P) in enumerate(((inter, hidden), (inter, hidden), (hidden, inter))):
+            g = torch.Generator(device=dev).manual_seed(1000 * li + pi)
+            W = (0.02 * torch.randn(Q, P, device=dev, generator=g)).to(torch.bfloat16)
+            mods.append(QVBandLinearV8.from_encoded(PK.encode_tensor(W, TAU, restore="fp16")))
+            del W
+        m = QVBandMLPV8(*mods)
+        if not m.fused_ready:
+            raise RuntimeError("bench mlp: the one-launch kernel cannot read this pack")
+        mlps.append(m)
+    x = torch.randn(M, hidden, device=dev, generator=torch.Generator(device=dev).manual_seed(7)).to(torch.bfloat16)
+    xh = torch.randn(M, inter, device=dev, generator=torch.Generator(device=dev).manual_seed(8)).to(torch.bfloat16)
+    Y = torch.empty(M, hidden, dtype=torch.bfloat16, device=dev)
+    Ygu = torch.empty(M, 2 * inter, dtype=torch.bfloat16, device=dev)
+    nbytes = sum(m.gate_up.ids.numel() + m.down.ids.numel() + 17 * (2 * inter + hidden) + 2 * M * (2 * hidden + inter) for m in mlps)
+
+    def one_launch():
+        s = torch.cuda.current_stream().cuda_stream
+        for m in mlps:
+            rc = lib.qvb8_mlp(ctypes.addressof(m._plan), x.data_ptr(), _lib.BF16, M, 0, _lib.BF16, Y.data_ptr(), _lib.BF16, m._ws.data_ptr(), s)
+            if rc != 0:
+                raise RuntimeError(lib.qvb8_last_error().decode())
+
+    def product(lin, xin, out):
+        perm, rowinfo, layout = lin._mma_order()
+        rc = lib.qvb8_mma(xin.data_ptr(), _lib.BF16, M, lin.ids.data_ptr(), lin.ids.numel(), lin.min_s.data_ptr(), lin.tau_s.data_ptr(),
+                          lin.nbits.data_ptr(), lin.bit_off.data_ptr(), lin.out_features, lin.in_features, None, None, 0,
+                          perm.data_ptr(), rowinfo.data_ptr(), ctypes.addressof(layout), 1 | 4 | 8, out.data_ptr(), None, 0,
+                          torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError(lib.qvb8_last_error().decode())
+
+    def separate():
+        for m in mlps:
+            product(m.gate_up, x, Ygu)
+            product(m.down, xh, Y)
+    fused_ms = min(max(time_graph(one_launch, args.steps, args.warmup)) for _ in range(2))
+    sep_ms = min(max(time_graph(separate, args.steps, args.warmup)) for _ in range(2))
+    if any(m.error_raised() for m in mlps):
+        raise RuntimeError("bench mlp: a wait for H ran out")
+    gbs = nbytes / (fused_ms * 1e-3) / 1e9
+    return {"metric": "decoder-layer MLP at decode in one launch (gate+up, SiLU, down): GB/s on packed bytes, 1 MI355X",
+            "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(fused_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16 activations narrowed to fp16, ids as exact fp16 operands, fp32 accumulate", "data": "synthetic",
+            "config": {"workload": "MLP hidden %d / inter %d, QVB8 tau=1e-3, M=%d, %d layers per replay" % (hidden, inter, M, args.layers),
+                       "bytes_per_step": nbytes, "one_launch_us_per_layer": round(fused_ms * 1e3 / args.layers, 2),
+                       "two_launches_us_per_layer": round(sep_ms * 1e3 / args.layers, 2)},
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "qvb8::mlp_kernel<4,3,1,true>",
+                         "bytes_per_launch": nbytes // args.layers, "launch_us": round(fused_ms * 1e3 / args.layers, 3)},
+            "cpu_baseline": None}
+
+
 def bench_floor(args, dev):
     """What a launch costs on this machine.  (1) A graph of 128 launches of a kernel with the tile kernel's launch shape
     (256 workgroups x 512 threads, 40 KB of LDS, the same scalar arguments) that does nothing: microseconds per graph
@@ -658,11 +727,12 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=None, help="layers of distinct packs (default 32; moe 4; qvb8r 2)")
-    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead", "embed", "attn", "floor"), default="decode9b",
+    ap.add_argument("--workload", choices=("decode9b", "smallm", "moe", "qvb8r", "lmhead", "embed", "attn", "floor", "mlp"), default="decode9b",
                     help="decode9b (default, the headline metric): 9B-shape decode step; moe: 35B-A3B-shape expert stack; "
                          "qvb8r: entropy-coded 27B-class FFN shapes; smallm: the 9B projections with --tokens rows (16, 64, 256); "
                          "lmhead / embed: the 248320 x 5120 vocabulary table; attn: decode-step attention over a banded KV cache; "
-                         "floor: what a launch costs (empty-kernel graph, tile kernel time against bytes)")
+                         "floor: what a launch costs (empty-kernel graph, tile kernel time against bytes); "
+                         "mlp: a layer's MLP in one launch (qvb8_mlp) against its two separate launches")
     ap.add_argument("--context", type=int, default=32768, help="keys in the cache of the attn workload")
     ap.add_argument("--head-major", action="store_true",
                     help="attn workload: ids stored (kv heads, keys, channels) instead of the reference's (keys, kv heads, channels)")
@@ -697,9 +767,9 @@ def main():
     torch.cuda.set_device(dev)
     lib = _lib.load()                                       # raises when the HIP library is missing: no fallback
     if args.layers is None:
-        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 1, "lmhead": 1, "embed": 1, "attn": 16, "floor": 1}[args.workload]
+        args.layers = {"decode9b": 32, "smallm": 8, "moe": 4, "qvb8r": 1, "lmhead": 1, "embed": 1, "attn": 16, "floor": 1, "mlp": 16}[args.workload]
     if args.workload != "decode9b":
-        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead, "embed": bench_embed, "attn": bench_attn, "floor": bench_floor}[args.workload]
+        fn = {"moe": bench_moe, "qvb8r": bench_qvb8r, "smallm": bench_smallm, "lmhead": bench_lmhead, "embed": bench_embed, "attn": bench_attn, "floor": bench_floor, "mlp": bench_mlp}[args.workload]
         print(json.dumps(fn(args, dev)))
         return 0
     if args.no_sort:

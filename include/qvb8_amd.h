@@ -205,32 +205,42 @@ int qvb8_launch_probe(int64_t blocks, int64_t threads, int64_t lds_bytes, void* 
  * Values are those of the separate calls and the caller's elementwise code between them: gate and up results rounded to
  * `mid_dtype` (QVB8_F32 = not rounded), SiLU computed in fp32 and rounded to it, the product rounded to it, then narrowed
  * to saturated fp16 (what qvb8_mma's QVB8_MMA_SATURATE_X does to the down product's input); Y rounded to `y_dtype`.
- * X: (M, hidden) fp16, or bf16 narrowed like QVB8_MMA_SATURATE_X; 16-byte aligned.
- * Both weights: rows stored in planes in position order with a row layout (see qvb8_mma; widths 4..8, every run of one
- * width whole tiles, no escapes), row records from qvb8_mma_prepare for the same order.  gate+up is ONE pack of 2 * inter
- * rows (rows 0..inter-1 gate, the rest up) whose position order goes unit by unit: positions 32 u .. 32 u + 15 hold 16
- * gate rows, 32 u + 16 .. 32 u + 31 the up rows of the same outputs (position 32 u + 16 + r is row inter + j when position
- * 32 u + r is row j; a pair that breaks this gives NaN for that output).  down: out_features rows of inter columns.
+ *
+ * qvb8_mlp_init, once per block (at load): checks the two weights, fills `plan` (a host struct the caller keeps) and
+ * launches a small kernel that zeroes `workspace` and writes the block's description into it.  Both weights: rows stored
+ * in planes in position order with a row layout (see qvb8_mma; widths 4..8, every run of one width whole tiles, no
+ * escapes), row records from qvb8_mma_prepare for the same order.  gate+up is ONE pack of 2 * inter rows (rows
+ * 0..inter-1 gate, the rest up) whose position order goes unit by unit: positions 32 u .. 32 u + 15 hold 16 gate rows,
+ * 32 u + 16 .. 32 u + 31 the up rows of the same outputs (position 32 u + 16 + r is row inter + j when position 32 u + r is
+ * row j; a pair that breaks this gives NaN for that output).  down: out_features rows of inter columns.
  * hidden % 128 == 0, inter % 128 == 0, out_features % 16 == 0; anything else: QVB8_ERR_UNSUPPORTED (call the products
- * separately).
- * `workspace`: qvb8_mlp_workspace_bytes(inter) bytes, 16-byte aligned, ZEROED ONCE by the caller before its first use and
- * then left to the library; it carries the state of the hand-over from call to call, so calls that share it must not
- * overlap (one per layer, or one per stream).  Its first words: [0] workgroups of the running call that have taken H,
- * [1] error, sticky: nonzero once a call's bounded wait for H ran out (QVB8_MLP_WAIT_US microseconds, default 20000;
- * that call's Y is NaN) -- it can only run out when the grid is not resident as a whole, e.g. while other kernels hold
- * CUs for that long.
- * `act`: QVB8_MLP_SILU_GATED.  QVB8_MLP_TEST_STALE_TAG ORed in makes the producers label H as another call's, so that the
- * wait runs out: for tests of that path only.
- * No single counterpart in the reference, which launches the products separately and removes the launch cost from the host's
- * side by replaying the MLP as a graph (install_mlp_graphs  formats/qvb8/moe_graph.py:145-178); the products are
- * qvb8_mma_multi_forward / the GEMV of qvb8_cuda.cu:1059-1166, 2566-2671. */
+ * separately).  The weights' buffers must stay where they are while the plan is in use.
+ * `workspace`: qvb8_mlp_workspace_bytes(inter) bytes of device memory, 16-byte aligned, the library's from qvb8_mlp_init
+ * on: it carries the description and the state of the hand-over from call to call, so calls that share it must not
+ * overlap (one workspace per block, or per stream).  Its second word (int32 [1]) is the error word, sticky: nonzero once a
+ * call's bounded wait for H ran out (QVB8_MLP_WAIT_US microseconds, default 20000; that call's Y is NaN) -- it can only run out when the grid is not resident as a whole, e.g. while
+ * other kernels hold CUs for that long.
+ *
+ * qvb8_mlp, per call: X (M, hidden) fp16, or bf16 narrowed like QVB8_MMA_SATURATE_X, 16-byte aligned; Y (M,
+ * out_features).  `act`: QVB8_MLP_SILU_GATED.  QVB8_MLP_TEST_STALE_TAG ORed in makes the producers label H as another
+ * call's, so that the wait runs out: for tests of that path only.
+ * No single counterpart in the reference, which launches the products separately (ext.gemv / ext.mma_multi,
+ * qvb8_cuda.cu:1059-1166, 2566-2671, with the elementwise code of decode/fused_pointwise.py:60-67, 194-204 between them)
+ * and removes the launch cost from the host's side by replaying the MLP as a graph (install_mlp_graphs
+ * formats/qvb8/moe_graph.py:145-178). */
 #define QVB8_MLP_MAX_ROWS 4
 enum qvb8_mlp_act { QVB8_MLP_SILU_GATED = 0, QVB8_MLP_TEST_STALE_TAG = 0x100 };
+typedef struct qvb8_mlp_plan {
+    int64_t hidden, inter, out_features;
+    int64_t magic;                          /* set by qvb8_mlp_init, checked by qvb8_mlp */
+} qvb8_mlp_plan;
 int64_t qvb8_mlp_workspace_bytes(int64_t inter);
-int qvb8_mlp(const void* X, int x_dtype, int64_t M, int64_t hidden, int64_t inter, int64_t out_features,
-             const uint8_t* gu_ids, int64_t gu_ids_bytes, const uint64_t* gu_rowinfo, const qvb8_mma_layout* gu_layout,
-             const uint8_t* dn_ids, int64_t dn_ids_bytes, const uint64_t* dn_rowinfo, const qvb8_mma_layout* dn_layout,
-             int act, int mid_dtype, void* Y, int y_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+int qvb8_mlp_init(int64_t hidden, int64_t inter, int64_t out_features,
+                  const uint8_t* gu_ids, int64_t gu_ids_bytes, const uint64_t* gu_rowinfo, const qvb8_mma_layout* gu_layout,
+                  const uint8_t* dn_ids, int64_t dn_ids_bytes, const uint64_t* dn_rowinfo, const qvb8_mma_layout* dn_layout,
+                  void* workspace, int64_t workspace_bytes, qvb8_mlp_plan* plan, void* stream);
+int qvb8_mlp(const qvb8_mlp_plan* plan, const void* X, int x_dtype, int64_t M, int act, int mid_dtype,
+             void* Y, int y_dtype, void* workspace, void* stream);
 
 /* ---- routed MoE expert stack (decode: a few tokens, top-k experts each) ---------------------------------------- */
 

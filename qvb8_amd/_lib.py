@@ -18,7 +18,7 @@ _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 # every symbol include/qvb8_amd.h declares
 SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_lookup_rows", "qvb8_scatter_escapes", "qvb8_certify",
-           "qvb8_sat_half", "qvb8_scale_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma", "qvb8_launch_probe", "qvb8_mlp_workspace_bytes", "qvb8_mlp",
+           "qvb8_sat_half", "qvb8_scale_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma", "qvb8_launch_probe", "qvb8_mlp_workspace_bytes", "qvb8_mlp_init", "qvb8_mlp",
            "qvb8_moe_workspace_bytes", "qvb8_moe_experts", "qvb8_moe_experts_static",
            "qvb8r_decode", "qvb8r_decode_blocks", "qvb8r_gemv_workspace_bytes", "qvb8r_gemv", "qvb8r_fix_escapes", "qvb8_attn_fwd", "qvb8_attn_combine")
 
@@ -74,7 +74,8 @@ def load(build_if_missing: bool = True):
     lib.qvb8_launch_probe.argtypes = [i64, i64, i64, vp]
     lib.qvb8_mlp_workspace_bytes.argtypes = [i64]
     lib.qvb8_mlp_workspace_bytes.restype = i64
-    lib.qvb8_mlp.argtypes = [vp, i32, i64, i64, i64, i64, vp, i64, vp, vp, vp, i64, vp, vp, i32, i32, vp, i32, vp, i64, vp]
+    lib.qvb8_mlp_init.argtypes = [i64, i64, i64, vp, i64, vp, vp, vp, i64, vp, vp, vp, i64, vp, vp]
+    lib.qvb8_mlp.argtypes = [vp, vp, i32, i64, i32, i32, vp, i32, vp, vp]
     lib.qvb8_moe_workspace_bytes.argtypes = [i64] * 6
     lib.qvb8_moe_workspace_bytes.restype = i64
     lib.qvb8_moe_experts.argtypes = ([vp, i32, i64, vp, vp, i64, i64] + [vp, i64, vp, vp, vp, vp, i64, i64] * 2
@@ -103,6 +104,11 @@ class MmaLayout(ctypes.Structure):
     """qvb8_mma_layout of include/qvb8_amd.h."""
     _fields_ = [("n_classes", ctypes.c_int32), ("first_pos", ctypes.c_int32 * (MMA_MAX_CLASSES + 1)),
                 ("nbits", ctypes.c_int32 * MMA_MAX_CLASSES)]
+
+
+class MlpPlan(ctypes.Structure):
+    """qvb8_mlp_plan of include/qvb8_amd.h."""
+    _fields_ = [("hidden", ctypes.c_int64), ("inter", ctypes.c_int64), ("out_features", ctypes.c_int64), ("magic", ctypes.c_int64)]
 
 
 class RCore(ctypes.Structure):

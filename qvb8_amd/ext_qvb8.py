@@ -480,25 +480,34 @@ MLP_MAX_ROWS = 4                                  # QVB8_MLP_MAX_ROWS
 MLP_SILU_GATED, MLP_TEST_STALE_TAG = 0, 0x100     # qvb8_mlp_act
 
 
-def mlp_workspace(inter: int, device) -> torch.Tensor:
-    """The workspace of mlp_fused for an MLP of `inter` hidden units: zeroed here, once; afterwards the library's (it carries
-    the hand-over's state from call to call, so calls that share it must not overlap).  Words 0 and 1 (int32 view): workgroups
-    of a running call that have taken H, and the sticky error word."""
-    lib = _lib.load()
-    return torch.zeros(int(lib.qvb8_mlp_workspace_bytes(int(inter))), dtype=torch.uint8, device=device)
+MLP_H_AT = 128                                    # byte of the workspace at which H starts (state words and description before it)
 
 
-def mlp_fused(X, gu_ids, gu_rowinfo, gu_layout, dn_ids, dn_rowinfo, dn_layout, hidden, inter, out_features, workspace,
-              mid_dtype=None, out_dtype=None, act=MLP_SILU_GATED):
-    """down(silu(gate(x)) * up(x)) for 1..4 rows of X as ONE launch (qvb8_mlp): the gate+up pack in unit order and the
-    down pack, both stored in planes with a row layout (see formats/qvb8/mlp.py, which builds them), `workspace` from
-    mlp_workspace.  `mid_dtype`: the type the values between the products are rounded to (X's by default), `out_dtype`
-    the result's (X's by default).  Raises RuntimeError for what the kernel does not cover: callers fall back to the
-    separate products."""
+def mlp_init(gu_ids, gu_rowinfo, gu_layout, dn_ids, dn_rowinfo, dn_layout, hidden, inter, out_features):
+    """(workspace, plan) of mlp_fused for one MLP (qvb8_mlp_init): the gate+up pack in unit order and the down pack, both
+    stored in planes with a row layout (formats/qvb8/mlp.py builds them).  The workspace is the library's from here on -- it
+    carries the block's description and the hand-over's state from call to call, so calls that share it must not overlap;
+    word 1 (int32 view) is the sticky error word.  Raises RuntimeError for packs the kernel cannot read."""
     lib = _lib.load()
-    _lib.require_cuda(X, gu_ids, gu_rowinfo, dn_ids, dn_rowinfo, workspace)
-    if X.dim() != 2 or X.shape[1] != int(hidden):
-        raise RuntimeError(f"X must be (M, {int(hidden)})")
+    _lib.require_cuda(gu_ids, gu_rowinfo, dn_ids, dn_rowinfo)
+    plan = _lib.MlpPlan()
+    with torch.cuda.device(gu_ids.device):
+        ws = torch.empty(int(lib.qvb8_mlp_workspace_bytes(int(inter))), dtype=torch.uint8, device=gu_ids.device)
+        _lib._check(lib.qvb8_mlp_init(int(hidden), int(inter), int(out_features),
+                                      gu_ids.data_ptr(), gu_ids.numel(), gu_rowinfo.data_ptr(), ctypes.addressof(gu_layout),
+                                      dn_ids.data_ptr(), dn_ids.numel(), dn_rowinfo.data_ptr(), ctypes.addressof(dn_layout),
+                                      ws.data_ptr(), ws.numel(), ctypes.addressof(plan), _lib.stream_of(gu_ids)), lib)
+    return ws, plan
+
+
+def mlp_fused(X, workspace, plan, mid_dtype=None, out_dtype=None, act=MLP_SILU_GATED):
+    """down(silu(gate(x)) * up(x)) for 1..4 rows of X as ONE launch (qvb8_mlp), on the (workspace, plan) of mlp_init.
+    `mid_dtype`: the type the values between the products are rounded to (X's by default), `out_dtype` the result's (X's by
+    default).  Raises RuntimeError for what the kernel does not cover: callers fall back to the separate products."""
+    lib = _lib.load()
+    _lib.require_cuda(X, workspace)
+    if X.dim() != 2 or X.shape[1] != int(plan.hidden):
+        raise RuntimeError(f"X must be (M, {int(plan.hidden)})")
     if X.dtype not in (torch.float16, torch.bfloat16):
         raise RuntimeError("qvb8 mlp: X must be fp16 or bf16")
     M = X.shape[0]
@@ -506,12 +515,9 @@ def mlp_fused(X, gu_ids, gu_rowinfo, gu_layout, dn_ids, dn_rowinfo, dn_layout, h
     out_dtype = X.dtype if out_dtype is None else out_dtype
     Xc = X.contiguous()
     with torch.cuda.device(Xc.device):
-        Y = torch.empty((M, int(out_features)), dtype=out_dtype, device=Xc.device)
-        _lib._check(lib.qvb8_mlp(_lib.ptr(Xc), _lib.dtype_code(Xc.dtype), M, int(hidden), int(inter), int(out_features),
-                                 gu_ids.data_ptr(), gu_ids.numel(), gu_rowinfo.data_ptr(), ctypes.addressof(gu_layout),
-                                 dn_ids.data_ptr(), dn_ids.numel(), dn_rowinfo.data_ptr(), ctypes.addressof(dn_layout),
-                                 int(act), _lib.dtype_code(mid_dtype), Y.data_ptr(), _lib.dtype_code(out_dtype),
-                                 workspace.data_ptr(), workspace.numel(), _lib.stream_of(Xc)), lib)
+        Y = torch.empty((M, int(plan.out_features)), dtype=out_dtype, device=Xc.device)
+        _lib._check(lib.qvb8_mlp(ctypes.addressof(plan), _lib.ptr(Xc), _lib.dtype_code(Xc.dtype), M, int(act), _lib.dtype_code(mid_dtype),
+                                 Y.data_ptr(), _lib.dtype_code(out_dtype), workspace.data_ptr(), _lib.stream_of(Xc)), lib)
     return Y
 
 

@@ -7,8 +7,9 @@ still is a launch, so here the block is one kernel: the gate+up product, the act
 resident grid and hand H over inside it.
 
 `QVBandMLPV8` stands where a model's `mlp` module stood (gate_proj / up_proj / down_proj of QVBandLinearV8, SiLU): for
-1..4 rows it makes the one launch, for anything else -- more rows, fp32 activations, a pack the kernel cannot read -- it
-computes the same chain with the separate products on the SAME stored bytes (nothing is held twice).  Values: gate and
+1..4 rows it can make the one launch (`one_launch`, off by default: see there), for anything else -- more rows, fp32
+activations, a pack the kernel cannot read -- it computes the same chain with the separate products on the SAME stored
+bytes (nothing is held twice).  Values: gate and
 up results rounded to the activations' type, SiLU in fp32 rounded to it, the product rounded to it, the down product's
 input narrowed like every fp16-path activation -- what the separate modules and torch's elementwise kernels produce.
 """
@@ -61,6 +62,11 @@ class QVBandMLPV8(nn.Module):
     """gate_proj / up_proj / down_proj (QVBandLinearV8, no bias, no escapes) with gated SiLU between them."""
 
     max_rows = ext.MLP_MAX_ROWS
+    # Whether 1..4 rows take the one-launch kernel.  Off by default: measured on the 9B shapes (hidden 4096, inter 12288) the
+    # one launch takes 29.6 us against 30.0 us for the two separate launches -- the hand-over inside the grid costs what the
+    # launch it saves costs (see the kernel's source) --, so the separate products, which every other row count uses anyway,
+    # stay the default.  QVB8_MLP_FUSED=1 in the environment (or True here) switches it on.
+    one_launch = False
 
     def __init__(self, gate: QVBandLinearV8, up: QVBandLinearV8, down: QVBandLinearV8):
         super().__init__()
@@ -71,7 +77,7 @@ class QVBandMLPV8(nn.Module):
         self.gate_up = concat_linears([gate, up])[0]
         self.down = down
         self.fused_ready = False
-        self._ws = None
+        self._ws = self._plan = None
         self._prepare_fused()
 
     def _prepare_fused(self):
@@ -91,13 +97,15 @@ class QVBandMLPV8(nn.Module):
         if ok:
             ok = _whole_tiles(gu._mma_cache[2], 32)
         self.fused_ready = bool(ok)
+        self._ws = self._plan = None
         if ok:
-            self._ws = ext.mlp_workspace(self.inter, gu.ids.device)
+            self._ws, self._plan = ext.mlp_init(gu.ids, gu._mma_cache[1], gu._mma_cache[2], dn.ids, d[1], d[2],
+                                                self.hidden, self.inter, self.out_features)
 
     def _apply(self, fn, recurse=True):
         out = super()._apply(fn, recurse)
-        if self._ws is not None and self._ws.device != self.gate_up.ids.device:
-            self._ws = ext.mlp_workspace(self.inter, self.gate_up.ids.device)
+        if self._ws is not None and self._ws.device != self.gate_up.ids.device:      # the weights moved: describe them anew
+            self._prepare_fused()
         return out
 
     def error_raised(self) -> bool:
@@ -114,11 +122,8 @@ class QVBandMLPV8(nn.Module):
         rows, out_dtype = activation_rows(x, self.gate_up.min_s.device)
         M = rows.shape[0]
         if (self.fused_ready and 1 <= M <= self.max_rows and rows.dtype in (torch.float16, torch.bfloat16)
-                and os.environ.get("QVB8_MLP_FUSED", "1") != "0"):
-            gperm, ginfo, glay = self.gate_up._mma_order()
-            dperm, dinfo, dlay = self.down._mma_order()
-            y = ext.mlp_fused(rows, self.gate_up.ids, ginfo, glay, self.down.ids, dinfo, dlay, self.hidden, self.inter,
-                              self.out_features, self._ws, mid_dtype=rows.dtype, out_dtype=rows.dtype)
+                and os.environ.get("QVB8_MLP_FUSED", "1" if self.one_launch else "0") != "0"):
+            y = ext.mlp_fused(rows, self._ws, self._plan, mid_dtype=rows.dtype, out_dtype=rows.dtype)
             return y.reshape(*x.shape[:-1], self.out_features).to(out_dtype)
         return self.separate(rows).reshape(*x.shape[:-1], self.out_features).to(out_dtype)
 

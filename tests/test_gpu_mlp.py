@@ -15,6 +15,11 @@ from qvb8_amd.formats.qvb8.module import QVBandLinearV8
 from tests import helpers as H
 
 pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _one_launch(monkeypatch):
+    monkeypatch.setenv("QVB8_MLP_FUSED", "1")          # the module's default is the separate products
 DEV = "cuda:0"
 NAME = {torch.bfloat16: "bf16", torch.float16: "fp16"}
 
@@ -55,7 +60,7 @@ def _check(y, x, Ws, dtype, M):
 
 def _h_of(mlp, M):
     """H as the last call with M rows left it in the workspace: (values as float32, tags)."""
-    words = mlp._ws[64:].view(torch.int32)
+    words = mlp._ws[ext.MLP_H_AT:].view(torch.int32)
     base = mlp.inter * (M * (M - 1) // 2)
     w = words[base: base + M * mlp.inter].cpu().numpy().astype(np.uint32)
     return (w & 0xFFFF).astype(np.uint16).view(np.float16).astype(np.float32).reshape(M, mlp.inter), w >> 16
@@ -163,15 +168,12 @@ def test_the_wait_for_h_is_bounded(monkeypatch):
     good = mlp(x)
     torch.cuda.synchronize()
     monkeypatch.setenv("QVB8_MLP_WAIT_US", "200")
-    _, ginfo, glay = mlp.gate_up._mma_order()
-    _, dinfo, dlay = mlp.down._mma_order()
-    args = (x, mlp.gate_up.ids, ginfo, glay, mlp.down.ids, dinfo, dlay, mlp.hidden, mlp.inter, mlp.out_features, mlp._ws)
     print("mlp stale tag", flush=True)
-    y = ext.mlp_fused(*args, act=ext.MLP_SILU_GATED | ext.MLP_TEST_STALE_TAG)
+    y = ext.mlp_fused(x, mlp._ws, mlp._plan, act=ext.MLP_SILU_GATED | ext.MLP_TEST_STALE_TAG)
     torch.cuda.synchronize()
     assert bool(torch.isnan(y.float()).all())
     assert mlp.error_raised()
-    state = mlp._ws[:64].view(torch.int32).cpu()
+    state = mlp._ws[:32].view(torch.int32).cpu()
     assert state[0].item() == 0                                        # every workgroup was counted, the count was closed
     monkeypatch.delenv("QVB8_MLP_WAIT_US")
     mlp._ws[4:8].zero_()
@@ -189,10 +191,9 @@ def test_what_the_kernel_does_not_cover_goes_the_separate_way():
         if dtype == torch.bfloat16:
             _check(y, x, Ws, dtype, M)
     with pytest.raises(RuntimeError):
-        _, ginfo, glay = mlp.gate_up._mma_order()
-        _, dinfo, dlay = mlp.down._mma_order()
-        ext.mlp_fused(torch.zeros(5, 512, dtype=torch.bfloat16, device=DEV), mlp.gate_up.ids, ginfo, glay, mlp.down.ids, dinfo,
-                      dlay, 512, 768, 512, mlp._ws)
+        ext.mlp_fused(torch.zeros(5, 512, dtype=torch.bfloat16, device=DEV), mlp._ws, mlp._plan)
+    with pytest.raises(RuntimeError):                                  # a plan goes with the workspace it was made for
+        ext.mlp_fused(torch.zeros(1, 512, dtype=torch.bfloat16, device=DEV), mlp._ws.clone(), mlp._plan)
 
 
 def test_install_replaces_a_models_mlps():
