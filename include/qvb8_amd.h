@@ -251,8 +251,9 @@ enum qvb8_moe_act {
      * no counterpart in the reference).  "Regular": every row of the stack has the width nbits[0], and row q of expert e
      * starts at bit  bit_off[0] + e * (bit_off[Q] - bit_off[0]) + q * P * nbits[0].  The matrix-core paths (1..16 tokens)
      * then work a row's place out instead of reading nbits / bit_off, which takes one dependent memory trip out of every
-     * launch; results are bit for bit those without the flag.  A stack for which the statement is false gives wrong
-     * results (never an access outside the ids buffer). */
+     * launch; results are bit for bit those without the flag (also when the rows do not start on dword boundaries: they
+     * are then read id by id, as without the flag).  A stack for which the statement is false gives wrong results (never
+     * an access outside the ids buffer). */
     QVB8_MOE_UP_REGULAR = 0x100,
     QVB8_MOE_DOWN_REGULAR = 0x200
 };
@@ -272,7 +273,9 @@ int64_t qvb8_moe_workspace_bytes(int64_t tokens, int64_t topk, int64_t n_experts
  *     token that chose it); the down projection adds the slots up with their routing weights;
  *   7 .. 16 tokens: four launches (plan, up, down, combine): the (token, choice) pairs are grouped by expert, the tokens
  *     that chose an expert are the token rows of one MFMA operand, and every selected expert is read ONCE however many
- *     tokens chose it.
+ *     tokens chose it.  An expert's pairs are the rows of one operand, as many as there are tokens: an expert with more
+ *     pairs than that (only possible when a token lists it twice) makes the whole output NaN instead of a sum with pairs
+ *     missing; the other paths take such lists.
  * Everything else takes the general path (four launches, H in fp32, an expert read once for up to 8 of its tokens).
  * Replaces: ext.moe_experts  qvb8_moe_experts_forward qvb8_cuda.cu:937-992 (kernels qvb8_moe_gemv :860-907,
  * qvb8_moe_act :910-918, qvb8_moe_combine :924-935) with act QVB8_MOE_SILU_GATED, and ext.moe_experts_relu2

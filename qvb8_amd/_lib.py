@@ -36,14 +36,25 @@ def load(build_if_missing: bool = True):
     if _LIB is not None:
         return _LIB
     path = lib_path()
-    if not os.path.exists(path):
-        if not build_if_missing or os.environ.get("QVB8_AMD_LIB"):
+    own = not os.environ.get("QVB8_AMD_LIB")           # a library named by the caller is taken as it is
+    missing = not os.path.exists(path)
+    stale = False
+    if own and not missing:
+        from . import build as _b
+        stale = _b.needs_build()                       # a source or the header is newer than the library
+    if missing or stale:
+        if not build_if_missing or not own:
             raise NativeLibraryError(f"{path} is missing: run `python -m qvb8_amd.build`")
         from . import build as _b
         try:
             _b.build(verbose=False)
         except Exception as ex:                      # noqa: BLE001
-            raise NativeLibraryError(f"cannot build {path}: {ex}") from None
+            if missing:
+                raise NativeLibraryError(f"cannot build {path}: {ex}") from None
+            # a box without the compiler (or with read-only sources) cannot refresh a library it did not build: say so and
+            # refuse rather than run code that no longer matches its sources
+            raise NativeLibraryError(f"{path} is older than its sources and cannot be rebuilt here ({ex}): "
+                                     "run `python -m qvb8_amd.build` where hipcc is") from None
     try:
         lib = ctypes.CDLL(path)
     except OSError as ex:

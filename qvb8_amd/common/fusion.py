@@ -3,8 +3,12 @@ share.  A format supplies `combine(members) -> (fused linear, row split points)`
 thin modules that hand out their slice of the fused result.
 
 Which siblings are fed the same tensor is a property of the model families the reference serves
-(src/qv_band/formats/qvb8r/fuse.py:17-21)."""
+(src/qv_band/formats/qvb8r/fuse.py:17-21); what the fused launch must do for its callers -- one product per distinct
+input, every member's slice handed out once -- is that of fuse.py:52-119 there.
+"""
 from __future__ import annotations
+
+import weakref
 
 import torch
 import torch.nn as nn
@@ -17,36 +21,46 @@ SAME_INPUT_GROUPS = (
 )
 
 
+class _Held:
+    """The fused result of one input, kept until each member has fetched its part: which tensor it was computed from (a weak
+    reference plus the tensor's version counter, so neither a new tensor at the old address nor the old tensor modified in
+    place can be mistaken for it), the parts, and one bit per member that has not fetched yet."""
+    __slots__ = ("source", "version", "parts", "waiting")
+
+    def __init__(self, x: torch.Tensor, parts):
+        self.source, self.version = weakref.ref(x), x._version
+        self.parts = parts
+        self.waiting = (1 << len(parts)) - 1
+
+    def serves(self, x: torch.Tensor, member: int) -> bool:
+        return self.source() is x and x._version == self.version and bool(self.waiting >> member & 1)
+
+
 class FusedGroup(nn.Module):
-    """Holds the fused linear of one group.  The first member that is called with a tensor computes every member's
-    output; the others take theirs from that result."""
+    """Holds the fused linear of one group.  The first member called with a tensor makes the one launch for all; the others
+    take their slices of that result.  This sharing lives in Python: a graph capture records forward() instead."""
 
     def __init__(self, lin: nn.Module, splits: list[int]):
         super().__init__()
         self.lin, self.splits = lin, list(splits)
-        self._x = None
-        self._ver = None
-        self._outs = None
-        self._left: set = set()
+        self._held: _Held | None = None
 
     def forward(self, x):
         """All members' outputs for `x`, as views of one result."""
         return torch.tensor_split(self.lin(x), self.splits, -1)
 
-    def get(self, x, i):
-        # A stored result is handed out only for the SAME tensor object (kept alive here, so its storage cannot be reused
-        # by another tensor meanwhile), unmodified since (its version counter), and only until every member has taken
-        # its part once (fuse.py:64-77 of the reference).  This reuse lives in Python: under graph replay capture
-        # forward() instead.
-        if self._x is not x or x._version != self._ver or i not in self._left:
-            self._outs = self.forward(x)
-            self._x, self._ver = x, x._version
-            self._left = set(range(len(self._outs)))
-        self._left.discard(i)
-        out = self._outs[i]
-        if not self._left:
-            self._x = self._outs = None
-        return out
+    def holding(self) -> bool:
+        """Whether a result is still kept for members that have not fetched their part."""
+        return self._held is not None
+
+    def part(self, x, member: int):
+        held = self._held
+        if held is None or not held.serves(x, member):
+            held = self._held = _Held(x, self.forward(x))
+        held.waiting &= ~(1 << member)
+        if held.waiting == 0:                              # every member has its part: nothing is kept alive
+            self._held = None
+        return held.parts[member]
 
 
 class FusedMember(nn.Module):
@@ -55,16 +69,33 @@ class FusedMember(nn.Module):
 
     def __init__(self, group: FusedGroup, i: int, in_features: int, out_features: int, bias=None):
         super().__init__()
-        object.__setattr__(self, "group", group)       # shared by the members: kept out of the module tree
+        self._group = (group,)                             # inside a tuple: the members share it, only its owner registers it
         self.i, self.in_features, self.out_features = i, in_features, out_features
         self.bias = bias
 
+    @property
+    def group(self) -> FusedGroup:
+        return self._group[0]
+
     def forward(self, x):
-        y = self.group.get(x, self.i)
-        return y if self.bias is None else y + self.bias.to(y.dtype)
+        out = self._group[0].part(x, self.i)
+        if self.bias is not None:
+            out = out + self.bias.to(out.dtype)
+        return out
 
     def extra_repr(self):
-        return f"in_features={self.in_features}, out_features={self.out_features}, fused member {self.i}"
+        return f"member {self.i} of a fused launch: {self.in_features} -> {self.out_features}"
+
+
+def _sibling_groups(model: nn.Module, eligible):
+    """(owner, names) of every same-input group under `model` whose members all pass `eligible`."""
+    found = []
+    for parent in model.modules():
+        for holder, names in SAME_INPUT_GROUPS:
+            owner = getattr(parent, holder, None)
+            if owner is not None and eligible(owner, names):
+                found.append((owner, names))
+    return found
 
 
 def fuse_groups(model: nn.Module, eligible, combine, attr: str, member_bias=lambda m: None) -> int:
@@ -72,23 +103,22 @@ def fuse_groups(model: nn.Module, eligible, combine, attr: str, member_bias=lamb
     FusedGroup built by `combine(list of members)`.  The group is registered once, as `attr` of the layer that owns the
     siblings.  Returns the number of groups fused.
 
-    No list of the model's modules is kept while groups are replaced, and a group's separate members are released before
-    the next group is built: otherwise the separate and the fused copies of the whole model would exist side by side."""
-    owners = [(owner, names) for parent in model.modules() for sub, names in SAME_INPUT_GROUPS
-              if (owner := getattr(parent, sub, None)) is not None and eligible(owner, names)]
-    done = 0
-    for owner, names in owners:
-        members = [getattr(owner, a) for a in names]
-        shapes = [(m.in_features, m.out_features, member_bias(m)) for m in members]
-        for a in names:
-            setattr(owner, a, None)
+    Only (owner, names) pairs are kept while groups are replaced, and a group's separate members are taken off their owner
+    before its fused linear is built: otherwise the separate and the fused copies of the whole model would exist side by
+    side."""
+    groups = _sibling_groups(model, eligible)
+    for owner, names in groups:
+        members = []
+        for name in names:
+            members.append(getattr(owner, name))
+            setattr(owner, name, None)
+        facts = [(m.in_features, m.out_features, member_bias(m)) for m in members]
         lin, splits = combine(members)
-        del members
+        members.clear()
         group = FusedGroup(lin, splits)
         setattr(owner, attr, group)
-        for i, (a, (pin, pout, b)) in enumerate(zip(names, shapes)):
-            setattr(owner, a, FusedMember(group, i, pin, pout, b))
-        done += 1
-    if done and torch.cuda.is_available():
+        for index, (name, (n_in, n_out, bias)) in enumerate(zip(names, facts)):
+            setattr(owner, name, FusedMember(group, index, n_in, n_out, bias))
+    if groups and torch.cuda.is_available():
         torch.cuda.empty_cache()
-    return done
+    return len(groups)

@@ -47,7 +47,10 @@ __host__ __device__ inline MoePlan moe_plan_at(void* ws, int64_t E, int64_t npai
 
 // One workgroup: pairs grouped by expert (counting sort), table of the experts that have pairs.  The two running
 // sums over the experts (pairs before expert e, selected experts before e) are a workgroup scan, 256 experts per round.
-__global__ void __launch_bounds__(kMoeThreads) moe_plan_kernel(const int64_t* __restrict__ idx, int npairs, int E, MoePlan pl) {
+// `cap`: the most pairs one expert may have for the path that follows (the grouped walk takes an expert's pairs as the token
+// rows of ONE operand: at most one per token); an expert with more counts as a bad entry, so the results come out as NaN
+// instead of sums with pairs missing.
+__global__ void __launch_bounds__(kMoeThreads) moe_plan_kernel(const int64_t* __restrict__ idx, int npairs, int E, MoePlan pl, int cap) {
     extern __shared__ int32_t s_cnt[];                        // [E] counts, then cursors; [E .. E + 8) scan scratch
     int32_t* s_scan = s_cnt + E;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -66,6 +69,7 @@ __global__ void __launch_bounds__(kMoeThreads) moe_plan_kernel(const int64_t* __
     for (int e0 = 0; e0 < E; e0 += blockDim.x) {
         const int e = e0 + tid;
         const int c = e < E ? s_cnt[e] : 0;
+        if (c > cap) atomicAdd(pl.n_bad, 1);
         // inclusive scan of (c, c > 0) packed as pairs * 2^16 + active: both stay below 2^15 per round... pairs can be
         // larger, so scan them separately
         int sc = c, sa = c > 0 ? 1 : 0;
@@ -459,7 +463,10 @@ __global__ void __launch_bounds__(64 * kOneWaves) moe_one_kernel(MoeOneArgs a) {
         // REG: one width for the whole stack, known without looking at the lanes (rows that cannot be read -- an expert
         // number outside the stack -- decode whatever was loaded; their results are replaced by NaN below)
         const uint32_t info0 = REG ? ((uint32_t)reg_nb | ((reg_nb >= 4 && reg_nb <= 8) ? 256u : 0u)) : (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
-        const bool uniform = REG ? (info0 >> 8) == 1u : (__builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u);
+        // (a regular stack whose rows do not start on dword boundaries has no sliced row: its lanes then multiply id 0 here and
+        // the rows are redone element by element below, as without the statement)
+        const bool uniform = REG ? ((info0 >> 8) == 1u && __builtin_amdgcn_ballot_w64(q.e_ok && !sliced) == 0)
+                                 : (__builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u);
 #pragma unroll
         for (int it = 0; it < T; ++it) {
             v4u_t b[4];
@@ -773,7 +780,9 @@ __device__ __forceinline__ void moe_walk_body(const MoeWalkArgs& a) {
             const uint32_t info = sliced ? ((uint32_t)nbr | 256u) : 0u;
             // REG: one width for the whole stack (rows that cannot be read decode what was loaded and end as NaN)
             const uint32_t info0 = REG ? ((uint32_t)reg_nb | ((reg_nb >= 4 && reg_nb <= 8) ? 256u : 0u)) : (uint32_t)__builtin_amdgcn_readfirstlane((int)info);
-            const bool uniform = REG ? (info0 >> 8) == 1u : (__builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u);
+            // (usable rows of a regular stack that do not start on dword boundaries are not sliced: zero here, redone below)
+            const bool uniform = REG ? ((info0 >> 8) == 1u && __builtin_amdgcn_ballot_w64((rec.flags & 256) != 0 && !sliced) == 0)
+                                     : (__builtin_amdgcn_ballot_w64(info != info0) == 0 && (info0 >> 8) == 1u);
 #pragma unroll
             for (int it = 0; it < T; ++it) {
                 v4u_t b[4];
@@ -1086,7 +1095,8 @@ extern "C" int qvb8_moe_experts(const void* X, int x_dtype, int64_t tokens, cons
         return launch_moe_one<true, false, 2>(o, dn_regular, dn_blocks, tk, s);
     }
 
-    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)(n_experts + 8) * 4, s, idx, (int)np, (int)n_experts, pl);
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kMoeThreads), (size_t)(n_experts + 8) * 4, s, idx, (int)np, (int)n_experts, pl,
+                       grouped ? (int)(tokens < 16 ? tokens : 16) : (int)np);
     if (int rc = host::check_launch("qvb8_moe_experts plan")) return rc;
     const int64_t slots = moe_slots(n_experts, np);
     if (grouped) {

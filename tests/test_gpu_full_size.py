@@ -71,12 +71,32 @@ def test_qvb8r_restore_equals_qvb8_restore_at_27b_shape():
     assert torch.equal(lin.dense(torch.float16), ext.decode(*_args(enc)))
     max_err, bad = ext.certify(lin.dense(torch.float16), W, 2e-3)
     assert bad == 0 and max_err < 2e-3
-    x = torch.randn(3, P, device=DEV, generator=torch.Generator(device=DEV).manual_seed(4)).to(torch.bfloat16)
-    y = lin(x).float().double()
     w32 = lin.dense(torch.float32).double()
-    ref = x.float().double() @ w32.t()
-    tol = (1e-3 + 2.0 ** -8) * ref.abs() + 1e-3 * w32.norm(dim=1)[None, :] * x.float().double().norm(dim=1)[:, None] / np.sqrt(P)
-    assert bool(((y - ref).abs() <= tol).all())
+    for M in (1, 3, 16):                                     # the configuration's row counts, and one in between
+        x = torch.randn(M, P, device=DEV, generator=torch.Generator(device=DEV).manual_seed(4 + M)).to(torch.bfloat16)
+        y = lin(x).float().double()
+        ref = x.float().double() @ w32.t()
+        tol = (1e-3 + 2.0 ** -8) * ref.abs() + 1e-3 * w32.norm(dim=1)[None, :] * x.float().double().norm(dim=1)[:, None] / np.sqrt(P)
+        assert bool(((y - ref).abs() <= tol).all()), (M, float(((y - ref).abs() / tol).max()))
+
+
+def test_qvb8r_products_at_the_27b_down_shape():
+    """The other 27B-class shape of the configuration: 5120 rows of 17408 columns would take minutes to encode on the CPU, so
+    rows of 5120 columns (gate / up: 17408 x 5120) stand for it with 1 and 16 rows of X."""
+    from qvb8_amd.formats.qvb8r import pack as RP
+    from qvb8_amd.formats.qvb8r.module import QVBandLinearV8R
+    Q, P = 4096, 5120
+    W = _weight(Q, P, seed=21)
+    enc = PK.encode_tensor(W, 2e-3, keep_ids=True)
+    lin = QVBandLinearV8R(RP.transcode(enc), device=DEV)
+    assert torch.equal(lin.dense(torch.float16), ext.decode(*_args(enc)))
+    w64 = lin.dense(torch.float32).double()
+    for M in (1, 16):
+        x = torch.randn(M, P, device=DEV, generator=torch.Generator(device=DEV).manual_seed(M)).to(torch.bfloat16)
+        y = lin(x).float().double()
+        ref = x.float().double() @ w64.t()
+        tol = (1e-3 + 2.0 ** -8) * ref.abs() + 1e-3 * w64.norm(dim=1)[None, :] * x.float().double().norm(dim=1)[:, None] / np.sqrt(P)
+        assert bool(((y - ref).abs() <= tol).all()), (M, float(((y - ref).abs() / tol).max()))
 
 
 @pytest.mark.parametrize("Q,P", [(28672, 8192), (8192, 28672)])

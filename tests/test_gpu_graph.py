@@ -53,14 +53,18 @@ class _Moe(nn.Module):
         super().__init__()
         gu = [_lin(2 * inter, h, 10 + e) for e in range(E)]
         dn = [_lin(h, inter, 40 + e) for e in range(E)]
+        self.restored = ([_RESTORED[m] for m in gu], [_RESTORED[m] for m in dn])     # before the stack re-stores the rows
         self.experts = QVBandExpertsV8(gu, dn, num_experts=E)
         self.router = nn.Linear(h, E, bias=False).to(DEV).to(torch.bfloat16)
         self.k = k
 
-    def forward(self, x):
+    def route(self, x):
         p = torch.softmax(self.router(x).float(), -1)
         w, idx = torch.topk(p, self.k, -1)
-        return self.experts(x, idx, (w / w.sum(-1, keepdim=True)))
+        return idx, w / w.sum(-1, keepdim=True)
+
+    def forward(self, x):
+        return self.experts(x, *self.route(x))
 
 
 class _Layer(nn.Module):
@@ -94,6 +98,12 @@ def test_graph_replay_is_bit_identical(kind):
             torch.cuda.synchronize()
             _ = (xs[rep].float() @ xs[rep].float().T).sum().item()  # the program's own eager work between replays
             assert torch.equal(got, want[rep]), (kind, rows, rep)
+            if kind == "moe":                                       # and the replayed result is the oracle's, not just eager's
+                idx, w = eager.route(xs[rep])
+                ref = O.moe_reference(xs[rep].float().cpu().numpy(), idx.cpu().numpy(), w.float().cpu().numpy(), *eager.restored)
+                diff = np.abs(got.float().cpu().numpy().astype(np.float64) - ref)
+                tol = (1e-3 + 2.0 ** -8) * np.abs(ref) + 2e-3 * np.sqrt(np.mean(ref ** 2))
+                assert np.all(diff <= tol), (rows, rep, float((diff / tol).max()))
     assert sum(1 for v in layer.mlp._graphs.values() if isinstance(v, tuple)) == 2
     big = torch.randn(64, h, device=DEV).to(torch.bfloat16)         # prefill-sized input: eager, no new graph
     assert torch.equal(layer.mlp(big), eager(big))

@@ -153,7 +153,7 @@ def test_same_input_fusion_is_bit_identical():
     got = [blk.self_attn.q_proj(x), blk.self_attn.k_proj(x), blk.self_attn.v_proj(x)]
     for a, b in zip(got, want):
         assert torch.equal(a, b)
-    assert blk.self_attn._qvb8_fused._x is None           # every member took its part: nothing is held
+    assert not blk.self_attn._qvb8_fused.holding()        # every member took its part: nothing is held
 
 
 @pytest.mark.parametrize("widths,sortable", [([7, 6, 9], True), ([5], True), ([4], True), ([8, 4], True), ([7, 6, 9, 3, 8, 5], False)])

@@ -313,3 +313,58 @@ def test_moe_regular_stack_changes_no_result(T, monkeypatch):
     # a claim that does not hold is not made for a stack built by hand
     ops, _ = _hand_made_stack(3, 64, 128, [5, 6], seed=5)
     assert not ext.stack_is_regular(ops[3], ops[4], 128)
+
+
+@pytest.mark.parametrize("T", [1, 8])
+def test_moe_regular_stack_off_dword_boundaries(T, monkeypatch):
+    """A stack that is regular as the interface defines it -- one width, rows at regular places -- but moved by one byte,
+    so that no row starts on a dword boundary: with the statement the kernels give what they give without it."""
+    E, hidden, inter, k = 6, 256, 128, 2
+    monkeypatch.setenv("QVB8_MOE_ONE_WIDTH_GROWTH", "0.25")
+    gu, dn, Wgu, Wdn = [], [], [], []
+    for e in range(E):
+        for lst, Wl, (Q, P) in ((gu, Wgu, (2 * inter, hidden)), (dn, Wdn, (hidden, inter))):
+            W = (0.02 * torch.randn(Q, P, generator=torch.Generator().manual_seed(900 + 2 * e + len(lst)))).to(torch.bfloat16).to(DEV)
+            enc = PK.encode_tensor(W, 2e-3, restore="fp16")
+            lst.append(QVBandLinearV8.from_encoded(enc))
+            v = H.oracle_view(enc)
+            Wl.append(O.reconstruct(v["min_s"], v["tau_s"], H.oracle_ids(v), v["esc_idx"], v["esc_vals"]))
+    mod = QVBandExpertsV8(gu, dn, num_experts=E)
+    assert mod.build_stack()
+    g, d = mod._stk
+    assert g["regular"] and d["regular"]
+
+    def moved(st):
+        ids = torch.cat([torch.zeros(1, dtype=torch.uint8, device=DEV), st["ids"]])
+        return ids, st["min_s"], st["tau_s"], st["nbits"], st["bit_off"] + 8
+
+    gm, dm = moved(g), moved(d)
+    assert ext.stack_is_regular(gm[3], gm[4], hidden) and ext.stack_is_regular(dm[3], dm[4], inter)
+    idx, w = _route(T, E, k, seed=3 + T)
+    x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(T)).to(torch.bfloat16).to(DEV)
+    args = (x, torch.from_numpy(idx).to(DEV), torch.from_numpy(w).to(DEV), *gm, 2 * inter, hidden, *dm, hidden, inter)
+    plain = ext.moe_experts(*args)
+    stated = ext.moe_experts(*args, regular=(True, True))
+    assert torch.equal(plain, stated)
+    _check(stated, O.moe_reference(x.float().cpu().numpy(), idx, w, Wgu, Wdn), torch.bfloat16)
+
+
+def test_moe_grouped_walk_and_an_expert_listed_twice_for_a_token():
+    """Seven to sixteen tokens group the pairs by expert, the pairs of an expert being the rows of ONE operand: as many as
+    there are tokens.  A token may list an expert twice as long as that holds (the pairs are rows of their own); an expert
+    with more pairs than tokens gives NaN everywhere rather than a sum with pairs missing."""
+    E, hidden, inter, k, T = 6, 256, 128, 2, 8
+    gu, dn, Wgu, Wdn = _experts(E, hidden, inter, 2e-3, seed=300)
+    mod = QVBandExpertsV8(gu, dn, num_experts=E)
+    idx, w = _route(T, E, k, seed=5)
+    x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(DEV)
+    twice = idx.copy()
+    twice[3, 1] = twice[3, 0]
+    out = mod(x, torch.from_numpy(twice).to(DEV), torch.from_numpy(w).to(DEV))
+    _check(out, O.moe_reference(x.float().cpu().numpy(), twice, w, Wgu, Wdn), torch.bfloat16)
+    crowded = idx.copy()
+    crowded[:, 0] = 2                                    # every token chooses expert 2 ...
+    crowded[:, 1] = np.where(crowded[:, 1] == 2, 3, crowded[:, 1])
+    crowded[0, 1] = 2                                    # ... and one of them twice: nine pairs for eight tokens
+    out = mod(x, torch.from_numpy(crowded).to(DEV), torch.from_numpy(w).to(DEV))
+    assert bool(torch.isnan(out.float()).all())

@@ -207,7 +207,7 @@ def test_same_input_fusion_against_the_oracle_and_the_members():
     got = [blk.self_attn.q_proj(x), blk.self_attn.k_proj(x), blk.self_attn.v_proj(x)]
     for a, b in zip(got, want):
         assert torch.equal(a, b)
-    assert blk.self_attn._qvb8r_fused._x is None
+    assert not blk.self_attn._qvb8r_fused.holding()
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16, torch.float32])
