@@ -49,9 +49,21 @@ def measured_traffic(profile, kernel):
     return out
 
 
-# symbols per second of the QVB8R walk with the activations and the multiply-adds taken out (same launch shape, the 65B
-# shapes, one row of X), measured once on this hardware: the ceiling the fused kernel is compared with
-WALK_CEILING_TSYM = 1.814
+def measured_figure(profile, key, kernel):
+    """{class: value} of the `<key> <kernel> <class> <value>` lines of a summary under profiles/ ({} without the file)."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", profile)
+    out = {}
+    try:
+        with open(path) as fh:
+            for line in fh:
+                f = line.split()
+                if len(f) == 4 and f[0] == key and f[1] == kernel:
+                    out[f[2]] = float(f[3])
+    except OSError:
+        pass
+    return out
+
+
 MMA_FLAGS = int(os.environ.get("QVB8_BENCH_MMA_FLAGS", "1"))     # 1 = QVB8_MMA_SATURATE_X: the operator's default for bf16 x
 
 
@@ -152,9 +164,10 @@ def cpu_baseline(layers, x_by_p, budget_s=12.0):
                       % (len(done), ",".join(done), nbytes / 1e6, dt)}
 
 
-def time_graph(step, steps, warmup):
+def time_graph(step, steps, warmup, spread=None):
     """Captures `step` (launches on torch's current stream) in a HIP graph, replays it `warmup` + `steps` times; returns
-    (ms per step by HIP events on the replay stream, ms per step by the host clock)."""
+    (ms per step by HIP events on the replay stream, ms per step by the host clock).  With a dict as `spread`, every
+    replay is bracketed by events of its own and the dict receives median / min / max of the replays in ms."""
     import torch
     step()
     torch.cuda.synchronize()
@@ -164,15 +177,21 @@ def time_graph(step, steps, warmup):
     for _ in range(warmup):
         graph.replay()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1 if spread is not None else 2)]
     t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
+    marks[0].record()
+    for i in range(steps):
         graph.replay()
-    e1.record()
+        if spread is not None:
+            marks[i + 1].record()
+    if spread is None:
+        marks[1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return e0.elapsed_time(e1) / steps, wall * 1e3 / steps
+    if spread is not None:
+        each = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+        spread.update(replays=steps, median_ms=round(each[len(each) // 2], 5), min_ms=round(each[0], 5), max_ms=round(each[-1], 5))
+    return marks[0].elapsed_time(marks[-1]) / steps, wall * 1e3 / steps
 
 
 def synthetic_routing(logits, k):
@@ -243,14 +262,15 @@ def bench_moe(args, dev):
                                       out.data_ptr(), 2, ws.data_ptr(), ws.numel(), s)
             if rc != 0:
                 raise RuntimeError(lib.qvb8_last_error().decode())
-    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
+    spread = {}
+    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup, spread)
     ms = max(ev_ms, wall_ms)
     gbs = step_bytes / (ms * 1e-3) / 1e9
     per_layer_us = ev_ms * 1e3 / n_calls
     return {"metric": "expert-gathered fused decode-GEMV GB/s on the bytes of the unique selected experts, 35B-A3B-shape MoE "
                       "layer, 1 MI355X",
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "ms_per_step": round(ms, 5), "spread": spread, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16 activations narrowed to fp16 x fp32 band value, fp32 accumulate", "data": "synthetic",
             "config": {"workload": "MoE layer: hidden 2048, 128 experts gate/up 2048->768 + down 768->2048, top-8, QVB8 "
                                    "tau=2e-3, %d token(s), %d layers x %d routings per step" % (T, args.layers, rounds),
@@ -298,11 +318,23 @@ def bench_qvb8r(args, dev, token_counts=None):
             coded_bytes += 4 * len(d["words"]) + 8 * 32 * len(d["tiles"]) + 4 * 4096 * d["K"] + 12 * Q + 8 * Q
             n_sym += Q * P
             del d
-    results = [_time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name) for M in (token_counts or [args.tokens])]
+    # the ceiling of this path, measured in the same run on the same packs: the launches of the one-row kernel with the
+    # activations and the multiply-adds taken out (qvb8r_walk_probe), i.e. the entropy decode alone
+    for u in units:
+        u["Yp"] = torch.empty(1, u["Q"], dtype=torch.float32, device=dev)
+
+    def walk_only():
+        s = torch.cuda.current_stream().cuda_stream
+        for u in units:
+            if lib.qvb8r_walk_probe(ctypes.byref(u["core"]), u["lin"].T, u["Yp"].data_ptr(), s) != 0:
+                raise RuntimeError(lib.qvb8_last_error().decode())
+    walk_ms = max(time_graph(walk_only, args.steps, args.warmup))
+    walk_tsym = n_sym / (walk_ms * 1e-3) / 1e12
+    results = [_time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name, walk_tsym) for M in (token_counts or [args.tokens])]
     return results if token_counts else results[0]
 
 
-def _time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name):
+def _time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name, walk_tsym):
     import ctypes
     import torch
     step_bytes = coded_bytes + sum(2 * M * (u["P"] + u["Q"]) for u in units)
@@ -319,14 +351,15 @@ def _time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name):
                                 u["ws"].data_ptr(), u["ws"].numel(), s)
             if rc != 0:
                 raise RuntimeError(lib.qvb8_last_error().decode())
-    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
+    spread = {}
+    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup, spread)
     ms = max(ev_ms, wall_ms)
     gbs = step_bytes / (ms * 1e-3) / 1e9
     launch_us = ev_ms * 1e3 / len(units)
     kernel = "qvb8::r_gemv_kernel<2>" if M == 1 else "qvb8::r_mma_kernel<%d, false> (+ r_pack_x_kernel)" % ((M + 15) // 16)
     return {"metric": "QVB8R fused entropy-decode + GEMV GB/s on coded bytes, large-dense FFN shapes, 1 MI355X",
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "ms_per_step": round(ms, 5), "spread": spread, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16 activations x fp32 band value (M > 1: exact fp16 operands on the matrix cores), fp32 accumulate",
             "data": "synthetic",
             "config": {"workload": "QVB8R tau=2e-3, %s, M=%d, %d layers" % (shape_name, M, args.layers),
@@ -337,9 +370,10 @@ def _time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name):
                          "kernel": kernel,
                          "bytes_per_launch": step_bytes // len(units), "launch_us": round(launch_us, 3),
                          "note": "the walk is bound by its instruction count (vector ALU 91 % busy), not by HBM"},
-            "roofline_walk": {"bound": "rANS walk alone (slot lookup, 64-bit state update, ballot / popcount, ring read) at this launch shape",
-                              "achieved": round(n_sym / (ms * 1e-3) / 1e12, 4), "peak": WALK_CEILING_TSYM, "unit": "T symbols/s",
-                              "frac": round(n_sym / (ms * 1e-3) / 1e12 / WALK_CEILING_TSYM, 4)},
+            "roofline_walk": {"bound": "the entropy decode alone: the same launches with the activations and the multiply-adds taken out "
+                                       "(qvb8r_walk_probe), timed in this run on these packs",
+                              "achieved": round(n_sym / (ms * 1e-3) / 1e12, 4), "peak": round(walk_tsym, 4), "unit": "T symbols/s",
+                              "frac": round(n_sym / (ms * 1e-3) / 1e12 / walk_tsym, 4)},
             "cpu_baseline": None}
 
 
@@ -666,39 +700,53 @@ def bench_smallm(args, dev, prebuilt=None, tokens=None):
     def step():
         for u in units:
             u["out"] = u["lin"](x_by_p[u["P"]])
-    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup)
+    spread = {}
+    ev_ms, wall_ms = time_graph(step, args.steps, args.warmup, spread)
     ms = max(ev_ms, wall_ms)
     gbs = step_bytes / (ms * 1e-3) / 1e9
     tflops = flops / (ms * 1e-3) / 1e12
+    # HBM bytes per layer and the matrix pipes' busy share, from hardware counters (profiles/, with the commands that took
+    # them): present for the row counts that were profiled
+    prof = "gemm_kernel_9b_small_m_trace_and_counters.md"
+    per_layer = measured_figure(prof, "traffic_bytes_per_layer", "qvb8_mma").get("M=%d" % M)
+    busy_cycles = measured_figure(prof, "mfma_busy_cycles_per_layer", "qvb8_mma").get("M=%d" % M)
+    # SQ_VALU_MFMA_BUSY_CYCLES summed over the chip's 1024 SIMDs, against this run's time per layer at 2.0 GHz
+    mfma_busy = None if busy_cycles is None else round(100.0 * busy_cycles / 1024.0 / (ms * 1e-3 / n_layers * 2.0e9), 2)
     path = ("fused decode + MFMA, X in registers (qvb8_mma, tile kernel)" if M <= 48 else
             "fused decode + MFMA GEMM, X staged in LDS (qvb8_mma, workgroup-tiled kernel)" if M <= 256 else "fp16 restore + library GEMM")
     bound = "hbm" if M <= 64 else "mfma"
     return {"metric": "small-M fused decode + GEMM: GB/s on packed bytes and TFLOP/s, 9B projections, 1 MI355X",
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "bf16 activations, fp32 accumulate, bf16 out", "data": "synthetic", "tflops": round(tflops, 3),
+            "ms_per_step": round(ms, 5), "spread": spread, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16 activations narrowed to fp16, ids as exact fp16 operands, fp32 accumulate, bf16 out", "data": "synthetic",
+            "tflops": round(tflops, 3), "mfma_busy_pct": mfma_busy,
             "config": {"workload": "9B-shape projections, QVB8 tau=1e-3, M=%d, %d layers, path: %s" % (M, n_layers, path),
                        "bytes_per_step": step_bytes, "flops_per_step": flops, "launch_units": len(units)},
             "roofline": ({"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None if per_layer is None else int(per_layer),
+                          "bytes_per_layer": step_bytes // n_layers}
                          if bound == "hbm" else
                          {"bound": "mfma", "achieved": round(tflops, 3), "peak": 2500.0, "unit": "TFLOP/s",
-                          "frac": round(tflops / 2500.0, 5), "traffic": None}),
+                          "frac": round(tflops / 2500.0, 5), "traffic": None if per_layer is None else int(per_layer),
+                          "bytes_per_layer": step_bytes // n_layers}),
             "cpu_baseline": None}
 
 
-def run_legs(args, dev, layers, units):
+def run_legs(args, dev, lib, layers, units):
     """Short runs of the other configurations, each on its own synthetic packs, appended to the headline's line under
-    `legs`: the 9B projections with 16 / 64 / 256 rows (the first 8 layers of the headline's packs), the 35B-A3B-shape MoE
-    layer with 1 and 8 tokens, the 65B-shape QVB8R pair with 1 and 16 rows.  Each entry: value, unit, ms_per_step,
-    roofline, config (and tflops for the small-M legs)."""
+    `legs`: the 9B projections with 16 / 64 / 256 rows (the first 8 layers of the headline's packs), the decode step on 8
+    layers of the 27B-class shapes, the 35B-A3B-shape MoE layer with 1 and 8 tokens, the QVB8R FFN pair of the 65B and of the
+    27B shapes with 1 and 16 rows.  Every leg is a HIP graph replayed at least 100 times, each replay between events of
+    its own: `ms_per_step` is the mean of the timed region, `spread` the median and the extremes of the replays."""
     import copy
     import gc
     import torch
-    keep = ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "tflops", "dtype", "roofline", "roofline_walk", "config")
+    keep = ("metric", "value", "unit", "ms_per_step", "spread", "steps", "warmup", "tflops", "mfma_busy_pct", "dtype",
+            "roofline", "roofline_walk", "config")
     legs = {}
     sub = copy.copy(args)
-    sub.steps, sub.warmup = max(5, min(args.steps, 20)), 3
+    sub.steps, sub.warmup = max(100, args.steps), 3
+    sub.copy_probe = False
     n8 = min(8, len(layers))
     per_layer = len(units) // len(layers)
     for M in (16, 64, 256):
@@ -708,6 +756,12 @@ def run_legs(args, dev, layers, units):
     units.clear()
     gc.collect()
     torch.cuda.empty_cache()
+    l27, u27 = build_layers(8, dev, fuse=True, shapes=LAYER_27B)
+    r = time_decode(sub, dev, lib, l27, u27, LAYER_27B, "27b")[0]
+    legs["decode27b"] = {k: r[k] for k in keep if k in r}
+    del l27, u27, r
+    gc.collect()
+    torch.cuda.empty_cache()
     sub.layers = 2
     for T in (1, 8):
         sub.tokens = T
@@ -715,10 +769,87 @@ def run_legs(args, dev, layers, units):
         legs["moe_T%d" % T] = {k: r[k] for k in keep if k in r}
         gc.collect()
         torch.cuda.empty_cache()
-    sub.layers, sub.model = 1, "65b"
-    for M, r in zip((1, 16), bench_qvb8r(sub, dev, token_counts=[1, 16])):
-        legs["qvb8r_M%d" % M] = {k: r[k] for k in keep if k in r}
+    sub.layers = 1
+    for model, tag in (("65b", "qvb8r"), ("27b", "qvb8r27b")):
+        sub.model = model
+        for M, r in zip((1, 16), bench_qvb8r(sub, dev, token_counts=[1, 16])):
+            legs["%s_M%d" % (tag, M)] = {k: r[k] for k in keep if k in r}
+        gc.collect()
+        torch.cuda.empty_cache()
     return legs
+
+
+def time_decode(args, dev, lib, layers, units, shapes, model):
+    """Times the decode step (one row of X through every launch unit of `layers`) as a replayed HIP graph: `args.steps`
+    replays between one pair of events give the line's value; a second pass of at least 100 replays, each between events of
+    its own, gives `spread`.  Returns (line, the function that launches a list of units, the activations by width)."""
+    import torch
+    from qvb8_amd import _lib
+    g = torch.Generator(device=dev).manual_seed(7)
+    x_by_p = {P: torch.randn(1, P, device=dev, generator=g).to(torch.bfloat16) for P in sorted({p for _, _, p in shapes})}
+    flat = [enc for lay in layers for enc in lay]
+    step_bytes = sum(algorithmic_bytes(e, 1) for e in flat)
+    assert step_bytes == sum(u["bytes"] for u in units)
+    n_launch = len(units)
+
+    def run_units(which):
+        s = torch.cuda.current_stream().cuda_stream
+        for u in which:
+            x, lin = x_by_p[u["P"]], u["lin"]
+            rc = lib.qvb8_mma(x.data_ptr(), _lib.dtype_code(x.dtype), 1, lin.ids.data_ptr(), lin.ids.numel(),
+                              lin.min_s.data_ptr(), lin.tau_s.data_ptr(), lin.nbits.data_ptr(), lin.bit_off.data_ptr(),
+                              u["Q"], u["P"], lin.esc_idx.data_ptr() if u["n_esc"] else None,
+                              lin.esc_vals.data_ptr() if u["n_esc"] else None, u["n_esc"],
+                              u["perm"].data_ptr(), u["rowinfo"].data_ptr(),
+                              ctypes.addressof(u["layout"]) if u["layout"] is not None else None,
+                              mma_flags(lin), u["Y"].data_ptr(), None, 0, s)
+            if rc != 0:
+                raise RuntimeError(lib.qvb8_last_error().decode())
+
+    def step():
+        run_units(units)
+
+    if getattr(args, "copy_probe", False):
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+    ev_per_step, wall_per_step = time_graph(step, args.steps, args.warmup)
+    ev_ms, wall = ev_per_step * args.steps, wall_per_step * args.steps * 1e-3
+    ms_per_step = max(wall * 1e3, ev_ms) / args.steps
+    spread = {}
+    time_graph(step, max(100, args.steps), 2, spread)
+    gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
+    launch_us = ev_ms * 1e3 / (args.steps * n_launch)
+    achieved = (step_bytes / n_launch) / (launch_us * 1e-6) / 1e9
+    esc = sum(e["esc_idx"].numel() for e in flat)
+    n_layers = len(layers)
+    fused = len(units) < len(flat)
+
+    out = {
+        "metric": decode_metric_name(model),
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "spread": spread, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": ("bf16 activations narrowed to fp16 (saturating), ids as exact fp16 matrix-core operands, fp32 accumulate, "
+                  "row scale and offset applied in double, fp32 out"), "data": "synthetic",
+        "tokens_per_s": round(1e3 / ms_per_step, 2), "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+        "config": {"workload": ("Qwen-9B-shape decoder layer set (q/k/v/o 4096x4096 with k/v 1024, gate/up 12288, down "
+                                "12288->4096), QVB8 tau=1e-3, bf16 activations, M=1, %d layers" % n_layers) if model == "9b" else
+                               ("27B-class decoder layer set (q/o 5120x5120, k/v 1024x5120, gate/up 17408, down 17408->5120), "
+                                "QVB8 tau=1e-3, bf16 activations, M=1, %d layers" % n_layers),
+                   "launches_per_step": n_launch, "launch_units": "+".join(sorted({u["name"] for u in units}, key=len)),
+                   "bytes_per_step": step_bytes, "escapes": esc,
+                   "bits_per_weight": round(8.0 * sum(u["lin"].ids.numel() for u in units) / sum(e["Q"] * e["P"] for e in flat), 3)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": tile_traffic(units, n_launch) if (MMA_FLAGS == 1 and model == "9b" and fused) else None,
+                     "kernel": "qvb8::tile_kernel<1,4,false,true,XP,PL> (XP = 1 or 4 pieces of X per thread through LDS; PL: rows stored in planes)" + (" / <1,5,false,true,XP,PL> for 5120-column rows" if model == "27b" else ""),
+                     "bytes_per_launch": step_bytes // n_launch,
+                     "launch_us": round(launch_us, 3)},
+    }
+    return out, run_units, x_by_p
 
 
 def main():
@@ -780,65 +911,7 @@ def main():
         return 2
     shapes = LAYER_27B if args.model == "27b" else LAYER_9B
     layers, units = build_layers(args.layers, dev, fuse=not args.no_fuse, shapes=shapes)
-    g = torch.Generator(device=dev).manual_seed(7)
-    x_by_p = {P: torch.randn(1, P, device=dev, generator=g).to(torch.bfloat16) for P in sorted({p for _, _, p in shapes})}
-    flat = [enc for lay in layers for enc in lay]
-    step_bytes = sum(algorithmic_bytes(e, 1) for e in flat)
-    assert step_bytes == sum(u["bytes"] for u in units)
-    n_launch = len(units)
-
-    def run_units(which):
-        s = torch.cuda.current_stream().cuda_stream
-        for u in which:
-            x, lin = x_by_p[u["P"]], u["lin"]
-            rc = lib.qvb8_mma(x.data_ptr(), _lib.dtype_code(x.dtype), 1, lin.ids.data_ptr(), lin.ids.numel(),
-                              lin.min_s.data_ptr(), lin.tau_s.data_ptr(), lin.nbits.data_ptr(), lin.bit_off.data_ptr(),
-                              u["Q"], u["P"], lin.esc_idx.data_ptr() if u["n_esc"] else None,
-                              lin.esc_vals.data_ptr() if u["n_esc"] else None, u["n_esc"],
-                              u["perm"].data_ptr(), u["rowinfo"].data_ptr(),
-                              ctypes.addressof(u["layout"]) if u["layout"] is not None else None,
-                              mma_flags(lin), u["Y"].data_ptr(), None, 0, s)
-            if rc != 0:
-                raise RuntimeError(lib.qvb8_last_error().decode())
-
-    def step():
-        run_units(units)
-
-    if args.copy_probe:
-        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            torch.add(src, 1.0, out=dst)
-        torch.cuda.synchronize()
-        del src, dst
-    ev_per_step, wall_per_step = time_graph(step, args.steps, args.warmup)
-    ev_ms, wall = ev_per_step * args.steps, wall_per_step * args.steps * 1e-3
-    ms_per_step = max(wall * 1e3, ev_ms) / args.steps
-    gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
-    launch_us = ev_ms * 1e3 / (args.steps * n_launch)
-    achieved = (step_bytes / n_launch) / (launch_us * 1e-6) / 1e9
-    esc = sum(e["esc_idx"].numel() for e in flat)
-
-    out = {
-        "metric": decode_metric_name(args.model),
-        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 activations x fp32 band value, fp32 accumulate", "data": "synthetic",
-        "tokens_per_s": round(1e3 / ms_per_step, 2), "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
-        "config": {"workload": ("Qwen-9B-shape decoder layer set (q/k/v/o 4096x4096 with k/v 1024, gate/up 12288, down "
-                                "12288->4096), QVB8 tau=1e-3, bf16 activations, M=1, %d layers" % args.layers) if args.model == "9b" else
-                               ("27B-class decoder layer set (q/o 5120x5120, k/v 1024x5120, gate/up 17408, down 17408->5120), "
-                                "QVB8 tau=1e-3, bf16 activations, M=1, %d layers" % args.layers),
-                   "launches_per_step": n_launch, "launch_units": "+".join(sorted({u["name"] for u in units}, key=len)),
-                   "bytes_per_step": step_bytes, "escapes": esc,
-                   "bits_per_weight": round(8.0 * sum(u["lin"].ids.numel() for u in units) / sum(e["Q"] * e["P"] for e in flat), 3)},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": tile_traffic(units, n_launch) if (MMA_FLAGS == 1 and args.model == "9b" and not args.no_fuse) else None,
-                     "kernel": "qvb8::tile_kernel<1,4,false,true,XP,PL> (XP = 1 or 4 pieces of X per thread through LDS; PL: rows stored in planes)" + (" / <1,5,false,true,XP,PL> for 5120-column rows" if args.model == "27b" else ""),
-                     "bytes_per_launch": step_bytes // n_launch,
-                     "launch_us": round(launch_us, 3)},
-    }
+    out, run_units, x_by_p = time_decode(args, dev, lib, layers, units, shapes, args.model)
     # GB/s per projection group: the launches of one kind over all layers, replayed on their own (not part of `value`)
     per = {}
     for name in sorted({u["name"] for u in units}, key=len):
@@ -853,7 +926,7 @@ def main():
     else:
         out["cpu_baseline"] = None
     if not args.no_legs and args.model == "9b" and not args.no_fuse:
-        out["legs"] = run_legs(args, dev, layers, units)
+        out["legs"] = run_legs(args, dev, lib, layers, units)
     print(json.dumps(out))
     return 0
 

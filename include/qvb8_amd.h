@@ -52,7 +52,7 @@ enum qvb8_status {
 
 /* Library identification: ABI version, bumped on any signature change or new entry point (3: row lookup, attention over
  * the banded KV cache, query preparation; 4: qvb8_moe_experts_static; 5: result-type flags of qvb8_mma; 6: rows stored
- * in planes, QVB8_MMA_PLANES; 7: qvb8_mlp).  A binding compares the loaded library's answer
+ * in planes, QVB8_MMA_PLANES; 7: qvb8_mlp, qvb8r_walk_probe).  A binding compares the loaded library's answer
  * with the QVB8_ABI_VERSION it was written for before it makes any other call. */
 #define QVB8_ABI_VERSION 7
 int qvb8_abi_version(void);
@@ -355,6 +355,12 @@ int64_t qvb8r_gemv_workspace_bytes(int64_t M, int64_t P);
  * (which multiplies fp16-rounded weights; this one keeps the fp32 band value). */
 int qvb8r_gemv(const void* X, int x_dtype, int64_t M, const qvb8r_core* core, int64_t max_tile_rows, float* Y,
                void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Measurement aid: the launch of qvb8r_gemv for one row of X with the activations not read and the two multiply-adds per
+ * symbol pair replaced by an exclusive-or of the symbols -- the rANS walk alone (slot lookups, 64-bit state updates, word
+ * hand-out, ring reads), the ceiling of the fused kernel on this hardware.  Y (f32, Q) receives values without meaning.
+ * No counterpart in the reference. */
+int qvb8r_walk_probe(const qvb8r_core* core, int64_t max_tile_rows, float* Y, void* stream);
 
 /* Y[m, uq[u]] += sum_{e in [ptr[u], ptr[u+1])} X[m, ec[e]] * ed[e]: one thread per (m, u), stored order, no atomics.
  * Replaces: ext.fix_escapes  qvb8r_fix_escapes qvb8r_cuda.cu:311-320. */

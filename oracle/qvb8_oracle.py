@@ -25,6 +25,10 @@ Pinning status (what fixes each function besides this file's own text):
                                       unpack_tensor / unpack_formula
   sat_half                            closed form (clamp, then numpy.float16)
   gemv / mma / moe references         float64 matmul of the restored weights
+  round_to                            closed forms (ties, fp16 subnormals, overflow)
+  swiglu                              torch's CPU silu and multiply on bf16 / fp16 / fp32
+                                      tensors (an independent implementation)
+  mlp_reference                       identity weights reduce it to swiglu and sat_half
 The synthetic ENCODER policy is not pinned by anything: the reference ships no
 writer.  Any writer whose bytes the readers accept and whose restore meets the
 certificate conforms.

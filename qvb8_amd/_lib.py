@@ -20,7 +20,7 @@ _DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 SYMBOLS = ("qvb8_abi_version", "qvb8_last_error", "qvb8_decode", "qvb8_lookup_rows", "qvb8_scatter_escapes", "qvb8_certify",
            "qvb8_sat_half", "qvb8_scale_sat_half", "qvb8_gemv_workspace_bytes", "qvb8_gemv", "qvb8_mma_rowinfo_bytes", "qvb8_mma_prepare", "qvb8_mma_workspace_bytes", "qvb8_mma", "qvb8_launch_probe", "qvb8_mlp_workspace_bytes", "qvb8_mlp_init", "qvb8_mlp",
            "qvb8_moe_workspace_bytes", "qvb8_moe_experts", "qvb8_moe_experts_static",
-           "qvb8r_decode", "qvb8r_decode_blocks", "qvb8r_gemv_workspace_bytes", "qvb8r_gemv", "qvb8r_fix_escapes", "qvb8_attn_fwd", "qvb8_attn_combine")
+           "qvb8r_decode", "qvb8r_decode_blocks", "qvb8r_gemv_workspace_bytes", "qvb8r_gemv", "qvb8r_walk_probe", "qvb8r_fix_escapes", "qvb8_attn_fwd", "qvb8_attn_combine")
 
 
 def lib_path() -> str:
@@ -98,6 +98,7 @@ def load(build_if_missing: bool = True):
     lib.qvb8r_gemv_workspace_bytes.argtypes = [i64, i64]
     lib.qvb8r_gemv_workspace_bytes.restype = i64
     lib.qvb8r_gemv.argtypes = [vp, i32, i64, vp, i64, vp, vp, i64, vp]
+    lib.qvb8r_walk_probe.argtypes = [vp, i64, vp, vp]
     lib.qvb8r_fix_escapes.argtypes = [vp, i32, i64, vp, vp, vp, vp, i64, vp, i64, i64, vp]
     lib.qvb8_attn_fwd.argtypes = ([vp, i64, i64, vp, vp, i32, i64, i64] + [vp] * 9 + [i64, vp, vp, vp] + [i64] * 6
                                   + [ctypes.c_double, i64, vp])

@@ -195,6 +195,9 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
                 }
             } else {
                 rec = a.loc[pos];
+                // a record that says "stored in planes" reaching the kernel variant for rows back to back (the caller left
+                // QVB8_MMA_PLANES out): its offset names the tile, not the row -- the row comes out as NaN, not as another row's values
+                if constexpr (!PL) { if ((rec >> 58) & 1ull) rec &= ~(3ull << 56); }
             }
         }
         my_loc[i] = rec;

@@ -182,7 +182,9 @@ __global__ void __launch_bounds__(kRThreads) r_decode_kernel(RCore c, int b0, in
 }
 
 // ---- fused decode + product, one row of X ------------------------------------------------------------------------------
-template <int DT>
+// WALK_ONLY (a measurement aid, qvb8r_walk_probe): the same launch with the activations not read and the two multiply-adds
+// per pair replaced by an exclusive-or that keeps the symbols alive -- what the walk alone costs, the ceiling of this path.
+template <int DT, bool WALK_ONLY = false>
 __global__ void __launch_bounds__(kRThreads) r_gemv_kernel(RCore c, const void* __restrict__ X, float* __restrict__ Y, int T) {
     __shared__ uint32_t st[4096];
     __shared__ uint32_t ring[kRTiles][kRing];
@@ -199,20 +201,30 @@ __global__ void __launch_bounds__(kRThreads) r_gemv_kernel(RCore c, const void* 
     // instead of a test per pair: the loop is bound by its instruction count)
     auto walk_row = [&](auto first) __attribute__((always_inline)) {
         constexpr bool FIRST = decltype(first)::value;
-        float acc = 0.f;
-        float x1 = load_as_f32<DT>(X, l32), x2 = load_as_f32<DT>(X, 32 + l32);
-        for (int s0 = 0; s0 < S; s0 += 2) {
-            const int sn = s0 + 2 < S ? s0 + 2 : s0;                       // the last pair reloads itself (unused)
-            const float n1 = load_as_f32<DT>(X, sn * 32 + l32), n2 = load_as_f32<DT>(X, (sn + 1) * 32 + l32);
-            uint32_t s1, s2;
-            walk_pair(z, st, rg, l32, half, t.room, s1, s2);
-            acc = __builtin_fmaf(x1, (float)s1, acc);
-            acc = __builtin_fmaf(x2, (float)s2, acc);
-            if constexpr (FIRST) sx += x1 + x2;
-            x1 = n1; x2 = n2;
+        if constexpr (WALK_ONLY) {
+            uint32_t keep = 0;
+            for (int s0 = 0; s0 < S; s0 += 2) {
+                uint32_t s1, s2;
+                walk_pair(z, st, rg, l32, half, t.room, s1, s2);
+                keep ^= s1 + s2;
+            }
+            return (float)keep;
+        } else {
+            float acc = 0.f;
+            float x1 = load_as_f32<DT>(X, l32), x2 = load_as_f32<DT>(X, 32 + l32);
+            for (int s0 = 0; s0 < S; s0 += 2) {
+                const int sn = s0 + 2 < S ? s0 + 2 : s0;                   // the last pair reloads itself (unused)
+                const float n1 = load_as_f32<DT>(X, sn * 32 + l32), n2 = load_as_f32<DT>(X, (sn + 1) * 32 + l32);
+                uint32_t s1, s2;
+                walk_pair(z, st, rg, l32, half, t.room, s1, s2);
+                acc = __builtin_fmaf(x1, (float)s1, acc);
+                acc = __builtin_fmaf(x2, (float)s2, acc);
+                if constexpr (FIRST) sx += x1 + x2;
+                x1 = n1; x2 = n2;
+            }
+            if constexpr (FIRST) sx = half_sum(sx);
+            return acc;
         }
-        if constexpr (FIRST) sx = half_sum(sx);
-        return acc;
     };
     for (int r = 0; r < T; ++r) {
         if (!(t.has && r < t.nr)) continue;                                // per half-wave
@@ -491,6 +503,16 @@ extern "C" int qvb8r_decode_blocks(const qvb8r_core* core, int64_t max_tile_rows
         default: hipLaunchKernelGGL(r_decode_kernel<3>, grid, block, 0, s, c, 0, (int64_t)0, out_rows, out, T, block_list); break;
     }
     return host::check_launch("qvb8r_decode_blocks");
+}
+
+extern "C" int qvb8r_walk_probe(const qvb8r_core* core, int64_t max_tile_rows, float* Y, void* stream) {
+    RCore c;
+    if (int rc = check_core("qvb8r_walk_probe", core, c)) return rc;
+    if (max_tile_rows < 1 || max_tile_rows > 0x7fffffff) return host::fail(QVB8_ERR_ARG, "qvb8r_walk_probe: bad rows-per-tile bound");
+    if (c.Q == 0 || c.n_blocks == 0) return QVB8_OK;
+    if (!Y) return host::fail(QVB8_ERR_ARG, "qvb8r_walk_probe: null pointer");
+    hipLaunchKernelGGL((r_gemv_kernel<0, true>), dim3((unsigned)c.n_blocks), dim3(kRThreads), 0, (hipStream_t)stream, c, (const void*)Y, Y, (int)max_tile_rows);
+    return host::check_launch("qvb8r_walk_probe");
 }
 
 extern "C" int64_t qvb8r_gemv_workspace_bytes(int64_t M, int64_t P) {

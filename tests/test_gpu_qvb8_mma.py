@@ -291,6 +291,14 @@ def test_rows_stored_in_planes_change_no_result(Q, P, widths):
                                ext.mma_tiles(x, *args_p, perm=perm, rowinfo=rowinfo_p, planes=True)), M
     _check(d, None, _x(3, P, torch.bfloat16, 3), ext.mma_tiles(_x(3, P, torch.bfloat16, 3), *args_p, perm=perm, rowinfo=rowinfo_p,
                                                               layout=layout_p, planes=True), saturate_ref=True)
+    # a caller that leaves the statement out while the records mark rows as stored in planes: those rows come out as NaN
+    # (their offset names a tile, not a row), every other row as usual -- never another row's values
+    x = _x(2, P, torch.bfloat16, 9)
+    left_out = ext.mma_tiles(x, *args_p, perm=perm, rowinfo=rowinfo_p)
+    right = ext.mma_tiles(x, *args_p, perm=perm, rowinfo=rowinfo_p, planes=True)
+    marked = ((off_p >> 62) & 1) == 1
+    assert bool(marked.any()) and bool(torch.isnan(left_out[:, marked]).all())
+    assert torch.equal(left_out[:, ~marked], right[:, ~marked])
 
 
 @pytest.mark.parametrize("Q,P,widths", [(300, 768, [7, 6, 5]), (136, 256, [8, 4]), (333, 256, [6, 9, 5]), (40, 128, [5, 6, 7, 8]), (64, 128, [7])])

@@ -99,6 +99,30 @@ def test_65b_row_lengths_against_the_oracle(Q, P):
         assert np.all(diff <= tol), (M, float((diff / tol).max()))
 
 
+def test_walk_probe_walks_the_symbols_of_the_product_kernel():
+    """The measurement aid that times the walk alone: it leaves, per row, tau_s times the sum over the 32 lanes of the
+    exclusive-or of (symbol of the even step + symbol of the odd step) over the lane's step pairs -- the same symbols, in
+    the same lanes, as the product kernel multiplies (symbol = id - the row's delta).  Nothing else is read: X is absent."""
+    import ctypes
+    from qvb8_amd import _lib
+    Q, P = 90, 768
+    W, enc, d = _make(Q, P, 2e-3, seed=21, rows_per_tile=4, n_classes=2)
+    lin = QVBandLinearV8R(d, device=DEV)
+    core = lin._core()
+    c, _, _ = ext._core(*core, P)
+    Y = torch.full((1, Q), float("nan"), dtype=torch.float32, device=DEV)
+    lib = _lib.load()
+    assert lib.qvb8r_walk_probe(ctypes.byref(c), lin.T, Y.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+    ids = ext.ids(P, *core, T=lin.T).cpu().numpy().astype(np.int64)
+    drow = core[9].cpu().numpy().astype(np.int64)
+    sym = (ids - drow[:, None]).reshape(Q, P // 64, 2, 32)
+    assert sym.min() >= 0
+    keep = np.bitwise_xor.reduce(sym[:, :, 0, :] + sym[:, :, 1, :], axis=1)          # [row, lane]
+    want = (lin.tau_s.cpu().numpy().astype(np.float64) * keep.sum(1).astype(np.float64)).astype(np.float32)
+    assert np.array_equal(Y.cpu().numpy()[0].view(np.uint32), want.view(np.uint32))
+    assert lib.qvb8r_walk_probe(ctypes.byref(c), 0, Y.data_ptr(), None) != 0                    # bad rows-per-tile bound
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_matrix_core_rows_agree_with_single_row_walk(dtype):
     """Every row of a many-row call against the one-row kernel on the same row: the two differ only in the order of the

@@ -268,3 +268,27 @@ def test_tile_uniform_widths_and_repack_rows_on_the_host():
     off2 = off.clone(); off2[1, 5] += 8
     nb2 = nb.clone(); nb2[0, 3] = 5
     assert not ext.stack_is_regular(nb, off2, 64) and not ext.stack_is_regular(nb2, off, 64)
+
+
+def test_unit_order_of_a_gate_up_pack():
+    """Units of 16 outputs, gate rows then up rows, every row of a unit at the unit's widest width, widths ascending."""
+    import torch
+    from qvb8_amd.formats.qvb8.mlp import unit_order, UNIT
+    inter = 96
+    g = torch.Generator().manual_seed(5)
+    nbits = torch.randint(3, 7, (2 * inter,), generator=g).to(torch.uint8)
+    perm, new_nbits = unit_order(nbits, inter)
+    perm = perm.to(torch.int64)
+    assert sorted(perm.tolist()) == list(range(2 * inter))                     # a permutation of the rows
+    blocks = perm.view(-1, 2, UNIT)
+    assert torch.equal(blocks[:, 1], blocks[:, 0] + inter)                      # a unit's up rows follow its gate rows
+    assert int(blocks[:, 0].max()) < inter
+    stored = new_nbits.to(torch.int64)[perm].view(-1, 2 * UNIT)
+    assert bool((stored == stored[:, :1]).all())                                 # one width per unit ...
+    assert bool((stored[1:, 0] >= stored[:-1, 0]).all())                         # ... ascending over the units
+    assert bool((new_nbits >= nbits.clamp(min=4)).all())                         # no row loses bits
+    need = torch.maximum(nbits[:inter], nbits[inter:]).clamp(min=4).to(torch.int64)
+    assert int(new_nbits.to(torch.int64).sum()) <= 2 * int(need.sum()) + 2 * UNIT * 3 * 4      # only the units at a width change are widened
+    assert unit_order(nbits, inter - 1) is None and unit_order(nbits[:-1], inter) is None
+    wide = nbits.clone(); wide[3] = 9
+    assert unit_order(wide, inter) is None                                       # a row wider than 8 bits

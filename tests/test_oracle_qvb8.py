@@ -264,3 +264,55 @@ def test_embedding_rows_escapes_and_narrowing():
     assert np.array_equal(h, out.astype(np.float16).astype(np.float32))
     b = O.embedding_rows(rows, min_s, tau_s, ids, P, esc_idx, esc_vals, dtype="bf16")
     assert np.array_equal(b, torch.from_numpy(out).to(torch.bfloat16).float().numpy())
+
+
+# ---- the dense MLP chain (gate / up -> SiLU * up -> down) -------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype,tdt", [("bf16", "bfloat16"), ("fp16", "float16"), ("fp32", "float32")])
+def test_swiglu_is_what_torch_computes_in_the_models_dtype(dtype, tdt):
+    """`act_fn(gate) * up` on tensors of the model's dtype, by torch's CPU kernels (which compute silu in fp32 and round its
+    result to the tensor's dtype, then round the product): an implementation that shares nothing with the oracle's.  A
+    missing intermediate rounding, a sigmoid with the wrong sign or gate and up swapped all fail it.  fp32 results may
+    differ in the last place (torch's expf against numpy's float64 exp); the narrow types must agree bit for bit except
+    where a value lies within that last place of a rounding boundary -- counted, and bounded."""
+    import torch
+    import torch.nn.functional as F
+    tdt = getattr(torch, tdt)
+    g = torch.randn(1 << 16, generator=torch.Generator().manual_seed(3)) * 4.0
+    u = torch.randn(1 << 16, generator=torch.Generator().manual_seed(4)) * 2.0
+    g[:8] = torch.tensor([0.0, -0.0, 30.0, -30.0, 1e-6, -1e-6, 88.0, -88.0])
+    g, u = g.to(tdt), u.to(tdt)
+    want = (F.silu(g) * u).float().numpy()
+    got = O.swiglu(g.float().numpy(), u.float().numpy(), dtype)
+    assert got.dtype == np.float32
+    if dtype == "fp32":
+        assert np.all(np.abs(got - want) <= 2.0 ** -22 * np.abs(want) + 1e-37)
+    else:
+        differ = got.view(np.uint32) != want.view(np.uint32)
+        assert differ.mean() < 2e-3, differ.mean()
+        ulp = {"bf16": 2.0 ** -7, "fp16": 2.0 ** -10}[dtype]
+        assert np.all(np.abs(got - want)[differ] <= ulp * np.abs(want)[differ] + 2.0 ** -24)
+    swapped = O.swiglu(u.float().numpy(), g.float().numpy(), dtype)
+    assert not np.array_equal(swapped.view(np.uint32), got.view(np.uint32))
+
+
+def test_round_to_closed_forms():
+    """One rounding to nearest even into each type: ties, the subnormal range of fp16, overflow to infinity."""
+    v = np.array([1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 2.0 ** -25, 3 * 2.0 ** -25, 65520.0, 65519.9], np.float64)
+    assert np.array_equal(O.round_to(v, "fp16"), np.array([1.0, 1.0 + 2.0 ** -9, 0.0, 2.0 ** -23, np.inf, 65504.0], np.float32))
+    v = np.array([1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, -1.0 - 2.0 ** -8], np.float64)
+    assert np.array_equal(O.round_to(v, "bf16"), np.array([1.0, 1.0 + 2.0 ** -6, -1.0], np.float32))
+    assert np.array_equal(O.round_to(np.array([1.0 + 2.0 ** -24, 1.0 + 3 * 2.0 ** -24]), "fp32"),
+                          np.array([1.0, 1.0 + 2.0 ** -22], np.float32))
+
+
+def test_mlp_reference_is_the_chain_of_its_parts():
+    """With identity-like weights the chain reduces to the pointwise function: W_gate = W_up = I, W_down = I gives
+    y = round(sat(swiglu(x, x))) for an x that fp16 holds exactly."""
+    x = np.linspace(-4.0, 4.0, 64, dtype=np.float32).astype(np.float16).astype(np.float32)[None, :]
+    I = np.eye(64, dtype=np.float32)
+    y, h = O.mlp_reference(x, I, I, I, "bf16")
+    assert np.array_equal(h, O.swiglu(O.round_to(x, "bf16"), O.round_to(x, "bf16"), "bf16"))
+    assert np.array_equal(y, O.round_to(O.sat_half(h), "bf16"))
+    y2, _ = O.mlp_reference(x, I, I, 2.0 * I, "bf16")
+    assert np.array_equal(y2, O.round_to(2.0 * O.sat_half(h).astype(np.float64), "bf16"))
