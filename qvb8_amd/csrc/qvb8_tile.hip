@@ -108,6 +108,8 @@ __device__ __forceinline__ void decode_slice8_top(const uint4& lo, const uint4& 
 // microsecond per launch): fin follows loc, n_steps follows P, the small counts share one word.
 // Waves a workgroup of this variant may have: twelve (three per SIMD) where the registers allow it -- long rows then take
 // fewer panels (12288 columns: two instead of three) --, else eight.
+constexpr uint32_t kTileTransitRow = 272;                     // bytes between rows of a wave's transit region (256 + 16: see XT)
+constexpr uint32_t kTileTransitBytes = 16 * kTileTransitRow;
 template <int NT, int T, bool BF, bool PL> constexpr int tile_max_waves() { return (NT == 1 && T == 4 && PL && !BF) ? 12 : 8; }
 
 template <int NT, int T, bool BF, bool XC, int XP = 0, bool PL = false>
@@ -134,7 +136,10 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
     uint4* s_fin = reinterpret_cast<uint4*>(smem);                                       // [rows_cap]
     uint64_t* s_loc = reinterpret_cast<uint64_t*>(s_fin + rows_cap);                     // [n_waves][wave_rows]
     float* sxs = reinterpret_cast<float*>(s_loc + (size_t)n_waves * wave_rows);          // [ranges][TM]
-    float* part = sxs + (size_t)ranges * TM;                                             // [rows_cap][ranges][M]
+    // [rows_cap][ranges][M].  (The lanes of a store -- 16 rows x 4 tokens -- fall into few banks this way; a layout without those
+    // conflicts, [ranges][M][rows_cap + 4], was measured and was 5 % slower at 8..16 rows of X: the stores are not waited for,
+    // and its addresses cost more instructions.)
+    float* part = sxs + (size_t)ranges * TM;
     const int MS = a.M;                                       // a row's partial sums hold M tokens, not the TM the tile could take
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -144,10 +149,20 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
     // XL: the whole of X (at most XP 16-byte pieces per thread) goes through LDS once: every thread requests its
     // pieces before anything else, the first tile's ids follow at once, and the workgroup shares X after one barrier --
     // so the trip of the activations and the first trip of the ids overlap, and later panels need no trip for theirs.
-    unsigned char* xs = reinterpret_cast<unsigned char*>(part + (size_t)rows_cap * ranges * MS);     // [M][P] in operand format
+    // [M][P] as in memory.  (Rows a multiple of 128 bytes apart put the lanes of an operand read, one row each, into the same
+    // banks; moving the rows 16..80 bytes further apart was measured and changed nothing: those reads are not what the
+    // launch waits for.)
+    unsigned char* xs = reinterpret_cast<unsigned char*>(part + (size_t)rows_cap * ranges * MS);
+    static_assert(!XL || NT == 1, "X as a whole in LDS exists for one token tile");
     // JIT: with one token tile and X in LDS a step's operands are read from LDS when the step is multiplied instead of being
     // held in 16 T registers for the whole panel (lanes without a row of X, and steps past the end, read 64 bytes of zeros)
     constexpr bool JIT = XL && NT == 1;
+    // XT (one token tile, X not in LDS as a whole): a wave fetches the activations of its columns in memory order -- a load
+    // instruction covers four rows of X, 256 contiguous bytes of each -- and turns them into operand order through a
+    // 16 x 256-byte region of LDS of its own, step by step.  (Fetched in operand order, every lane reads 64 bytes of a row of
+    // its own: 64 cache lines per instruction, and with 9..16 rows of X the CU's L1 spent more cycles on those accesses than
+    // the launch needs for everything else.)
+    constexpr bool XT = !XL && NT == 1;
     const int x_pieces = (a.M * a.P) >> 3;
     v4u_t xg[XL ? XP : 1];
     if constexpr (XL) {
@@ -273,6 +288,7 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
         return has_tile && ((uint32_t)(rec2 >> 56) & 3u) == 1u ? (((uint32_t)(rec2 >> 48) & 0xFFu) | (1u << 8)) : 0u;
     };
 
+    const uint32_t x_row_bytes = (uint32_t)a.P * 2u, x_zero_at = (uint32_t)a.M * x_row_bytes;
     if constexpr (XL) {
         info = issue_tile(0, wc * T, wlo, whi, n_tiles > 0);   // steps past the row's end read the buffer's start as well
 #pragma unroll
@@ -286,7 +302,7 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
             if (idx < x_pieces) reinterpret_cast<v4u_t*>(xs)[idx] = v;
             __builtin_amdgcn_sched_barrier(0);
         }
-        if constexpr (JIT) { if (tid < 16) reinterpret_cast<uint32_t*>(xs + (size_t)x_pieces * 16)[tid] = 0u; }   // 64 bytes of zeros behind X
+        if constexpr (JIT) { if (tid < 16) reinterpret_cast<uint32_t*>(xs + x_zero_at)[tid] = 0u; }   // 64 bytes of zeros behind X
         // A bare barrier behind this wave's own LDS writes: __syncthreads() carries a release fence that would also wait
         // for the ids just requested.
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -305,15 +321,38 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
         // ---- activations of this wave's columns, in MFMA operand layout: lane (t = l % 16, kg) holds
         //      X[16*nt + t][128*(step0+it) + 32*kg + 8*j + 0..7] ----
         v4u_t xa[NT][T][4];
-        const uint32_t x_zero = (uint32_t)x_pieces * 16u;
         auto x_operand = [&](int it, v4u_t (&xv)[4]) __attribute__((always_inline)) {
             const bool on = active && r < a.M && (step0 + it) < a.n_steps;
-            const uint32_t at = on ? 2u * ((uint32_t)r * (uint32_t)a.P + (uint32_t)(step0 + it) * kStepCols + (uint32_t)kg * 32u) : x_zero;
+            const uint32_t at = on ? (uint32_t)r * x_row_bytes + 2u * ((uint32_t)(step0 + it) * kStepCols + (uint32_t)kg * 32u) : x_zero_at;
 #pragma unroll
             for (int j = 0; j < 4; ++j) xv[j] = *reinterpret_cast<const v4u_t*>(xs + at + 16 * j);
         };
+        if constexpr (XT) {
+            // lane l of load i: row 4 i + l / 16 (rows past the last one read the last one again: their products are never
+            // stored; leaving those requests and their narrowing out under a test of the row count was measured and cost 7 %
+            // at 16 rows, where nothing is left out: the tests break up the burst), bytes 16 (l % 16) .. of the step's 256; a
+            // step past the end of the rows holds zeros
+            const uint32_t row4 = (uint32_t)lane >> 4, last_row = (uint32_t)a.M - 1u;
+            uint32_t lane_at[4];
 #pragma unroll
-        for (int nt = 0; nt < (JIT ? 0 : NT); ++nt) {
+            for (int i = 0; i < 4; ++i) lane_at[i] = min(4u * i + row4, last_row) * (uint32_t)a.P * 2u + ((uint32_t)lane & 15u) * 16u;
+#pragma unroll
+            for (int it = 0; it < T; ++it) {
+                if (active && (step0 + it) < a.n_steps) {                  // wave-uniform
+                    const unsigned char* base = reinterpret_cast<const unsigned char*>(a.X) + (size_t)(step0 + it) * (kStepCols * 2);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint4 v = *reinterpret_cast<const uint4*>(base + lane_at[i]);
+                        xa[0][it][i] = v4u_t{v.x, v.y, v.z, v.w};
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) xa[0][it][i] = v4u_t{0, 0, 0, 0};
+                }
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < ((JIT || XT) ? 0 : NT); ++nt) {
             const int t = nt * 16 + r;
 #pragma unroll
             for (int it = 0; it < T; ++it) {
@@ -345,6 +384,21 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
 #pragma unroll
                         for (int k = 0; k < 4; ++k) xa[nt][it][j][k] = XI::pair(xa[nt][it][j][k]);
         }
+        if constexpr (XT) {
+            // into operand order: piece (row, chunk) is written where lane (row, chunk / 4) finds it as its register chunk % 4;
+            // rows are 272 bytes apart, so that the eight lanes LDS serves per cycle touch all banks both ways.  The region is
+            // this wave's own and a wave's LDS accesses keep their order: no barrier, and the next step may overwrite it.
+            unsigned char* tr = xs + (size_t)wave * kTileTransitBytes;
+            const uint32_t put = (uint32_t)(lane >> 4) * kTileTransitRow + (uint32_t)(lane & 15) * 16u;
+            const uint32_t get = (uint32_t)r * kTileTransitRow + (uint32_t)kg * 64u;
+#pragma unroll
+            for (int it = 0; it < T; ++it) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) *reinterpret_cast<v4u_t*>(tr + put + 4u * i * kTileTransitRow) = xa[0][it][i];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xa[0][it][j] = *reinterpret_cast<const v4u_t*>(tr + get + 16u * j);
+            }
+        }
         // sums of x over the wave's columns: the product with a matrix of ones, in the accumulator layout
         // (lane (row r, token group kg) register e <-> token 4*kg + e; identical for every r)
         const v4u_t ones = {F::one_bits, F::one_bits, F::one_bits, F::one_bits};
@@ -375,6 +429,8 @@ __global__ void __launch_bounds__((64 * tile_max_waves<NT, T, BF, PL>())) tile_k
         // The first tile's ids are requested only now, after the activations have ARRIVED: requesting them earlier --
         // before the activations, or right behind them -- was measured to cost about a microsecond per launch (the few
         // activation requests then compete with the flood of id requests of the whole chip).
+        // (Measured again with the activations fetched in memory order, 16 rows of X: ids right behind the activations 0.532 ms
+        // for 8 layers against 0.500 this way.)
         // Later panels' first ids are in flight already (requested at the end of the panel before).
         if constexpr (!XL) { if (n_mine > 0 && first_panel) info = issue_tile(0, step0, wlo, whi); }
 
@@ -1056,7 +1112,7 @@ constexpr size_t kTileLdsLimit = 128 * 1024;
 constexpr size_t kTileXLdsLimit = 64 * 1024;     // X through LDS: up to this many bytes of activations on top
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;
 
-bool plan_tile_for(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int wave_cap, int per_cu) {
+bool plan_tile_for(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int wave_cap, int per_cu, size_t lds_limit = kTileLdsLimit) {
     const int n_steps = (int)(P / kStepCols);
     const int ranges = (n_steps + T - 1) / T;                 // column ranges of T steps
     // more than eight waves only where that saves a panel
@@ -1077,10 +1133,10 @@ bool plan_tile_for(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl,
     for (;;) {
         const size_t rows = (size_t)tw * kTileRows;
         pl.lds = rows * 16 + (size_t)pl.W * pl.G * (tw / pl.G) * kTileRows * 8 + rg * TM * 4 + rows * rg * (size_t)M * 4;
-        if (pl.lds <= kTileLdsLimit || tw <= pl.G) break;
+        if (pl.lds <= lds_limit || tw <= pl.G) break;
         tw -= pl.G;
     }
-    if (pl.lds > kTileLdsLimit) return false;
+    if (pl.lds > lds_limit) return false;
     // more workgroups than the target (LDS or the thread count capped the tiles of one): a whole number of rounds over the
     // CUs, the tiles spread evenly -- 1035 workgroups on 256 CUs would leave the fifth round to 11 of them
     int64_t blocks = (tiles + tw - 1) / tw;
@@ -1102,12 +1158,13 @@ bool plan_tile_for(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl,
 // and LDS for both (`x_lds` = the activations' bytes on top of the plan's own) -- else one.  Two resident workgroups keep
 // more requests in flight and let one's epilogue overlap the other's stream (9B gate+up 19.5 -> 18.4 us); where only one
 // fits, twice the workgroups would just be a second round (27B down, twelve waves: 23.2 -> 26.7 us).
-bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int wave_cap = 8, bool pair_fits = false, size_t x_lds = 0) {
+bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int wave_cap = 8, bool pair_fits = false, size_t x_lds = 0,
+               size_t lds_limit = kTileLdsLimit) {
     const int forced = host::env_int("QVB8_TILE_WGS_PER_CU", 0);
-    if (forced > 0) return plan_tile_for(NT, T, M, Q, P, pl, wave_cap, forced);
-    if (pair_fits && plan_tile_for(NT, T, M, Q, P, pl, wave_cap, 2) && pl.panels == 1 && pl.threads <= 512
+    if (forced > 0) return plan_tile_for(NT, T, M, Q, P, pl, wave_cap, forced, lds_limit);
+    if (pair_fits && plan_tile_for(NT, T, M, Q, P, pl, wave_cap, 2, lds_limit) && pl.panels == 1 && pl.threads <= 512
         && 2 * (pl.lds + x_lds) <= kLdsPerWorkgroup) return true;
-    return plan_tile_for(NT, T, M, Q, P, pl, wave_cap, 1);
+    return plan_tile_for(NT, T, M, Q, P, pl, wave_cap, 1, lds_limit);
 }
 
 // Whether the registers of this kernel let two workgroups of eight waves share a CU (asked of the runtime once per device).
@@ -1130,8 +1187,10 @@ template <int NT, int T, bool BF, bool XC, int XP = 0, bool PL = false>
 int launch_tile(TileArgs& a, hipStream_t s) {
     TilePlan pl;
     const bool jit = tile_pair_fits<NT, T, BF, XC, XP, PL>();
-    const size_t x_lds = XP > 0 ? (size_t)a.M * (size_t)a.P * 2 + 64 : 0;
-    if (!plan_tile(NT, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<NT, T, BF, PL>() : 8, jit, x_lds))
+    // on top of the plan's own: all of X (XP > 0), or a transit region per wave (one token tile, X not in LDS as a whole)
+    const size_t x_lds = XP > 0 ? (size_t)a.M * (size_t)a.P * 2 + 64 : (NT == 1 ? (size_t)tile_max_waves<NT, T, BF, PL>() * kTileTransitBytes : 0);
+    const size_t limit = XP > 0 ? kTileLdsLimit : (kLdsPerWorkgroup - x_lds < kTileLdsLimit ? kLdsPerWorkgroup - x_lds : kTileLdsLimit);
+    if (!plan_tile(NT, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<NT, T, BF, PL>() : 8, jit, x_lds, limit))
         return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
     pl.lds += x_lds;
     a.W = pl.W; a.G = pl.G; a.panels = pl.panels; a.TW = pl.TW;

@@ -47,10 +47,13 @@ def test_mma_all_m(M, dtype):
         _check(H.oracle_view(enc), None, x, y, saturate_ref=False)
 
 
-@pytest.mark.parametrize("M,P", [(1, 4096), (3, 4096), (8, 4096), (1, 12288), (1, 17408), (2, 5120), (1, 28672)])
+@pytest.mark.parametrize("M,P", [(1, 4096), (3, 4096), (8, 4096), (1, 12288), (1, 17408), (2, 5120), (1, 28672),
+                                 (9, 3072), (12, 2048), (16, 2048), (16, 1024), (13, 1280)])
 def test_activations_through_lds_change_no_bit(M, P, monkeypatch):
     """Small X is staged through LDS once (1, 4 or 8 sixteen-byte pieces per thread); the same call with that path
-    switched off reads X from global memory per panel.  Same arithmetic in the same order: identical bits."""
+    switched off fetches X per wave and panel in memory order and turns it into operand order through the wave's own
+    piece of LDS -- the path every larger X takes (9..16 rows of 4096 columns, 3.. rows of 12288).  Same arithmetic in
+    the same order: identical bits."""
     W = H.synth_weight(80, P, seed=P + M).to(DEV)
     enc = PK.encode_tensor(W, 1e-3, restore="fp16", force_escapes=[9, P * 79 + P - 1])
     perm = _perm_by_width(enc["nbits"])
@@ -62,6 +65,31 @@ def test_activations_through_lds_change_no_bit(M, P, monkeypatch):
         y0 = ext.mma_tiles(x, *H.pack_args(enc), perm=perm, saturate=saturate)
         assert torch.equal(y1, y0), (dtype, saturate)
     _check(H.oracle_view(enc), None, x, y1, saturate_ref=False)
+
+
+@pytest.mark.parametrize("M", [2, 5, 9, 12, 16])
+def test_rows_in_planes_and_both_ways_of_fetching_x(M, monkeypatch):
+    """The module's default storage (rows in planes, width order): X through LDS as a whole against X fetched per wave, bit
+    for bit, and both against the oracle.  4 rows of 12288 columns exceed what LDS takes as a whole: that weight takes the
+    per-wave path either way and is checked against the oracle alone."""
+    from qvb8_amd.formats.qvb8.module import QVBandLinearV8
+    for Q, P in ((272, 2048), (96, 12288)):
+        W = H.synth_weight(Q, P, seed=Q + M).to(DEV)
+        enc = PK.encode_tensor(W, 1e-3, restore="fp16")
+        lin = QVBandLinearV8.from_encoded(enc)
+        x = _x(M, P, torch.bfloat16, 5 * M)
+        monkeypatch.setenv("QVB8_TILE_X_LDS", "1")
+        y1 = lin(x)
+        monkeypatch.setenv("QVB8_TILE_X_LDS", "0")
+        y0 = lin(x)
+        assert torch.equal(y1, y0), (Q, P)
+        d = H.oracle_view(enc)
+        Wr = O.reconstruct(d["min_s"], d["tau_s"], d["ids_dense"] if "ids_dense" in d else H.oracle_ids(d), d["esc_idx"], d["esc_vals"])
+        xs = O.sat_half(x.float().cpu().numpy())
+        ref = O.linear_f64(xs, Wr)
+        tol = H.gemv_tolerance(ref, Wr, xs) + 2.0 ** -8 * np.abs(ref)           # the module rounds to the caller's bf16
+        diff = np.abs(y1.float().cpu().numpy().astype(np.float64) - ref)
+        assert y1.dtype == torch.bfloat16 and np.all(diff <= tol), (Q, P, float((diff / tol).max()))
 
 
 @pytest.mark.parametrize("Q,P,tau", [(1024, 4096, 1e-3), (200, 12288, 1e-3), (130, 768, 2e-3), (96, 2048, 2e-3),
