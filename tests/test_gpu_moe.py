@@ -41,7 +41,12 @@ def _check(out, ref, out_dtype, roundings=1):
     eps = {torch.float32: 0.0, torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[out_dtype] * roundings
     got = out.float().cpu().numpy().astype(np.float64)
     scale = np.sqrt(np.mean(ref ** 2)) + 1e-30
-    tol = (1e-3 + eps) * np.abs(ref) + (2e-3 + eps * (roundings > 1)) * scale
+    # Relative part: the bar of every product test here (1e-3) plus the roundings to out_dtype.  Absolute part, in units of
+    # the output's rms: the two chained products each carry the product tests' error (fp32 accumulation over 768..2048
+    # terms), and on the matrix-core paths H goes from the first to the second as fp16 (2^-11 per element, which the down
+    # product averages over its terms rather than adds up).  Measured over these tests the worst element uses about half of
+    # 1e-3 rms; half that bound fails 7 of them.
+    tol = (1e-3 + eps) * np.abs(ref) + (1e-3 + eps * (roundings > 1)) * scale
     diff = np.abs(got - ref)
     assert np.all(diff <= tol), (float(diff.max()), float((diff / tol).max()))
 
