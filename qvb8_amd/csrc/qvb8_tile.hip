@@ -883,7 +883,8 @@ constexpr int kG2AStride = kG2Cols * 2 + 16;                       // bytes per 
 constexpr int kG2BStride = 2 * kG2Cols * 2 + 16;                   // bytes per weight row of one 128-column block
 
 template <int WM, bool BF, int NB>
-__device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_end, int run_first, uint64_t run_byte0, unsigned char* smem) {
+__device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_end, int run_first, uint64_t run_byte0, unsigned char* smem,
+                                          int by, int bz) {
     using F = Fmt<BF>;
     constexpr int BM = 64 * WM, WN = kG2Mul / WM, NT = kG2Rows / (32 * WN);   // WM = 4: 256 rows of X, 64 x 64 sums per wave; WM = 2: 128 rows, 64 x 32
     constexpr int MT = 2;
@@ -892,8 +893,8 @@ __device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_e
     unsigned char* Bs = smem + (size_t)2 * BM * kG2AStride;        // [2][kG2Rows][kG2BStride]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int tok0 = (int)blockIdx.y * BM;
-    const int s_begin = (int)blockIdx.z * a.stages_per_split * 2;  // stages_per_split counts 128-column stages
+    const int tok0 = by * BM;
+    const int s_begin = bz * a.stages_per_split * 2;  // stages_per_split counts 128-column stages
     const int s_end = min(a.P / kG2Cols, s_begin + a.stages_per_split * 2);
     const int n_st = s_end - s_begin;                              // a multiple of 4
     if (n_st <= 0) return;
@@ -947,7 +948,7 @@ __device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_e
         const uint16_t* x_piece[XL];
 #pragma unroll
         for (int i = 0; i < XL; ++i)
-            x_piece[i] = a.X + (((size_t)blockIdx.y * (a.P / kG2Cols) + s_begin) * BM + min(xrow + 64 * i, M - 1 - tok0)) * kG2Cols + 8 * xch;
+            x_piece[i] = a.X + (((size_t)by * (a.P / kG2Cols) + s_begin) * BM + min(xrow + 64 * i, M - 1 - tok0)) * kG2Cols + 8 * xch;
         v4u_t xg[4][XL];
         auto request_x = [&](int st, v4u_t (&g)[XL]) __attribute__((always_inline)) {
             const size_t c = (size_t)min(st, n_st - 1) * (BM * kG2Cols);
@@ -1041,10 +1042,10 @@ __device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_e
     }
     // ---- the end: a multiplying lane holds, for weight row n of each row tile, rows of X 32 mt + 8 (i / 4) + 4 kh + i % 4 ----
     float* sxs = reinterpret_cast<float*>(smem);                   // the buffers are no longer read (barrier above)
-    if (tid < BM) sxs[tid] = tok0 + tid < a.M ? a.sx[(size_t)blockIdx.z * a.M + tok0 + tid] : 0.f;
+    if (tid < BM) sxs[tid] = tok0 + tid < a.M ? a.sx[(size_t)bz * a.M + tok0 + tid] : 0.f;
     __syncthreads();
     if (wave >= kG2Mul) return;
-    float* out = a.out + (size_t)blockIdx.z * (size_t)a.M * (size_t)a.Q;
+    float* out = a.out + (size_t)bz * (size_t)a.M * (size_t)a.Q;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const int pos = pos0 + wn * (32 * NT) + 32 * nt + n;
@@ -1070,8 +1071,26 @@ __device__ __forceinline__ void gemm2_run(const GemmArgs& a, int pos0, int pos_e
 template <int WM, bool BF>
 __global__ void __launch_bounds__(64 * kG2Waves) gemm2_kernel(GemmArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
+    // Which block of weight rows (bx), block of rows of X (by) and column range (bz) this workgroup takes.  Workgroups go
+    // to the eight XCDs in turn (flat number % 8), each XCD with an L2 of its own; dealt in the grid's order, every XCD
+    // meets every column range and so fetches all of X (at 256 rows: 8 x 6.3 MB for `down`, more than its ids).  When the
+    // number of column ranges divides 8, XCD j instead takes range j % nz only, both blocks of X of it, and every
+    // (8 / nz)-th block of weight rows: X crosses the fabric 8 / nz times instead of 8, every id still once.  Measured, 8
+    // layers of the 9B shapes: 192 rows of X 1.549 -> 1.521 ms, 256 rows 1.618 -> 1.568 ms, HBM-side traffic per layer
+    // 437 -> 383 MB; with one block of X (up to 128 rows: X is 1 MB or less) the grid's own order is 1.5 % faster and is kept.
+    int bx = (int)blockIdx.x, by = (int)blockIdx.y, bz = (int)blockIdx.z;
+    {
+        const int nx = (int)gridDim.x, ny = (int)gridDim.y, nz = (int)gridDim.z;
+        const int per = nz <= 8 ? 8 / nz : 0;                      // XCDs that share a column range
+        if (ny > 1 && nz > 1 && per * nz == 8 && nx % per == 0) {
+            const int flat = bx + nx * (by + ny * bz);
+            const int xcd = flat & 7, k = flat >> 3;               // k: the XCD's own count, 0 .. nx * ny / per - 1
+            bz = xcd % nz;
+            by = k % ny;
+            bx = (k / ny) * per + xcd / nz;
+        }
+    }
     // which run of equal widths this workgroup's 128 positions belong to
-    const int bx = (int)blockIdx.x;
     const int c = (bx >= a.blocks1 ? 1 : 0) + (bx >= a.blocks2 ? 1 : 0);
     const uint32_t nb0 = a.widths & 255u, nb1 = (a.widths >> 8) & 255u, nb2 = (a.widths >> 16) & 255u;
     const uint64_t row0 = (uint64_t)a.P * nb0 / 8, row1 = (uint64_t)a.P * nb1 / 8;
@@ -1081,11 +1100,11 @@ __global__ void __launch_bounds__(64 * kG2Waves) gemm2_kernel(GemmArgs a) {
     const int pos0 = run_first + (bx - (c == 0 ? 0 : c == 1 ? a.blocks1 : a.blocks2)) * kG2Rows;
     if (pos0 >= run_end) return;
     switch (c == 0 ? nb0 : c == 1 ? nb1 : nb2) {
-        case 4: gemm2_run<WM, BF, 4>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 5: gemm2_run<WM, BF, 5>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 6: gemm2_run<WM, BF, 6>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 7: gemm2_run<WM, BF, 7>(a, pos0, run_end, run_first, byte0, smem); break;
-        case 8: if constexpr (!BF) gemm2_run<WM, BF, 8>(a, pos0, run_end, run_first, byte0, smem); break;
+        case 4: gemm2_run<WM, BF, 4>(a, pos0, run_end, run_first, byte0, smem, by, bz); break;
+        case 5: gemm2_run<WM, BF, 5>(a, pos0, run_end, run_first, byte0, smem, by, bz); break;
+        case 6: gemm2_run<WM, BF, 6>(a, pos0, run_end, run_first, byte0, smem, by, bz); break;
+        case 7: gemm2_run<WM, BF, 7>(a, pos0, run_end, run_first, byte0, smem, by, bz); break;
+        case 8: if constexpr (!BF) gemm2_run<WM, BF, 8>(a, pos0, run_end, run_first, byte0, smem, by, bz); break;
         default: break;
     }
 }
