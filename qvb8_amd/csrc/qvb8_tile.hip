@@ -1129,6 +1129,7 @@ struct TilePlan { int W, G, panels, TW, threads; size_t lds; unsigned blocks; };
 
 constexpr size_t kTileLdsLimit = 128 * 1024;
 constexpr size_t kTileXLdsLimit = 64 * 1024;     // X through LDS: up to this many bytes of activations on top
+constexpr size_t kTileXLdsMost = 140000;         // ... and up to this many for at most 8 rows of X
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;
 
 bool plan_tile_for(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int wave_cap, int per_cu, size_t lds_limit = kTileLdsLimit) {
@@ -1183,6 +1184,8 @@ bool plan_tile(int NT, int T, int64_t M, int64_t Q, int64_t P, TilePlan& pl, int
     if (forced > 0) return plan_tile_for(NT, T, M, Q, P, pl, wave_cap, forced, lds_limit);
     if (pair_fits && plan_tile_for(NT, T, M, Q, P, pl, wave_cap, 2, lds_limit) && pl.panels == 1 && pl.threads <= 512
         && 2 * (pl.lds + x_lds) <= kLdsPerWorkgroup) return true;
+    // (Where two copies of X do not fit -- 5..8 rows of 4096 columns -- one workgroup of sixteen waves sharing one copy was
+    // measured: no faster than one of eight, 0.464 against 0.460 ms for 8 layers at 8 rows.)
     return plan_tile_for(NT, T, M, Q, P, pl, wave_cap, 1, lds_limit);
 }
 
@@ -1208,7 +1211,7 @@ int launch_tile(TileArgs& a, hipStream_t s) {
     const bool jit = tile_pair_fits<NT, T, BF, XC, XP, PL>();
     // on top of the plan's own: all of X (XP > 0), or a transit region per wave (one token tile, X not in LDS as a whole)
     const size_t x_lds = XP > 0 ? (size_t)a.M * (size_t)a.P * 2 + 64 : (NT == 1 ? (size_t)tile_max_waves<NT, T, BF, PL>() * kTileTransitBytes : 0);
-    const size_t limit = XP > 0 ? kTileLdsLimit : (kLdsPerWorkgroup - x_lds < kTileLdsLimit ? kLdsPerWorkgroup - x_lds : kTileLdsLimit);
+    const size_t limit = kLdsPerWorkgroup - x_lds < kTileLdsLimit ? kLdsPerWorkgroup - x_lds : kTileLdsLimit;   // what X or the transit regions leave
     if (!plan_tile(NT, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<NT, T, BF, PL>() : 8, jit, x_lds, limit))
         return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
     pl.lds += x_lds;
@@ -1228,20 +1231,30 @@ int launch_tile(TileArgs& a, hipStream_t s) {
                        (uint32_t)a.nb[0] | ((uint32_t)a.nb[1] << 8) | ((uint32_t)a.nb[2] << 16) | ((uint32_t)a.n_classes << 24));
     return host::check_launch("qvb8_mma");
 }
-// One to sixteen rows of X on the NT = 1 kernel: X goes through LDS when all of it fits (64 KB, and the workgroup's LDS),
-// with 1, 4 or 8 pieces of 16 bytes per thread (a request past the end of X would be a wasted one: the count is exact to
-// within those three variants).
+// One to sixteen rows of X on the NT = 1 kernel: X goes through LDS when all of it fits (the limits below, and the
+// workgroup's LDS), with 1, 4, 8 or 16 pieces of 16 bytes per thread (a request past the end of X would be a wasted one:
+// the count is exact to within those four variants).
 template <int T, bool BF, bool XC, bool PL = false>
 int launch_tile_rows16(TileArgs& a, hipStream_t s) {
     TilePlan pl;
     const size_t x_bytes = (size_t)a.M * (size_t)a.P * 2;
-    if (!plan_tile(1, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<1, T, BF, PL>() : 8, tile_pair_fits<1, T, BF, XC, 1, PL>(), x_bytes + 64))
-        return host::fail(QVB8_ERR_UNSUPPORTED, "qvb8_mma: shape does not fit a workgroup's LDS");
-    const size_t per_thread = (x_bytes / 16 + pl.threads - 1) / pl.threads;
-    const bool fits = x_bytes <= kTileXLdsLimit && pl.lds + x_bytes + 64 <= kLdsPerWorkgroup && host::env_int("QVB8_TILE_X_LDS", 1) != 0;
+    // Up to 8 rows of X whatever fits (measured on the 9B `down`, 12288 columns: 3 rows 74 KB, 5 rows 123 KB of X in LDS
+    // against fetched per wave: 8 layers 0.420 -> 0.385 ms at 3 rows, 0.428 -> 0.404 at 5); more rows only up to 64 KB (9..16
+    // rows of 4096 columns through LDS as a whole leave room for three tiles per workgroup: 0.478 -> 0.543 ms at 16 rows).
+    const size_t x_limit = a.M <= 8 ? (size_t)host::env_int("QVB8_TILE_X_LDS_LIMIT", (int)kTileXLdsMost) : kTileXLdsLimit;
+    bool fits = x_bytes <= x_limit && x_bytes + 64 + 8192 <= kLdsPerWorkgroup && host::env_int("QVB8_TILE_X_LDS", 1) != 0;
+    size_t per_thread = 0;
+    if (fits) {
+        // the plan as the kernel with X in LDS will make it: its own LDS within what X leaves
+        const size_t left = kLdsPerWorkgroup - (x_bytes + 64);
+        fits = plan_tile(1, T, a.M, a.Q, a.P, pl, host::env_int("QVB8_TILE_WAVES12", 1) ? tile_max_waves<1, T, BF, PL>() : 8,
+                         tile_pair_fits<1, T, BF, XC, 1, PL>(), x_bytes + 64, left < kTileLdsLimit ? left : kTileLdsLimit);
+        per_thread = fits ? (x_bytes / 16 + pl.threads - 1) / pl.threads : 0;
+    }
     if (fits && per_thread <= 1) return launch_tile<1, T, BF, XC, 1, PL>(a, s);
     if (fits && per_thread <= 4) return launch_tile<1, T, BF, XC, 4, PL>(a, s);
     if (fits && per_thread <= 8) return launch_tile<1, T, BF, XC, 8, PL>(a, s);
+    if (fits && per_thread <= 16) return launch_tile<1, T, BF, XC, 16, PL>(a, s);
     return launch_tile<1, T, BF, XC, 0, PL>(a, s);
 }
 

@@ -48,12 +48,12 @@ def test_mma_all_m(M, dtype):
 
 
 @pytest.mark.parametrize("M,P", [(1, 4096), (3, 4096), (8, 4096), (1, 12288), (1, 17408), (2, 5120), (1, 28672),
-                                 (9, 3072), (12, 2048), (16, 2048), (16, 1024), (13, 1280)])
+                                 (9, 3072), (12, 2048), (16, 2048), (16, 1024), (13, 1280), (4, 12288), (5, 12288), (3, 17408)])
 def test_activations_through_lds_change_no_bit(M, P, monkeypatch):
-    """Small X is staged through LDS once (1, 4 or 8 sixteen-byte pieces per thread); the same call with that path
-    switched off fetches X per wave and panel in memory order and turns it into operand order through the wave's own
-    piece of LDS -- the path every larger X takes (9..16 rows of 4096 columns, 3.. rows of 12288).  Same arithmetic in
-    the same order: identical bits."""
+    """Small X is staged through LDS once (1, 4, 8 or 16 sixteen-byte pieces per thread; up to 8 rows whatever fits, more
+    rows up to 64 KB); the same call with that path switched off fetches X per wave and panel in memory order and turns it
+    into operand order through the wave's own piece of LDS -- the path every larger X takes (9..16 rows of 4096 columns,
+    6.. rows of 12288).  Same arithmetic in the same order: identical bits."""
     W = H.synth_weight(80, P, seed=P + M).to(DEV)
     enc = PK.encode_tensor(W, 1e-3, restore="fp16", force_escapes=[9, P * 79 + P - 1])
     perm = _perm_by_width(enc["nbits"])
@@ -70,8 +70,8 @@ def test_activations_through_lds_change_no_bit(M, P, monkeypatch):
 @pytest.mark.parametrize("M", [2, 5, 9, 12, 16])
 def test_rows_in_planes_and_both_ways_of_fetching_x(M, monkeypatch):
     """The module's default storage (rows in planes, width order): X through LDS as a whole against X fetched per wave, bit
-    for bit, and both against the oracle.  4 rows of 12288 columns exceed what LDS takes as a whole: that weight takes the
-    per-wave path either way and is checked against the oracle alone."""
+    for bit, and both against the oracle.  9 and more rows of 12288 columns exceed what LDS takes as a whole: that weight
+    then takes the per-wave path either way and is checked against the oracle alone."""
     from qvb8_amd.formats.qvb8.module import QVBandLinearV8
     for Q, P in ((272, 2048), (96, 12288)):
         W = H.synth_weight(Q, P, seed=Q + M).to(DEV)
