@@ -33,22 +33,6 @@ LAYER_9B = (("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096,
 LAYER_27B = (("q", 5120, 5120), ("k", 1024, 5120), ("v", 1024, 5120), ("o", 5120, 5120),
              ("gate", 17408, 5120), ("up", 17408, 5120), ("down", 5120, 17408))
 TAU = 1e-3
-def measured_traffic(profile, kernel):
-    """HBM bytes per launch by launch class, from the `traffic_bytes_per_launch <kernel> <class> <bytes>` lines of a
-    summary under profiles/ (hardware counters, recorded there with the commands that took them); {} without the file."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", profile)
-    out = {}
-    try:
-        with open(path) as fh:
-            for line in fh:
-                f = line.split()
-                if len(f) == 4 and f[0] == "traffic_bytes_per_launch" and f[1] == kernel:
-                    out[f[2]] = int(f[3])
-    except OSError:
-        pass
-    return out
-
-
 def measured_figure(profile, key, kernel):
     """{class: value} of the `<key> <kernel> <class> <value>` lines of a summary under profiles/ ({} without the file)."""
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", profile)
@@ -62,6 +46,12 @@ def measured_figure(profile, key, kernel):
     except OSError:
         pass
     return out
+
+
+def measured_traffic(profile, kernel):
+    """HBM bytes per launch by launch class: the `traffic_bytes_per_launch <kernel> <class> <bytes>` lines of a summary under
+    profiles/ (hardware counters, recorded there with the commands that took them)."""
+    return {k: int(v) for k, v in measured_figure(profile, "traffic_bytes_per_launch", kernel).items()}
 
 
 MMA_FLAGS = int(os.environ.get("QVB8_BENCH_MMA_FLAGS", "1"))     # 1 = QVB8_MMA_SATURATE_X: the operator's default for bf16 x
