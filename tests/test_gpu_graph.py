@@ -102,7 +102,7 @@ def test_graph_replay_is_bit_identical(kind):
                 idx, w = eager.route(xs[rep])
                 ref = O.moe_reference(xs[rep].float().cpu().numpy(), idx.cpu().numpy(), w.float().cpu().numpy(), *eager.restored)
                 diff = np.abs(got.float().cpu().numpy().astype(np.float64) - ref)
-                tol = (1e-3 + 2.0 ** -8) * np.abs(ref) + 1e-3 * np.sqrt(np.mean(ref ** 2))        # the MoE tests' bar
+                tol = (1e-3 + 2.0 ** -8) * np.abs(ref) + 1.5e-3 * np.sqrt(np.mean(ref ** 2))      # the MoE tests' bar
                 assert np.all(diff <= tol), (rows, rep, float((diff / tol).max()))
     assert sum(1 for v in layer.mlp._graphs.values() if isinstance(v, tuple)) == 2
     big = torch.randn(64, h, device=DEV).to(torch.bfloat16)         # prefill-sized input: eager, no new graph

@@ -44,9 +44,9 @@ def _check(out, ref, out_dtype, roundings=1):
     # Relative part: the bar of every product test here (1e-3) plus the roundings to out_dtype.  Absolute part, in units of
     # the output's rms: the two chained products each carry the product tests' error (fp32 accumulation over 768..2048
     # terms), and on the matrix-core paths H goes from the first to the second as fp16 (2^-11 per element, which the down
-    # product averages over its terms rather than adds up).  Measured over these tests the worst element uses about half of
-    # 1e-3 rms; half that bound fails 7 of them.
-    tol = (1e-3 + eps) * np.abs(ref) + (1e-3 + eps * (roundings > 1)) * scale
+    # product averages over its terms rather than adds up).  Measured: the worst element of these tests uses about half of
+    # 1e-3 rms, the worst of 1500 randomised calls (2..11 experts, 1..16 tokens, hidden 128..2048) 1.25e-3 rms.
+    tol = (1e-3 + eps) * np.abs(ref) + (1.5e-3 + eps * (roundings > 1)) * scale
     diff = np.abs(got - ref)
     assert np.all(diff <= tol), (float(diff.max()), float((diff / tol).max()))
 
