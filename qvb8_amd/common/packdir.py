@@ -133,8 +133,11 @@ def swap_modules(model: nn.Module, pack_dir, *, device: str = "cuda", out_dtype=
         elif pd.spec.experts is None:
             report["skipped"][block] = f"format {pd.spec.name} has no expert reader"
         else:
-            _set(model, block, pd.spec.experts.from_packfiles(gu, dn, num_experts=n, act_fn=getattr(owner, "act_fn", None),
-                                                              device=device, tau=pd.tau))
+            stack = pd.spec.experts.from_packfiles(gu, dn, num_experts=n, act_fn=getattr(owner, "act_fn", None),
+                                                   device=device, tau=pd.tau)
+            if hasattr(stack, "prepare"):
+                stack.prepare()                  # the stacks' rows are re-stored now, not on the first routed call
+            _set(model, block, stack)
             report["experts"].append(block)
 
     for key in pd.tensors:
