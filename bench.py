@@ -63,9 +63,9 @@ def mma_flags(lin) -> int:
     return MMA_FLAGS | (8 if lin._planes else 0)
 
 
-def tile_traffic(units, n_launch):
+def tile_traffic(units, n_launch, model="9b"):
     """Mean measured HBM bytes per launch of the step's launch mix (None when the counters' summary is not there)."""
-    t = measured_traffic("tile_kernel_9b_decode_step_hbm_traffic.md", "tile_kernel")
+    t = measured_traffic("tile_kernel_%s_decode_step_hbm_traffic.md" % model, "tile_kernel")
     if any(u["name"] not in t for u in units):
         return None
     return round(sum(t[u["name"]] for u in units) / n_launch)
@@ -357,6 +357,10 @@ def _time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name, walk_t
     ms = max(ev_ms, wall_ms)
     gbs = step_bytes / (ms * 1e-3) / 1e9
     launch_us = ev_ms * 1e3 / len(units)
+    # HBM bytes per launch of the one-row kernel from hardware counters (profiles/): the mean over the shapes' tensors
+    key = "65b" if "8192" in shape_name else "27b"
+    r_traffic = measured_traffic("r_gemv_kernel_65b_ffn_trace_and_counters.md" if key == "65b" else "r_gemv_kernel_27b_ffn_kernel_trace.md",
+                                 "r_gemv_kernel").get(key) if M == 1 else None
     kernel = "qvb8::r_gemv_kernel<2>" if M == 1 else "qvb8::r_mma_kernel<%d, false> (+ r_pack_x_kernel)" % ((M + 15) // 16)
     return {"metric": "QVB8R fused entropy-decode + GEMV GB/s on coded bytes, large-dense FFN shapes, 1 MI355X",
             "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -367,7 +371,7 @@ def _time_qvb8r(args, dev, lib, units, M, coded_bytes, n_sym, shape_name, walk_t
                        "bytes_per_step": step_bytes, "bits_per_weight": round(8.0 * step_bytes / n_sym, 3),
                        "symbols_per_s": round(n_sym / (ms * 1e-3), 1)},
             "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": r_traffic,
                          "kernel": kernel,
                          "bytes_per_launch": step_bytes // len(units), "launch_us": round(launch_us, 3),
                          "note": "the walk is bound by its instruction count (vector ALU 91 % busy), not by HBM"},
@@ -845,7 +849,7 @@ def time_decode(args, dev, lib, layers, units, shapes, model):
                    "bits_per_weight": round(8.0 * sum(u["lin"].ids.numel() for u in units) / sum(e["Q"] * e["P"] for e in flat), 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": tile_traffic(units, n_launch) if (MMA_FLAGS == 1 and model == "9b" and fused) else None,
+                     "traffic": tile_traffic(units, n_launch, model) if (MMA_FLAGS == 1 and fused) else None,
                      "kernel": "qvb8::tile_kernel<1,4,false,true,XP,PL> (XP = 1 or 4 pieces of X per thread through LDS; PL: rows stored in planes)" + (" / <1,5,false,true,XP,PL> for 5120-column rows" if model == "27b" else ""),
                      "bytes_per_launch": step_bytes // n_launch,
                      "launch_us": round(launch_us, 3)},
