@@ -52,18 +52,33 @@ struct Walker {
     const uint32_t* wp;
 };
 
-__device__ __forceinline__ void walk_init(Walker& z, uint32_t* rg, const RCore& c, int tile, int l32) {
+// Returns the last word index (from the tile's first word) the walk may read ahead to: the end of the buffer, and -- when
+// the next tile's words follow this tile's, as every writer lays them out -- the tile's own last word.  The ring always
+// asks for 128..384 words more than the walk has used; past the tile's end those lines belong to a tile that another
+// workgroup walks at another time, so they came from memory twice (measured at the 65B shapes, one row per tile of 1150
+// words: 325 MB fetched for 267 MB of stream).  Requests past the bound read the bound's word again.
+__device__ __forceinline__ int64_t walk_init(Walker& z, uint32_t* rg, const RCore& c, int tile, int l32) {
     int64_t off = c.tile_off[tile];
+    const int64_t next = c.tile_off[tile + 1];
     const int64_t last = c.n_words - (kRing + kRing / 2);                  // the furthest start that keeps every read inside
     off = off < 0 ? 0 : (off > last ? last : off);
     z.wp = c.words + off;
+    int64_t room = c.n_words - 1 - off;
+    if (next > off && next - off - 1 < room) room = next - off - 1;
     const uint64_t s = c.states[(int64_t)tile * 32 + l32];
     z.xl = (uint32_t)s; z.xh = (uint32_t)(s >> 32);
     z.ptr = z.sb = 0;
 #pragma unroll
-    for (int q = 0; q < kRing / 32; ++q) rg[32 * q + l32] = z.wp[32 * q + l32];
+    for (int q = 0; q < kRing / 32; ++q) {
+        const int64_t i = 32 * q + l32;
+        rg[32 * q + l32] = z.wp[i < room ? i : room];
+    }
 #pragma unroll
-    for (int q = 0; q < kRing / 64; ++q) z.pre[q] = z.wp[kRing + 32 * q + l32];
+    for (int q = 0; q < kRing / 64; ++q) {
+        const int64_t i = kRing + 32 * q + l32;
+        z.pre[q] = z.wp[i < room ? i : room];
+    }
+    return room;
 }
 
 // one symbol: x' = f * (x >> 12) + d on the 64-bit state
@@ -151,8 +166,7 @@ __global__ void __launch_bounds__(kRThreads) r_decode_kernel(RCore c, int b0, in
     TileCtx t = block_setup(c, block_no, st, h8);
     uint32_t* rg = ring[h8];
     Walker z;
-    walk_init(z, rg, c, t.tile, l32);
-    t.room = c.n_words - 1 - (z.wp - c.words);
+    t.room = walk_init(z, rg, c, t.tile, l32);
     __syncthreads();
     const int S = c.P >> 5;
     for (int r = 0; r < T; ++r) {
@@ -192,8 +206,7 @@ __global__ void __launch_bounds__(kRThreads) r_gemv_kernel(RCore c, const void* 
     TileCtx t = block_setup(c, blockIdx.x, st, h8);
     uint32_t* rg = ring[h8];
     Walker z;
-    walk_init(z, rg, c, t.tile, l32);
-    t.room = c.n_words - 1 - (z.wp - c.words);
+    t.room = walk_init(z, rg, c, t.tile, l32);
     __syncthreads();
     const int S = c.P >> 5;
     float sx = 0.f;                  // sum of x over this lane's columns (the same for every row): taken while the first row is walked
@@ -336,8 +349,7 @@ __global__ void __launch_bounds__(kRThreads) r_mma_kernel(RCore c, RPacked xp, i
     TileCtx t = block_setup(c, blockIdx.x, st, h8);
     uint32_t* rg = ring[h8];
     Walker z;
-    walk_init(z, rg, c, t.tile, l32);
-    t.room = c.n_words - 1 - (z.wp - c.words);
+    t.room = walk_init(z, rg, c, t.tile, l32);
     __syncthreads();
     const int S = c.P >> 5;
     const int n_batches = (c.P + kRBatchCols - 1) / kRBatchCols;
